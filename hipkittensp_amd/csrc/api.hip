@@ -1,0 +1,118 @@
+// C ABI of the MXFP6 GEMM library (declared in include/mxfp6_gemm.h): argument validation and
+// kernel selection.  Nothing here allocates or synchronises.
+#include "../../include/mxfp6_gemm.h"
+
+#include <atomic>
+
+#include "kernels.hpp"
+
+namespace {
+
+std::atomic<int> g_force{0};
+
+int check_device() {
+  // cached per process: the library only carries gfx950 code objects
+  static int cached = [] {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MXFP6_ENODEVICE;
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, dev) != hipSuccess) return MXFP6_ENODEVICE;
+    return __builtin_strncmp(p.gcnArchName, "gfx950", 6) == 0 ? MXFP6_OK : MXFP6_ENODEVICE;
+  }();
+  return cached;
+}
+
+int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
+                int fmt_b, bool f32out, void* stream) {
+  if (M < 0 || N < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
+  if ((fmt_a != MXFP6_FMT_E2M3 && fmt_a != MXFP6_FMT_E3M2) || (fmt_b != MXFP6_FMT_E2M3 && fmt_b != MXFP6_FMT_E3M2))
+    return MXFP6_EINVAL_FMT;
+  if (M == 0 || N == 0) return MXFP6_OK;
+  if (!C) return MXFP6_EINVAL_PTR;
+  if (K > 0 && (!A || !B || !As || !Bs)) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)A & 3) || ((uintptr_t)B & 3) || ((uintptr_t)C & (f32out ? 3 : 1))) return MXFP6_EINVAL_ALIGN;
+  if ((long)M * N >= (1L << 40) || (long)K / 4 * 3 * 256 >= (1L << 31)) return MXFP6_EINVAL_SHAPE;
+  int rc = check_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (K == 0) {
+    hipError_t e = mxfp6::launch_fill_zero(C, (size_t)M * N * (f32out ? 4 : 2), s);
+    return e == hipSuccess ? MXFP6_OK : (int)e;
+  }
+  mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out};
+  const int force = g_force.load(std::memory_order_relaxed);
+  hipError_t e;
+  if (force == 1) {
+    e = mxfp6::launch_gemm_generic(g, s);
+  } else if (force == 2) {
+    if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
+    e = mxfp6::launch_gemm_tiled(g, s);
+  } else if (force == 3) {
+    if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
+    e = mxfp6::launch_gemm_skinny(g, s);
+  } else if (mxfp6::gemm_skinny_supports(g)) {
+    e = mxfp6::launch_gemm_skinny(g, s);
+  } else if (mxfp6::gemm_tiled_supports(g)) {
+    e = mxfp6::launch_gemm_tiled(g, s);
+  } else {
+    e = mxfp6::launch_gemm_generic(g, s);
+  }
+  return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+int mxfp6_gemm(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
+               int fmt_b, void* stream) {
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, stream);
+}
+
+int mxfp6_gemm_f32out(const void* A, const void* B, const void* As, const void* Bs, float* C, int M, int N, int K,
+                      int fmt_a, int fmt_b, void* stream) {
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, true, stream);
+}
+
+int mxfp6_set_kernel(int which) {
+  if (which < 0 || which > 3) return g_force.load();
+  return g_force.exchange(which);
+}
+
+int mxfp6_quantize(const float* X, void* packed, void* scales, int rows, int K, int fmt, void* stream) {
+  if (rows < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
+  if (fmt != MXFP6_FMT_E2M3 && fmt != MXFP6_FMT_E3M2) return MXFP6_EINVAL_FMT;
+  if (rows == 0 || K == 0) return MXFP6_OK;
+  if (!X || !packed || !scales) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)X & 15) || ((uintptr_t)packed & 3)) return MXFP6_EINVAL_ALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  hipError_t e = mxfp6::launch_quantize(X, (uint8_t*)packed, (uint8_t*)scales, rows, K, fmt, (hipStream_t)stream);
+  return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
+const char* mxfp6_strerror(int code) {
+  switch (code) {
+    case MXFP6_OK: return "success";
+    case MXFP6_EINVAL_PTR: return "mxfp6: a required pointer is NULL";
+    case MXFP6_EINVAL_SHAPE: return "mxfp6: bad shape (M, N, K >= 0 and K % 32 == 0 required; a forced kernel may need more)";
+    case MXFP6_EINVAL_FMT: return "mxfp6: format must be 2 (e2m3) or 3 (e3m2)";
+    case MXFP6_EINVAL_ALIGN: return "mxfp6: pointer alignment (packed operands 4 bytes, fp32 input 16 bytes)";
+    case MXFP6_ENODEVICE: return "mxfp6: the current device is not gfx950 (MI355X)";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "mxfp6: unknown error code";
+}
+
+int mxfp6_abi_version(void) { return 100; }
+
+// development knob (not part of the ABI header)
+int mxfp6_dev_set(const char* name, int value) {
+  if (!__builtin_strcmp(name, "tiled_waves")) { mxfp6::set_tiled_waves(value); return 0; }
+  return -1;
+}
+
+#pragma GCC visibility pop
+}  // extern "C"

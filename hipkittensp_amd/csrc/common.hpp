@@ -1,0 +1,58 @@
+// Shared device/host helpers for the MXFP6 GEMM kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mxfp6 {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define MXFP6_LDS __attribute__((address_space(3)))
+
+// Output element traits: the kernels are instantiated for bf16 (the operator) and float (the
+// unrounded accumulators, used to state the accuracy contract before the bf16 rounding).
+struct OutBf16 { typedef uint16_t type; };
+struct OutF32 { typedef float type; };
+
+// fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  f2 v = {lo, hi};
+  bf2 r = __builtin_convertvector(v, bf2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// Store 4 consecutive outputs (n .. n+3) of one row.
+__device__ __forceinline__ void store4(uint16_t* p, float a, float b, float c, float d) {
+  u32x2 v = {pack_bf16x2(a, b), pack_bf16x2(c, d)};
+  *reinterpret_cast<u32x2*>(p) = v;
+}
+__device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
+  v4f v = {a, b, c, d};
+  *reinterpret_cast<v4f*>(p) = v;
+}
+__device__ __forceinline__ void store1(uint16_t* p, float a) { *p = (uint16_t)(pack_bf16x2(a, 0.f) & 0xffffu); }
+__device__ __forceinline__ void store1(float* p, float a) { *p = a; }
+
+// Raw buffer resource over [base, base + bytes): out-of-range lanes of a buffer load read 0.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// D(32x32, fp32) += SA(32 x 64) . SB(32 x 64)^T with per-lane E8M0 block scales.
+//   lane l supplies row l%32, K-block l/32 (32 fp6 values = 6 dwords) of each source;
+//   result register v of lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32]   (row from SA, column from SB).
+//   OPA/OPB select which byte of the scale dword is used.
+template <int FMT_SA, int FMT_SB, int OPA, int OPB>
+__device__ __forceinline__ v16f mfma_fp6(v8i sa, v8i sb, v16f acc, int scale_sa, int scale_sb) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(sa, sb, acc, FMT_SA, FMT_SB, OPA, scale_sa, OPB, scale_sb);
+}
+
+}  // namespace mxfp6

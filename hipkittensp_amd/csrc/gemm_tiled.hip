@@ -1,0 +1,244 @@
+// LDS-tiled MXFP6 GEMM for gfx950: 256x256 output tile per workgroup, K-tile 128.
+//
+// Data path (no operand byte ever passes through a VGPR on its way to LDS):
+//   global --buffer_load_dwordx4 ... lds--> LDS (3-stage ring) --ds_read_b128--> MFMA source VGPRs
+//   v_mfma_scale_f32_32x32x64_f8f6f4 (fp32 accumulate, E8M0 block scales applied by the instruction)
+//   accumulators --v_cvt_pk_bf16_f32--> global
+//
+// LDS image of one operand tile (256 rows x 96 bytes = 6 chunks of 16 B per row): row-major, 96 bytes
+// per row, with chunks 2p and 2p+1 exchanged in every row whose bit 3 is set:
+//     chunk c of row r lives at  r * 96 + (c ^ ((r >> 3) & 1)) * 16.
+// A direct-to-LDS load writes lane l's 16 bytes at base + 16*l, so the image is produced by choosing
+// which global bytes each lane fetches (the same idea as the reference's swizzled global offsets,
+// include/ops/warp/memory/tile/global_to_shared.cuh:46-72).  Consecutive lanes fetch consecutive
+// 16-byte pieces of one row, so the texture-address unit sees 64..96 contiguous bytes per 4..6 lanes.
+// The pair exchange is what makes the reads conflict-free: a ds_read_b128 executes in 16-lane phases
+// ({0-3,12-15,20-23,24-27}, {4-11,16-19,28-31}, ... measured in
+// analysis/paper_experiments/phases/ds_read_b128/phase_results.txt:4-7); with a 96-byte pitch rows r
+// and r+8 would share banks, and every phase holds each (r mod 8) once with bit 3 clear and once set.
+//
+// MFMA operand mapping: lane l of a 32x32x64 MFMA supplies row l%32 and one 32-element K-block.  Lanes
+// 0-31 take K-blocks {0,1} of the K-tile and lanes 32-63 take K-blocks {2,3}: each lane reads its row's
+// 48 contiguous bytes (three aligned 16-byte chunks) once and feeds two MFMAs (K-blocks {0,2} then {1,3}).
+// Any assignment of K-blocks to lane halves is legal as long as both operands use the same one.
+//
+// E8M0 scales ride in LDS too: 16 bytes per row cover four K-tiles, fetched by one dwordx4 direct
+// load per 64 rows per four K-tiles; a lane reads the 2 bytes it needs with ds_read_u16 and the MFMA's
+// op_sel picks byte 0 / byte 1.
+//
+// Schedule: all waves are consumers (the reference measures all-consumer above producer/consumer,
+// analysis/paper_experiments/producer_consumer_micro/plot.py:26-30); one s_barrier per K-tile; DMA for
+// tile k+2 is issued right after the barrier that publishes tile k.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace mxfp6 {
+
+constexpr int kBM = 256, kBN = 256, kBK = 128;
+constexpr int kOpStage = 256 * 96;  // bytes of one operand tile
+constexpr int kScStage = 256 * 16;  // bytes of one operand's scales for four K-tiles
+constexpr int kGroupM = 4;          // tile rows per raster group
+constexpr int kStages = 3;          // operand ring depth
+
+// One direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff and the hardware
+// writes them at LDS address lds_base + 16 * lane.  Issued from inline assembly so that the VMEM
+// counter is managed by hand (wait_tile below): the ring keeps two K-tiles in flight across
+// barriers, which the compiler's automatic waits would serialise.  M0 is used by nothing else here.
+__device__ __forceinline__ void dma16(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_barrier() {
+  // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int FA, int FB, typename Out, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                                 const uint8_t* __restrict__ As,
+                                                                 const uint8_t* __restrict__ Bs,
+                                                                 typename Out::type* __restrict__ C, int M, int N, int K,
+                                                                 int tiles_m, int tiles_n) {
+  constexpr int NW = WM * WN;
+  constexpr int TM = 8 / WM, TN = 8 / WN;  // 32x32 MFMA tiles per wave in M and N
+  constexpr int OPS = 24 / NW;             // operand DMA instructions per wave per operand per K-tile
+  static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+  // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
+  constexpr int kStage = 2 * kOpStage, kScaleBase = kStages * kStage, kScaleBuf = 2 * kScStage;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[kScaleBase + 2 * kScaleBuf];
+  static_assert(sizeof(smem) <= 163840, "LDS budget");
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
+
+  // ---- workgroup -> output tile: undo the round-robin XCD placement, then a grouped raster.
+  // Hardware places workgroup b on XCD b % 8; remapping gives each XCD a contiguous run of logical
+  // tiles so that the 32 tiles an XCD works on at once share operand rows in its L2
+  // (the idea of chiplet_transform_chunked, include/common/util.cuh:78-101, as an exact bijection).
+  const int nb = tiles_m * tiles_n;
+  int L;
+  {
+    const int bid = blockIdx.x, xcd = bid & 7, idx = bid >> 3;
+    const int per = nb >> 3, rem = nb & 7;
+    L = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+  }
+  int pm, pn;
+  {
+    const int width = kGroupM * tiles_n, group = L / width, first = group * kGroupM;
+    const int gsz = min(tiles_m - first, kGroupM), in = L - group * width;
+    pm = first + in % gsz;
+    pn = in / gsz;
+  }
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int h = lane >> 5, r32 = lane & 31;
+
+  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK;
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A + (size_t)pm * kBM * rowbytes, (uint32_t)kBM * rowbytes);
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)pn * kBN * rowbytes, (uint32_t)kBN * rowbytes);
+  const __amdgpu_buffer_rsrc_t rSA = make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)kBM * sbytes);
+  const __amdgpu_buffer_rsrc_t rSB = make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)kBN * sbytes);
+
+  // per-lane global byte offsets of the OPS direct loads (identical for A and B: same row pitch)
+  int voff[OPS];
+#pragma unroll
+  for (int i = 0; i < OPS; i++) {
+    const int o = (wave * OPS + i) * 64 + lane;  // linear 16-byte slot inside the LDS image
+    const int r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
+    voff[i] = r * rowbytes + c * 16;
+  }
+  // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; with 4 waves every wave
+  // loads 64 rows of A and of B, with 8 waves waves 0-3 load A and waves 4-7 load B
+  const int voff_s = ((wave & 3) * 64 + lane) * sbytes;
+
+  // per-lane LDS read offsets (bytes from the start of a stage): the lane's three chunks 3h..3h+2
+  const int sw = (r32 >> 3) & 1;
+  int a_rd[3], b_rd[3];
+#pragma unroll
+  for (int c = 0; c < 3; c++) {
+    a_rd[c] = (wm * (TM * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
+    b_rd[c] = kOpStage + (wn * (TN * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
+  }
+  const int sa_rd = kScaleBase + (wm * (TM * 32) + r32) * 16 + 2 * h;
+  const int sb_rd = kScaleBase + kScStage + (wn * (TN * 32) + r32) * 16 + 2 * h;
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+  // ---- DMA issue slot of K-tile t: its operand loads, then (every fourth tile) the scales of the
+  // four K-tiles starting at t + 2.  Every slot therefore ends with at most a scale load, and a
+  // wait that leaves 2*OPS loads outstanding always covers the whole previous slot.
+  auto issue_scales = [&](int grp) {
+    const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + (wave & 3) * 1024;
+    const int soff = grp * 16;
+    if (NW == 4 || wave < 4) dma16(rSA, dst, voff_s, soff);
+    if (NW == 4 || wave >= 4) dma16(rSB, dst + kScStage, voff_s, soff);
+  };
+  auto issue_slot = [&](int t) {
+    const uint32_t dst = lds0 + (t % kStages) * kStage + wave * (OPS * 1024);
+    const int soff = t * 96;
+#pragma unroll
+    for (int i = 0; i < OPS; i++) dma16(rA, dst + i * 1024, voff[i], soff);
+#pragma unroll
+    for (int i = 0; i < OPS; i++) dma16(rB, dst + kOpStage + i * 1024, voff[i], soff);
+    if ((t & 3) == 2 && t + 2 < nkt) issue_scales((t + 2) >> 2);
+  };
+
+  // ---- prologue: scales of the first four K-tiles, then K-tiles 0 and 1
+  issue_scales(0);
+  issue_slot(0);
+  if (nkt > 1) issue_slot(1);
+
+  for (int kt = 0; kt < nkt; kt++) {
+    // tile kt has landed (this wave's share) once at most the next slot's 2*OPS loads are pending;
+    // the barrier publishes every wave's share and retires the ring slot tile kt+2 will overwrite
+    if (kt + 1 < nkt) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();
+    if (kt + 2 < nkt) issue_slot(kt + 2);
+
+    const uint8_t* st = smem + (kt % kStages) * kStage;
+    const uint8_t* sc = smem + ((kt >> 2) & 1) * kScaleBuf + (kt & 3) * 4;
+    v4i fa[TM][3], fb[TN][3];
+    int sca[TM], scb[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+      for (int c = 0; c < 3; c++) fb[j][c] = *reinterpret_cast<const v4i*>(st + b_rd[c] + j * 3072);
+      scb[j] = *reinterpret_cast<const uint16_t*>(sc + sb_rd + j * 512);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int c = 0; c < 3; c++) fa[i][c] = *reinterpret_cast<const v4i*>(st + a_rd[c] + i * 3072);
+      sca[i] = *reinterpret_cast<const uint16_t*>(sc + sa_rd + i * 512);
+    }
+    // first K-block of every lane for all tiles, then the second: two MFMAs into the same
+    // accumulator are TM*TN instructions apart.  First source = B rows (index n), second = A rows
+    // (index m): a lane ends up owning 4 consecutive n of one m, which keeps the C store wide.
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const v8i a0 = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, -1, -1);
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const v8i b0 = __builtin_shufflevector(fb[j][0], fb[j][1], 0, 1, 2, 3, 4, 5, -1, -1);
+        acc[i][j] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[i][j], scb[j], sca[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const v8i a1 = __builtin_shufflevector(fa[i][1], fa[i][2], 2, 3, 4, 5, 6, 7, -1, -1);
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const v8i b1 = __builtin_shufflevector(fb[j][1], fb[j][2], 2, 3, 4, 5, 6, 7, -1, -1);
+        acc[i][j] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[i][j], scb[j], sca[i]);
+      }
+    }
+  }
+
+  // ---- epilogue: lane owns C[m][n .. n+3] for 4 values of n per 32x32 tile
+  typename Out::type* cbase = C + ((size_t)pm * kBM + wm * (TM * 32) + r32) * (size_t)N + (size_t)pn * kBN + wn * (TN * 32) + 4 * h;
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++)
+        store4(cbase + (size_t)i * 32 * N + j * 32 + 8 * g, acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+               acc[i][j][4 * g + 3]);
+}
+
+bool gemm_tiled_supports(const GemmArgs& g) {
+  return g.M > 0 && g.N > 0 && g.K > 0 && g.M % kBM == 0 && g.N % kBN == 0 && g.K % kBK == 0 &&
+         (long)kBM * (g.K / 4 * 3) < (1L << 31) && ((uintptr_t)g.C % (g.f32out ? 16 : 8)) == 0;
+}
+
+static int g_tiled_waves = 8;
+void set_tiled_waves(int w) { g_tiled_waves = w; }
+
+template <int FA, int FB, typename Out>
+static hipError_t launch(const GemmArgs& g, hipStream_t s) {
+  const int tm = g.M / kBM, tn = g.N / kBN;
+  if (g_tiled_waves == 4)
+    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn);
+  else
+    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s) {
+#define MXFP6_CASE(FA, FB) \
+  if (g.fmt_a == FA && g.fmt_b == FB) return g.f32out ? launch<FA, FB, OutF32>(g, s) : launch<FA, FB, OutBf16>(g, s);
+  MXFP6_CASE(2, 2) MXFP6_CASE(2, 3) MXFP6_CASE(3, 2) MXFP6_CASE(3, 3)
+#undef MXFP6_CASE
+  return hipErrorInvalidValue;
+}
+
+}  // namespace mxfp6

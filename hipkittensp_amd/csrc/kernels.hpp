@@ -1,0 +1,25 @@
+// Internal launcher interface between the C ABI (api.hip) and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mxfp6 {
+
+struct GemmArgs {
+  const uint8_t *A, *B, *As, *Bs;  // packed operands and E8M0 scales (device)
+  void* C;                         // bf16 or float [M, N]
+  int M, N, K;
+  int fmt_a, fmt_b;  // 2 = e2m3, 3 = e3m2
+  bool f32out;
+};
+
+hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
+bool gemm_tiled_supports(const GemmArgs& g);
+hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
+void set_tiled_waves(int w);
+bool gemm_skinny_supports(const GemmArgs& g);
+hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
+hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, hipStream_t s);
+hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t s);
+
+}  // namespace mxfp6

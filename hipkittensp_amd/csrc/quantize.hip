@@ -1,0 +1,112 @@
+// fp32 -> MXFP6 quantise + pack on the GPU, and the zero fill used for K == 0.
+// One lane handles one 32-element block: 128 bytes in (8 x 16-byte loads), 24 bytes + 1 scale byte out.
+// HBM-bound elementwise work: 4 B/element read, 0.78 B/element written.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace mxfp6 {
+
+// Round a non-negative, already scaled magnitude to the fp6 grid (ties to even, saturating) with
+// integer arithmetic on the fp32 bits.  MB = mantissa bits, BIAS = exponent bias, EB = exponent bits.
+template <int MB, int BIAS, int EB>
+__device__ __forceinline__ uint32_t quantise_mag(float a) {
+  const uint32_t u = __float_as_uint(a);
+  if (a != a) return 31u;
+  const int be = (int)(u >> 23);
+  if (be == 0) return 0u;  // fp32 subnormal: far below half of the smallest fp6 step
+  const int ex = be - 127;
+  constexpr int emin = 1 - BIAS;
+  const int e = ex < emin ? emin : ex;
+  const int shift = 23 - MB + (e - ex);
+  uint32_t q = 0;
+  if (shift < 32) {
+    const uint32_t man = (u & 0x7FFFFFu) | 0x800000u;
+    const uint32_t half = 1u << (shift - 1), frac = man & ((half << 1) - 1);
+    q = man >> shift;
+    q += (frac > half || (frac == half && (q & 1u))) ? 1u : 0u;
+  }
+  uint32_t code;
+  if (ex < emin) {
+    code = q;  // subnormal (q == 2^MB lands on the smallest normal)
+  } else {
+    int ee = e;
+    if (q == (2u << MB)) { q = 1u << MB; ee += 1; }
+    code = ((uint32_t)(ee + BIAS) << MB) | (q - (1u << MB));
+    if (ee + BIAS >= (1 << EB)) code = 31u;
+  }
+  return code > 31u ? 31u : code;
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ X, uint8_t* __restrict__ packed,
+                                                       uint8_t* __restrict__ scales, long nblocks) {
+  constexpr int MB = FMT == 2 ? 3 : 2, BIAS = FMT == 2 ? 1 : 3, EB = FMT == 2 ? 2 : 3, EMAX = FMT == 2 ? 2 : 4;
+  const long b = (long)blockIdx.x * 256 + threadIdx.x;
+  if (b >= nblocks) return;
+  const v4f* src = reinterpret_cast<const v4f*>(X + b * 32);
+  v4f x[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) x[i] = src[i];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) amax = fmaxf(amax, fabsf(x[i][j]));
+  int sb = 0;
+  if (amax > 0.f) {
+    const uint32_t u = __float_as_uint(amax);
+    const int be = (int)(u >> 23);
+    const int fl = be ? be - 127 : (31 - __clz((int)u)) - 149;  // floor(log2(amax)), fp32 subnormals included
+    sb = fl - EMAX + 127;
+    sb = sb < 0 ? 0 : (sb > 254 ? 254 : sb);
+  }
+  // multiply by 2^(127 - sb) exactly: split the power of two so that each factor is a normal fp32
+  const int ex = 127 - sb;  // in [-127, 127]
+  const float f1 = __uint_as_float((uint32_t)((ex / 2) + 127) << 23);
+  const float f2 = __uint_as_float((uint32_t)((ex - ex / 2) + 127) << 23);
+  uint32_t w[6] = {0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    uint32_t g = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const float v = x[i][j];
+      const float y = fabsf(v) * f1 * f2;
+      const uint32_t code = quantise_mag<MB, BIAS, EB>(y) | ((__float_as_uint(v) >> 31) << 5);
+      g |= code << (6 * j);
+    }
+    // group i is 24 bits at bit 24*i of the 192-bit block
+    const int bit = 24 * i, d = bit >> 5, sh = bit & 31;
+    w[d] |= g << sh;
+    if (sh > 8) w[d + 1] |= g >> (32 - sh);
+  }
+  uint32_t* dst = reinterpret_cast<uint32_t*>(packed + b * 24);
+#pragma unroll
+  for (int i = 0; i < 6; i++) dst[i] = w[i];
+  scales[b] = (uint8_t)sb;
+}
+
+hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, hipStream_t s) {
+  const long nblocks = (long)rows * (K / 32);
+  const unsigned grid = (unsigned)((nblocks + 255) / 256);
+  if (fmt == 2)
+    quantize_kernel<2><<<grid, 256, 0, s>>>(X, packed, scales, nblocks);
+  else
+    quantize_kernel<3><<<grid, 256, 0, s>>>(X, packed, scales, nblocks);
+  return hipGetLastError();
+}
+
+__global__ void fill_zero_kernel(uint8_t* p, size_t n) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, st = (size_t)gridDim.x * 256;
+  for (; i < n; i += st) p[i] = 0;
+}
+
+hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t s) {
+  size_t blocks = (bytes + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks == 0) return hipSuccess;
+  fill_zero_kernel<<<(unsigned)blocks, 256, 0, s>>>((uint8_t*)p, bytes);
+  return hipGetLastError();
+}
+
+}  // namespace mxfp6

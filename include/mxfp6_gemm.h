@@ -1,0 +1,91 @@
+/*
+ * mxfp6_gemm.h -- C ABI of the MI355X (gfx950) MXFP6 block-scaled GEMM.
+ *
+ *   C[M,N] = dq(A)[M,K] . dq(B)[N,K]^T        fp32 accumulation, bf16 (or fp32) output
+ *
+ * Operands are packed fp6 (e2m3 or e3m2, chosen per operand): row-major, K contiguous, value j of
+ * a row at bits [6j, 6j+6) of the row's little-endian bitstream (4 values per 3 bytes, so a row is
+ * 3K/4 bytes and a 32-element block is 24 contiguous bytes).  Each 32-element K-block of each row
+ * carries one E8M0 scale byte (value 2^(b-127)); scale tensors are row-major [rows, K/32] uint8.
+ *
+ * This is the library a binding replaces the reference's per-kernel pybind module with.  The
+ * reference convention it follows (benenzhu/HipKittensP):
+ *   - entry point dispatch_micro(A, B, C): tensors in, C written in place, returns nothing,
+ *     asynchronous launch, caller synchronises          analysis/bf16_gemm/mi325x/kernel_8192.cpp:227-237
+ *   - C = A . B^T with both operands K-contiguous        kernels/gemm/bf16fp32/utils.py:28-37
+ *   - tensor -> raw pointer conversion at the boundary   include/pyutils/pyutils.cuh:15-72
+ * All pointers are DEVICE pointers.  All functions return 0 on success, a negative MXFP6_E* code
+ * for rejected arguments (nothing launched), or a positive hipError_t value if the runtime failed.
+ * No function allocates device memory or synchronises; work is queued on `hip_stream`
+ * (a hipStream_t; NULL = the null stream).
+ */
+#ifndef MXFP6_GEMM_H
+#define MXFP6_GEMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* operand formats: the numbering of the scaled-MFMA format field */
+#define MXFP6_FMT_E2M3 2
+#define MXFP6_FMT_E3M2 3
+
+#define MXFP6_OK 0
+#define MXFP6_EINVAL_PTR (-1)   /* a required pointer is NULL                                  */
+#define MXFP6_EINVAL_SHAPE (-2) /* M, N or K negative, K not a multiple of 32, or out of range */
+#define MXFP6_EINVAL_FMT (-3)   /* format code is not 2 (e2m3) or 3 (e3m2)                     */
+#define MXFP6_EINVAL_ALIGN (-4) /* a pointer violates the stated alignment                     */
+#define MXFP6_ENODEVICE (-5)    /* current device is not gfx950                                */
+
+/*
+ * The operator.  Replaces the reference's dispatch_micro(A, B, C) launcher
+ * (analysis/bf16_gemm/mi325x/kernel_8192.cpp:227-231, distributed-kernels/bf16_gemm/kernel.cpp:247-265)
+ * for packed-fp6 operands with E8M0 block scales.
+ *   A_packed [M, 3K/4] u8, B_packed [N, 3K/4] u8, A_scale [M, K/32] u8, B_scale [N, K/32] u8,
+ *   C [M, N] bf16 row-major.  K % 32 == 0.  A_packed/B_packed 4-byte aligned, C 2-byte aligned.
+ *   M == 0 or N == 0 is a successful no-op; K == 0 writes zeros.
+ */
+int mxfp6_gemm(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, void *C_bf16,
+               int M, int N, int K, int fmt_a, int fmt_b, void *hip_stream);
+
+/*
+ * Same product with the fp32 accumulators stored unrounded (C is float [M, N]).  The accuracy
+ * contract (max relative error vs the fp32 dequantise-and-matmul) is stated before the bf16
+ * rounding, so this is the entry the parity tests measure; it shares every kernel with mxfp6_gemm.
+ * Reference analogue: the float accumulator tile the reference converts at store time
+ * (analysis/bf16_gemm/mi325x/kernel_8192.cpp:223-224).
+ */
+int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale,
+                      float *C_f32, int M, int N, int K, int fmt_a, int fmt_b, void *hip_stream);
+
+/*
+ * Kernel selection override for measurement and tests: 0 = automatic (default), 1 = generic
+ * one-wave-per-tile kernel, 2 = LDS-tiled MFMA kernel (needs M,N % 256 == 0, K % 128 == 0),
+ * 3 = skinny-M streaming kernel (needs M <= 32).  A forced kernel that cannot run the given
+ * shape makes the gemm calls return MXFP6_EINVAL_SHAPE.  Returns the previous value.
+ * No counterpart in the reference, whose shapes are compile-time constants per binary
+ * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
+ */
+int mxfp6_set_kernel(int which);
+
+/*
+ * Quantise + pack on the GPU: X [rows, K] fp32 row-major -> packed [rows, 3K/4] u8 + scales
+ * [rows, K/32] u8, scale = 2^(floor(log2(blockmax)) - emax(fmt)) (emax 2 for e2m3, 4 for e3m2),
+ * round-to-nearest-even, saturating; an all-zero block gets scale byte 0.  K % 32 == 0.
+ * The producer of this path's inputs; the reference's harness creates its operands on the device
+ * the same way (kernels/gemm/bf16fp32/utils.py:28-34).
+ */
+int mxfp6_quantize(const float *X, void *packed, void *scales, int rows, int K, int fmt, void *hip_stream);
+
+/* Human-readable text for a return code of this library (never NULL). */
+const char *mxfp6_strerror(int code);
+
+/* ABI version of this header: major * 100 + minor. */
+int mxfp6_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXFP6_GEMM_H */
