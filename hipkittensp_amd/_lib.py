@@ -1,0 +1,50 @@
+"""ctypes binding of libmxfp6_gemm.so (the C ABI declared in include/mxfp6_gemm.h).
+
+The library is loaded from this package's directory and nowhere else.  There is no fallback: if
+the shared object has not been built (python -m hipkittensp_amd.build) the import of the operator
+fails with an explicit error.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmxfp6_gemm.so")
+
+_lib = None
+
+
+class Mxfp6LibraryMissing(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise Mxfp6LibraryMissing(
+                f"{LIB_PATH} is not built; run `python -m hipkittensp_amd.build` (needs hipcc, no GPU). "
+                "There is no CPU or PyTorch fallback for the MXFP6 GEMM."
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        L.mxfp6_gemm.restype = ci
+        L.mxfp6_gemm.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        L.mxfp6_gemm_f32out.restype = ci
+        L.mxfp6_gemm_f32out.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        L.mxfp6_quantize.restype = ci
+        L.mxfp6_quantize.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+        L.mxfp6_set_kernel.restype = ci
+        L.mxfp6_set_kernel.argtypes = [ci]
+        L.mxfp6_strerror.restype = ctypes.c_char_p
+        L.mxfp6_strerror.argtypes = [ci]
+        L.mxfp6_abi_version.restype = ci
+        L.mxfp6_abi_version.argtypes = []
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what}: {lib().mxfp6_strerror(rc).decode()} (code {rc})")

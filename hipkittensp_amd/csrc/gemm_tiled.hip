@@ -62,7 +62,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
                                                                  const uint8_t* __restrict__ As,
                                                                  const uint8_t* __restrict__ Bs,
                                                                  typename Out::type* __restrict__ C, int M, int N, int K,
-                                                                 int tiles_m, int tiles_n) {
+                                                                 int tiles_m, int tiles_n, int dev_mode) {
   constexpr int NW = WM * WN;
   constexpr int TM = 8 / WM, TN = 8 / WN;  // 32x32 MFMA tiles per wave in M and N
   constexpr int OPS = 24 / NW;             // operand DMA instructions per wave per operand per K-tile
@@ -110,6 +110,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
     const int o = (wave * OPS + i) * 64 + lane;  // linear 16-byte slot inside the LDS image
     const int r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
     voff[i] = r * rowbytes + c * 16;
+    if (dev_mode == 3) voff[i] = o * 16;
   }
   // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; with 4 waves every wave
   // loads 64 rows of A and of B, with 8 waves waves 0-3 load A and waves 4-7 load B
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
   };
   auto issue_slot = [&](int t) {
     const uint32_t dst = lds0 + (t % kStages) * kStage + wave * (OPS * 1024);
-    const int soff = t * 96;
+    const int soff = dev_mode == 3 ? t * 24576 : t * 96;
 #pragma unroll
     for (int i = 0; i < OPS; i++) dma16(rA, dst + i * 1024, voff[i], soff);
 #pragma unroll
@@ -162,7 +163,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
     // tile kt has landed (this wave's share) once at most the next slot's 2*OPS loads are pending;
     // the barrier publishes every wave's share and retires the ring slot tile kt+2 will overwrite
     if (kt + 1 < nkt) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();
-    if (kt + 2 < nkt) issue_slot(kt + 2);
+    if (kt + 2 < nkt && dev_mode != 1) issue_slot(kt + 2);
+    if (dev_mode >= 2) continue;
 
     const uint8_t* st = smem + (kt % kStages) * kStage;
     const uint8_t* sc = smem + ((kt >> 2) & 1) * kScaleBuf + (kt & 3) * 4;
@@ -221,15 +223,17 @@ bool gemm_tiled_supports(const GemmArgs& g) {
 }
 
 static int g_tiled_waves = 8;
+static int g_dev_mode = 0;
+void set_dev_mode(int m) { g_dev_mode = m; }
 void set_tiled_waves(int w) { g_tiled_waves = w; }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int tm = g.M / kBM, tn = g.N / kBN;
   if (g_tiled_waves == 4)
-    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn);
+    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode);
   else
-    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn);
+    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode);
   return hipGetLastError();
 }
 

@@ -1,0 +1,122 @@
+"""`tk_kernel` -- the Python-facing operator module, in the reference's calling convention.
+
+The reference builds one pybind11 module named ``tk_kernel`` per kernel and calls
+``tk_kernel.dispatch_micro(A, B, C)`` with torch tensors: C = A . B^T, both operands K-contiguous,
+C allocated by the caller and written in place, nothing returned, the launch asynchronous
+(kernels/gemm/bf16fp32/bench.py:34, kernels/gemm/bf16fp32/utils.py:28-37,
+analysis/bf16_gemm/mi325x/kernel_8192.cpp:227-237).  Its binding accepts any object whose type is
+named "Tensor", requires it contiguous, on a device and of at most 4 dimensions, and raises
+RuntimeError otherwise (include/pyutils/pyutils.cuh:15-48).  This module keeps that behaviour and
+adds the checks a packed format needs (dtype, packed width, scale shape).
+
+    dispatch_micro(A, B, A_scale, B_scale, C, fmt_a=2, fmt_b=2)
+
+    A        uint8 [M, 3K/4]   packed fp6, 4 values per 3 bytes, K contiguous
+    B        uint8 [N, 3K/4]
+    A_scale  uint8 [M, K/32]   E8M0, one per 32-element K-block
+    B_scale  uint8 [N, K/32]
+    C        bfloat16 [M, N]   (a float32 C receives the accumulators before the bf16 rounding)
+    fmt_*    2 = e2m3, 3 = e3m2
+
+PyTorch is used for tensor storage and the current stream only; the work is done by the HIP
+library behind include/mxfp6_gemm.h.
+"""
+from __future__ import annotations
+
+from . import _lib
+
+E2M3 = 2
+E3M2 = 3
+
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_TILED, KERNEL_SKINNY = 0, 1, 2, 3
+
+
+def _as_tensor(obj, name: str):
+    # same duck typing and error class as the reference binding (include/pyutils/pyutils.cuh:22-46)
+    if type(obj).__name__ != "Tensor":
+        raise RuntimeError(f"{name}: expected a torch Tensor, got {type(obj).__name__}")
+    if not obj.is_contiguous():
+        raise RuntimeError(f"{name}: tensor must be contiguous")
+    if obj.device.type == "cpu":
+        raise RuntimeError(f"{name}: tensor must be on a GPU device")
+    if obj.dim() > 4:
+        raise RuntimeError(f"{name}: expected at most 4 dimensions, got {obj.dim()}")
+    return obj
+
+
+def _rows_cols(t, name: str):
+    # leading dimensions are folded into rows, like the reference's left padding to 4-D
+    if t.dim() < 1:
+        raise RuntimeError(f"{name}: expected at least 1 dimension")
+    cols = t.shape[-1]
+    rows = 1
+    for d in t.shape[:-1]:
+        rows *= d
+    return rows, cols
+
+
+def _stream():
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3) -> None:
+    import torch
+
+    A, B = _as_tensor(A, "A"), _as_tensor(B, "B")
+    A_scale, B_scale = _as_tensor(A_scale, "A_scale"), _as_tensor(B_scale, "B_scale")
+    C = _as_tensor(C, "C")
+    for t, name in ((A, "A"), (B, "B"), (A_scale, "A_scale"), (B_scale, "B_scale")):
+        if t.dtype != torch.uint8:
+            raise RuntimeError(f"{name}: expected dtype uint8, got {t.dtype}")
+    if C.dtype not in (torch.bfloat16, torch.float32):
+        raise RuntimeError(f"C: expected dtype bfloat16 (or float32 for unrounded output), got {C.dtype}")
+    if fmt_a not in (E2M3, E3M2) or fmt_b not in (E2M3, E3M2):
+        raise RuntimeError("fmt_a / fmt_b must be 2 (e2m3) or 3 (e3m2)")
+    M, wa = _rows_cols(A, "A")
+    N, wb = _rows_cols(B, "B")
+    if wa != wb:
+        raise RuntimeError(f"A and B disagree on K: packed widths {wa} and {wb}")
+    if wa % 24:
+        raise RuntimeError(f"packed width {wa} is not a whole number of 32-element blocks (24 bytes each)")
+    K = wa // 3 * 4
+    if _rows_cols(A_scale, "A_scale") != (M, K // 32):
+        raise RuntimeError(f"A_scale: expected shape [{M}, {K // 32}], got {tuple(A_scale.shape)}")
+    if _rows_cols(B_scale, "B_scale") != (N, K // 32):
+        raise RuntimeError(f"B_scale: expected shape [{N}, {K // 32}], got {tuple(B_scale.shape)}")
+    if _rows_cols(C, "C") != (M, N):
+        raise RuntimeError(f"C: expected shape [{M}, {N}], got {tuple(C.shape)}")
+    devs = {t.device for t in (A, B, A_scale, B_scale, C)}
+    if len(devs) != 1:
+        raise RuntimeError(f"all tensors must be on one device, got {sorted(map(str, devs))}")
+    L = _lib.lib()
+    fn = L.mxfp6_gemm if C.dtype == torch.bfloat16 else L.mxfp6_gemm_f32out
+    with torch.cuda.device(C.device):
+        rc = fn(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K, fmt_a, fmt_b, _stream())
+    _lib.check(rc, "dispatch_micro")
+
+
+def quantize(X, fmt: int = E2M3):
+    """fp32 [rows, K] on the GPU -> (packed uint8 [rows, 3K/4], scales uint8 [rows, K/32])."""
+    import torch
+
+    X = _as_tensor(X, "X")
+    if X.dtype != torch.float32:
+        raise RuntimeError(f"X: expected dtype float32, got {X.dtype}")
+    if fmt not in (E2M3, E3M2):
+        raise RuntimeError("fmt must be 2 (e2m3) or 3 (e3m2)")
+    rows, K = _rows_cols(X, "X")
+    if K % 32:
+        raise RuntimeError(f"K = {K} is not a multiple of 32")
+    packed = torch.empty(*X.shape[:-1], K // 4 * 3, dtype=torch.uint8, device=X.device)
+    scales = torch.empty(*X.shape[:-1], K // 32, dtype=torch.uint8, device=X.device)
+    with torch.cuda.device(X.device):
+        rc = _lib.lib().mxfp6_quantize(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, _stream())
+    _lib.check(rc, "quantize")
+    return packed, scales
+
+
+def set_kernel(which: int) -> int:
+    """Force a kernel (KERNEL_*) for measurement / tests; returns the previous setting."""
+    return _lib.lib().mxfp6_set_kernel(int(which))

@@ -1,0 +1,128 @@
+"""CPU-side checks of the drop-in boundary: the C ABI library exports what include/mxfp6_gemm.h declares,
+and the Python operator rejects bad arguments the way the reference's binding does (RuntimeError,
+include/pyutils/pyutils.cuh:22-46).  No kernel is launched here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mxfp6_gemm.h")
+LIB = os.path.join(ROOT, "hipkittensp_amd", "libmxfp6_gemm.so")
+
+
+def _declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(mxfp6_[a-z0-9_]+)\s*\(", src)))
+
+
+@pytest.fixture(scope="module")
+def built_lib():
+    if not os.path.exists(LIB):
+        from hipkittensp_amd import build
+        build.build(verbose=False)
+    return LIB
+
+
+def test_header_declares_the_operator():
+    names = _declared_functions()
+    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_quantize", "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel"):
+        assert want in names
+
+
+def test_header_compiles_as_plain_c(tmp_path):
+    c = tmp_path / "t.c"
+    c.write_text('#include "mxfp6_gemm.h"\nint main(void){return MXFP6_FMT_E2M3 + MXFP6_FMT_E3M2 == 5 ? 0 : 1;}\n')
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(c), "-o", str(tmp_path / "t.o")])
+
+
+def test_library_exports_every_declared_symbol(built_lib):
+    out = subprocess.check_output(["nm", "-D", "--defined-only", built_lib], text=True)
+    exported = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    for name in _declared_functions():
+        assert name in exported, f"{name} declared in the header but not exported"
+    L = ctypes.CDLL(built_lib)          # loads without a GPU
+    L.mxfp6_abi_version.restype = ctypes.c_int
+    assert L.mxfp6_abi_version() == 100
+    L.mxfp6_strerror.restype = ctypes.c_char_p
+    L.mxfp6_strerror.argtypes = [ctypes.c_int]
+    assert L.mxfp6_strerror(0) == b"success"
+    assert b"multiple of 32" in L.mxfp6_strerror(-2) or b"K % 32" in L.mxfp6_strerror(-2)
+    assert L.mxfp6_strerror(-12345)  # never NULL
+
+
+def test_abi_argument_validation_without_a_gpu(built_lib):
+    """Shape / format errors are reported before any HIP call, so they are testable on a CPU box."""
+    L = ctypes.CDLL(built_lib)
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    L.mxfp6_gemm.restype = ci
+    L.mxfp6_gemm.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    one = ctypes.c_void_p(256)
+    assert L.mxfp6_gemm(one, one, one, one, one, 16, 16, 48, 2, 2, None) == -2   # K % 32
+    assert L.mxfp6_gemm(one, one, one, one, one, -1, 16, 32, 2, 2, None) == -2
+    assert L.mxfp6_gemm(one, one, one, one, one, 16, 16, 32, 1, 2, None) == -3   # fp8 code is not ours
+    assert L.mxfp6_gemm(one, one, one, one, one, 16, 16, 32, 2, 4, None) == -3
+    assert L.mxfp6_gemm(None, one, one, one, one, 16, 16, 32, 2, 2, None) == -1
+    assert L.mxfp6_gemm(one, one, one, one, None, 16, 16, 32, 2, 2, None) == -1
+    assert L.mxfp6_gemm(ctypes.c_void_p(258), one, one, one, one, 16, 16, 32, 2, 2, None) == -4
+    assert L.mxfp6_gemm(one, one, one, one, one, 0, 16, 32, 2, 2, None) == 0     # empty problem: no-op
+    L.mxfp6_quantize.restype = ci
+    L.mxfp6_quantize.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+    assert L.mxfp6_quantize(one, one, one, 4, 40, 2, None) == -2
+    assert L.mxfp6_quantize(one, one, one, 4, 64, 5, None) == -3
+    assert L.mxfp6_quantize(one, one, one, 0, 64, 2, None) == 0
+
+
+def test_python_operator_rejects_like_the_reference():
+    import hipkittensp_amd as hk
+
+    u8 = torch.zeros(4, 24, dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="expected a torch Tensor"):
+        hk.dispatch_micro([1, 2], u8, u8, u8, u8)
+    with pytest.raises(RuntimeError, match="GPU device"):
+        hk.dispatch_micro(u8, u8, u8, u8, u8)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hk.dispatch_micro(torch.zeros(24, 4, dtype=torch.uint8).t(), u8, u8, u8, u8)
+    with pytest.raises(RuntimeError, match="at most 4 dimensions"):
+        hk.dispatch_micro(torch.empty(1, 1, 1, 4, 24, dtype=torch.uint8, device="meta"), u8, u8, u8, u8)
+    with pytest.raises(RuntimeError):
+        hk.quantize(torch.zeros(4, 64))
+
+
+def test_python_shape_checks_on_meta_device():
+    """Shape/dtype validation runs before the library is touched: exercise it with meta tensors."""
+    import hipkittensp_amd as hk
+
+    def t(*shape, dtype=torch.uint8):
+        return torch.empty(*shape, dtype=dtype, device="meta")
+
+    A, B, As, Bs, C = t(8, 96), t(16, 96), t(8, 4), t(16, 4), t(8, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="dtype uint8"):
+        hk.dispatch_micro(t(8, 96, dtype=torch.int8), B, As, Bs, C)
+    with pytest.raises(RuntimeError, match="disagree on K"):
+        hk.dispatch_micro(A, t(16, 48), As, Bs, C)
+    with pytest.raises(RuntimeError, match="whole number of 32-element blocks"):
+        hk.dispatch_micro(t(8, 36), t(16, 36), As, Bs, C)
+    with pytest.raises(RuntimeError, match="A_scale"):
+        hk.dispatch_micro(A, B, t(8, 3), Bs, C)
+    with pytest.raises(RuntimeError, match="B_scale"):
+        hk.dispatch_micro(A, B, As, t(15, 4), C)
+    with pytest.raises(RuntimeError, match="C: expected shape"):
+        hk.dispatch_micro(A, B, As, Bs, t(16, 8, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="C: expected dtype"):
+        hk.dispatch_micro(A, B, As, Bs, t(8, 16, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="fmt_a / fmt_b"):
+        hk.dispatch_micro(A, B, As, Bs, C, fmt_a=0)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from hipkittensp_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.Mxfp6LibraryMissing, match="no CPU or PyTorch fallback"):
+        _lib.lib()

@@ -1,0 +1,274 @@
+"""GPU parity: the HIP path (called through the C ABI via hipkittensp_amd.tk_kernel) against the CPU
+oracle on the same seeded inputs.  Bars (BASELINE.json): fp6 -> fp32 decode bit-exact; GEMM within
+max relative error 2e-3 of the dequantise-and-matmul result, measured on the fp32 accumulators
+before the bf16 rounding (metric: oracle.rel_err); bf16 output = RNE of those accumulators;
+quantiser bit-exact.  Full-size configurations are checked on sampled rows/columns against the
+fp64 oracle plus size-independent properties (exact scale linearity, operand swap = transpose,
+kernel-vs-kernel agreement)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import mxfp6_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3  # BASELINE.json north_star: max relative error vs the fp32 dequantise-and-matmul
+# What the hardware actually delivers, measured on MI355X: with at least one e2m3 operand every fp6
+# product and every partial sum of these workloads is exactly representable and the scaled MFMA
+# returns the fp64 result rounded once (metric 0 .. 1e-7), so those cases are held to 1e-5.  With
+# e3m2 on BOTH operands the MFMA's internal sum of the 64 products of a K-pair is itself inexact
+# (|err| up to 3e-5 of sum|a||b|, metric up to 6e-3 where results cancel); that combination is not
+# one of BASELINE.json's configurations and is held to 1e-2 plus a bound relative to sum|a||b|.
+TOL_TIGHT = 1e-5
+TOL_E3M2_BOTH = 1e-2
+
+
+def tol(fa, fb):
+    return TOL_E3M2_BOTH if (fa == 3 and fb == 3) else TOL_TIGHT
+
+
+def check(got, ref, fa, fb, ap=None, asc=None, bp=None, bsc=None):
+    assert np.isfinite(got).all()
+    e = o.rel_err(got, ref)
+    assert e <= tol(fa, fb), f"rel_err {e} > {tol(fa, fb)} for formats {fa},{fb}"
+    if fa == 3 and fb == 3 and ap is not None:
+        l1 = np.abs(o.dequantise(ap, asc, fa, np.float64)) @ np.abs(o.dequantise(bp, bsc, fb, np.float64)).T
+        assert np.max(np.abs(got - ref) / np.maximum(l1, 1e-300)) <= 1e-4
+
+
+@pytest.fixture(scope="module")
+def hk():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import hipkittensp_amd as m
+    from hipkittensp_amd import _lib
+
+    _lib.lib()  # fails loudly if the HIP library is not built: there is no fallback path
+    yield m
+    m.tk_kernel.set_kernel(0)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def gemm(hk, ap, bp, asc, bsc, fa=2, fb=2, out="f32", kernel=0):
+    M, N = ap.shape[0], bp.shape[0]
+    C = torch.full((M, N), float("nan"), dtype=torch.float32 if out == "f32" else torch.bfloat16, device="cuda")
+    prev = hk.tk_kernel.set_kernel(kernel)
+    try:
+        hk.dispatch_micro(dev(ap), dev(bp), dev(asc), dev(bsc), C, fa, fb)
+        torch.cuda.synchronize()
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+    if out == "f32":
+        return C.cpu().numpy()
+    return C.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def operands(M, N, K, fa, fb, seed, kind_a="normal", kind_b="normal"):
+    xa = o.make_source(kind_a, (M, K), np.random.default_rng(seed))
+    xb = o.make_source(kind_b, (N, K), np.random.default_rng(seed + 1000))
+    ap, asc = co.quantise(xa, fa)
+    bp, bsc = co.quantise(xb, fb)
+    return ap, asc, bp, bsc
+
+
+def one_hot_b(K):
+    codes = np.zeros((K, K), np.uint8)
+    codes[np.arange(K), np.arange(K)] = 0b001000  # 1.0 in e2m3
+    return o.pack_fp6(codes), np.full((K, K // 32), 127, np.uint8)
+
+
+# ------------------------------------------------------------------ decode: bit exact
+@pytest.mark.parametrize("kernel,M", [(1, 64), (1, 37), (2, 256), (3, 16), (3, 32)])
+@pytest.mark.parametrize("fmt", [2, 3])
+def test_decode_bit_exact_through_the_mfma(hk, kernel, M, fmt):
+    K = 256
+    rng = np.random.default_rng(fmt * 10 + kernel)
+    codes = rng.integers(0, 64, size=(M, K), dtype=np.uint8)
+    codes[0, :64] = np.arange(64)  # every code of the format at least once
+    ap = o.pack_fp6(codes)
+    asc = rng.integers(110, 140, size=(M, K // 32), dtype=np.uint8)
+    bp, bsc = one_hot_b(K)
+    got = gemm(hk, ap, bp, asc, bsc, fmt, 2, kernel=kernel)
+    exp = o.dequantise(ap, asc, fmt)
+    # bit for bit, except that the code -0 comes back as +0: an accumulator that starts at +0 cannot return -0
+    nz = exp != 0
+    assert np.array_equal(got.view(np.uint32)[nz], exp.view(np.uint32)[nz])
+    assert np.all(got[~nz] == 0)
+
+
+# ------------------------------------------------------------------ BASELINE configs[0]
+@pytest.mark.parametrize("kernel", [0, 1, 2])
+def test_cfg0_256_cubed(hk, kernel):
+    ap, asc = o.make_operand("normal", 256, 256, 2, seed=0)
+    bp, bsc = o.make_operand("normal", 256, 256, 2, seed=1)
+    ref64 = o.gemm_ref(ap, bp, asc, bsc, acc=np.float64)
+    c32 = gemm(hk, ap, bp, asc, bsc, kernel=kernel)
+    assert o.rel_err(c32, ref64) <= TOL_TIGHT <= TOL
+    assert o.rel_err(c32, co.gemm_f32(ap, bp, asc, bsc)) <= TOL           # vs the fp32 CPU path itself
+    cb = gemm(hk, ap, bp, asc, bsc, out="bf16", kernel=kernel)
+    assert np.array_equal(cb, o.f32_to_bf16_bits(c32))                     # epilogue = RNE of the accumulators
+    assert o.rel_err(o.bf16_bits_to_f32(cb), ref64) <= 2.0 ** -8 + TOL
+
+
+# ------------------------------------------------------------------ generic kernel: ragged shapes
+@pytest.mark.parametrize("M,N,K", [(1, 1, 32), (5, 3, 64), (31, 33, 96), (32, 32, 32), (65, 127, 160), (100, 40, 1024), (257, 255, 416)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
+def test_generic_kernel_any_shape(hk, M, N, K, fa, fb):
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + N + K, kind_b="weights_outliers")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=1)
+    check(got, ref, fa, fb, ap, asc, bp, bsc)
+    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=1)
+    assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+
+
+# ------------------------------------------------------------------ tiled kernel
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (256, 512, 384), (512, 256, 1664), (768, 1024, 1024)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
+def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb):
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M * 3 + N + K, kind_a="laplace" if fa == 3 else "normal", kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=2)
+    check(got, ref, fa, fb, ap, asc, bp, bsc)
+    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=2)
+    assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+
+
+def test_tiled_rejects_shapes_it_cannot_take(hk):
+    ap, asc, bp, bsc = operands(64, 64, 64, 2, 2, seed=1)
+    with pytest.raises(RuntimeError, match="bad shape"):
+        gemm(hk, ap, bp, asc, bsc, kernel=2)
+
+
+# ------------------------------------------------------------------ skinny kernel
+@pytest.mark.parametrize("M,N,K", [(16, 64, 128), (1, 32, 256), (7, 100, 2048), (16, 512, 3584), (32, 96, 1152), (13, 33, 128 * 17)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
+def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + 2 * N + K, kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=3)
+    check(got, ref, fa, fb, ap, asc, bp, bsc)
+    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=3)
+    assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+
+
+# ------------------------------------------------------------------ edge cases
+def test_empty_and_degenerate(hk):
+    z = lambda *s: torch.zeros(*s, dtype=torch.uint8, device="cuda")
+    C = torch.ones(0, 8, dtype=torch.bfloat16, device="cuda")
+    hk.dispatch_micro(z(0, 24), z(8, 24), z(0, 1), z(8, 1), C)                 # M == 0: no-op
+    C = torch.full((4, 8), 7.0, dtype=torch.bfloat16, device="cuda")
+    hk.dispatch_micro(z(4, 0), z(8, 0), z(4, 0), z(8, 0), C)                   # K == 0: zeros
+    torch.cuda.synchronize()
+    assert float(C.float().abs().max()) == 0.0
+    # extreme scales: 2^-127 * 2^-127 underflows to 0, 2^127 stays finite against 2^-100
+    ap, asc, bp, bsc = operands(32, 32, 64, 2, 2, seed=5)
+    got = gemm(hk, ap, bp, np.zeros_like(asc), np.zeros_like(bsc), kernel=1)
+    assert np.all(got == 0)
+    got = gemm(hk, ap, bp, np.full_like(asc, 254), np.full_like(bsc, 27), kernel=1)
+    ref = o.gemm_ref(ap, bp, np.full_like(asc, 254), np.full_like(bsc, 27), acc=np.float64)
+    assert np.isfinite(got).all() and o.rel_err(got, ref) <= TOL
+
+
+def test_leading_dimensions_fold_into_rows(hk):
+    ap, asc, bp, bsc = operands(64, 32, 128, 2, 2, seed=9)
+    C = torch.empty(2, 32, 32, dtype=torch.float32, device="cuda")
+    hk.dispatch_micro(dev(ap).view(2, 32, -1), dev(bp), dev(asc).view(2, 32, -1), dev(bsc), C)
+    torch.cuda.synchronize()
+    assert o.rel_err(C.view(64, 32).cpu().numpy(), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64)) <= TOL
+
+
+# ------------------------------------------------------------------ quantiser: bit exact
+@pytest.mark.parametrize("fmt", [2, 3])
+@pytest.mark.parametrize("kind", ["normal", "weights", "weights_outliers", "laplace"])
+def test_gpu_quantiser_bit_exact(hk, fmt, kind):
+    x = o.make_source(kind, (300, 1024), np.random.default_rng(fmt + len(kind)))
+    x[0, :32] = 0.0                       # zero block
+    x[1, :32] = 0.0; x[1, 3] = 1e-42      # denormal-only block
+    x[2, 5] = 3e38                        # huge
+    x[3, :64] = np.float32(2.0) ** np.arange(-30, 34, dtype=np.float32)  # powers of two
+    tab = o.decode_table(fmt)[:32]
+    mids = ((tab[:-1] + tab[1:]) / 2).astype(np.float32)
+    x[4, :31] = mids; x[4, 31] = tab[-1]  # exact rounding ties under scale 2^0... (blockmax = max -> scale 1)
+    x[5, :31] = -mids * 4; x[5, 31] = tab[-1] * 4
+    packed, scales = hk.quantize(dev(x), fmt)
+    torch.cuda.synchronize()
+    ep, es = co.quantise(x, fmt)
+    assert np.array_equal(scales.cpu().numpy(), es)
+    assert np.array_equal(packed.cpu().numpy(), ep)
+    codes, s2 = o.quantise(x, fmt)
+    assert np.array_equal(o.pack_fp6(codes), ep) and np.array_equal(s2, es)
+
+
+# ------------------------------------------------------------------ full-size configurations
+def _sampled_check(hk, ap, asc, bp, bsc, fa, fb, kernel, rng, ns=48):
+    M, N = ap.shape[0], bp.shape[0]
+    C = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
+    prev = hk.tk_kernel.set_kernel(kernel)
+    try:
+        hk.dispatch_micro(dA, dB, dAs, dBs, C, fa, fb)
+        rows = np.sort(rng.choice(M, size=min(ns, M), replace=False))
+        cols = np.sort(rng.choice(N, size=min(ns, N), replace=False))
+        ref = o.gemm_ref(ap[rows], bp[cols], asc[rows], bsc[cols], fa, fb, acc=np.float64)
+        got = C[torch.from_numpy(rows).cuda()][:, torch.from_numpy(cols).cuda()].cpu().numpy()
+        check(got, ref, fa, fb)
+        # exact linearity in the block scales: +1 on every A scale byte doubles every output bit for bit
+        C2 = torch.empty_like(C)
+        hk.dispatch_micro(dA, dB, dAs + 1, dBs, C2, fa, fb)
+        assert torch.equal(C2, 2 * C)
+        # bf16 output is the RNE rounding of the accumulators
+        Cb = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        hk.dispatch_micro(dA, dB, dAs, dBs, Cb, fa, fb)
+        assert torch.equal(Cb, C.to(torch.bfloat16))
+        torch.cuda.synchronize()
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+    return C
+
+
+def test_cfg1_square_8192(hk):
+    M = N = K = 8192
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=1)
+    C = _sampled_check(hk, ap, asc, bp, bsc, 2, 2, 0, np.random.default_rng(1))
+    # operand swap = transpose (the two operands take different paths through the kernel)
+    Ct = torch.empty(N, M, dtype=torch.float32, device="cuda")
+    hk.dispatch_micro(dev(bp), dev(ap), dev(bsc), dev(asc), Ct, 2, 2)
+    torch.cuda.synchronize()
+    d = (Ct.t() - C).abs().max().item()
+    assert d <= 1e-4 * C.abs().max().item()
+    # tiled kernel agrees with the independent generic kernel on a 1024-row band
+    prev = hk.tk_kernel.set_kernel(1)
+    Cg = torch.empty(1024, N, dtype=torch.float32, device="cuda")
+    hk.dispatch_micro(dev(ap[:1024]), dev(bp), dev(asc[:1024]), dev(bsc), Cg, 2, 2)
+    torch.cuda.synchronize()
+    hk.tk_kernel.set_kernel(prev)
+    assert (Cg - C[:1024]).abs().max().item() <= 1e-4 * C.abs().max().item()
+
+
+def test_cfg2_prefill_outliers(hk):
+    M, N, K = 4096, 28672, 8192
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=2, kind_a="normal", kind_b="weights_outliers")
+    assert int(bsc.max()) - int(bsc.min()) >= 3      # the outliers widen the E8M0 range
+    _sampled_check(hk, ap, asc, bp, bsc, 2, 2, 0, np.random.default_rng(2))
+
+
+def test_cfg3_decode_skinny(hk):
+    M, N, K = 16, 8192, 28672
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=3, kind_a="normal", kind_b="weights")
+    _sampled_check(hk, ap, asc, bp, bsc, 2, 2, 0, np.random.default_rng(3), ns=64)
+    ref = o.gemm_ref(ap, bp[:256], asc, bsc[:256], acc=np.float64)
+    for kernel in (1, 3):  # generic and skinny kernels against the full first 256 columns
+        got = gemm(hk, ap, bp[:256], asc, bsc[:256], kernel=kernel)
+        check(got, ref, 2, 2)
+
+
+def test_cfg4_mixed_formats(hk):
+    M, N, K = 8192, 8192, 16384
+    ap, asc, bp, bsc = operands(M, N, K, 3, 2, seed=4, kind_a="laplace", kind_b="weights")
+    _sampled_check(hk, ap, asc, bp, bsc, 3, 2, 0, np.random.default_rng(4))
