@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the MXFP6 GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" = one pass of the operator over one batch of synthetic inputs that already sit in HBM:
+C[8192,8192] (bf16) = A[8192,8192] . B[8192,8192]^T with MXFP6 e2m3 operands (BASELINE.json
+configs[1]: N(0,1) sources, per-32 E8M0 scales).  Inputs are produced on the GPU (torch.randn with a
+fixed seed -> the library's own quantise+pack kernel) and the timed loop cycles through several
+independent input sets, the counterpart of the reference protocol's fresh inputs per iteration
+(kernels/gemm/bf16fp32/utils.py:36-54: warm-up launches, then timed launches bracketed by device
+events, TFLOPS = 2*M*N*K / t).
+
+Prints ONE JSON line.  `value` is TFLOP/s of the whole job (wall clock between two device
+synchronisations / steps).  `roofline` prices the tiled GEMM kernel against the dense MXFP6 MFMA peak
+using the mean per-launch duration measured with device events on the launch stream; `decode` does
+the same for the M=16 skinny kernel (BASELINE.json configs[3]) against the HBM peak.  `cpu_baseline`
+times the CPU oracle (oracle/mxfp6_oracle.c, an OpenMP port of dequantise-and-matmul) on a bounded
+sample of the same bytes; it is a reported baseline, not a target.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 10066.0  # MI355X dense MXFP6: 256 CU x 4 SIMD x 4096 FLOP/clk x 2.4 GHz
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+PUBLISHED_FP6_8192 = 2861.52  # reference's own FP6 GEMM at 8192^3 on MI355X
+# HBM bytes per launch of the 8192^3 tiled kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a
+# copy kernel of known size (profiles/); None until that measurement exists.
+TILED_TRAFFIC_BYTES = None
+
+
+def algorithmic_bytes(M, N, K):
+    return 0.75 * K * (M + N) + (K // 32) * (M + N) + 2 * M * N
+
+
+def make_inputs(hk, torch, M, N, K, fmt_a, fmt_b, seed, sets, std_b=1.0):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    out = []
+    for _ in range(sets):
+        xa = torch.randn(M, K, device="cuda", dtype=torch.float32, generator=g)
+        ap, asc = hk.quantize(xa, fmt_a)
+        del xa
+        xb = torch.randn(N, K, device="cuda", dtype=torch.float32, generator=g)
+        if std_b != 1.0:
+            xb *= std_b
+        bp, bsc = hk.quantize(xb, fmt_b)
+        del xb
+        out.append((ap, bp, asc, bsc))
+    torch.cuda.synchronize()
+    return out
+
+
+def timed_loop(hk, torch, inputs, C, steps, warmup):
+    """W untimed + K timed launches; returns (wall seconds for K steps, mean per-launch event ms)."""
+    n = len(inputs)
+    for i in range(warmup):
+        ap, bp, asc, bsc = inputs[i % n]
+        hk.dispatch_micro(ap, bp, asc, bsc, C)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ap, bp, asc, bsc = inputs[i % n]
+        ev[i][0].record()
+        hk.dispatch_micro(ap, bp, asc, bsc, C)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = [a.elapsed_time(b) for a, b in ev]
+    return wall, sum(per) / len(per), min(per)
+
+
+def cpu_baseline(inputs, M_sample):
+    """The C oracle (OpenMP) on the first M_sample rows of A against all of B: same bytes as the GPU run."""
+    from oracle import c_oracle as co
+
+    ap, bp, asc, bsc = inputs
+    ap_h = ap[:M_sample].cpu().numpy()
+    asc_h = asc[:M_sample].cpu().numpy()
+    bp_h, bsc_h = bp.cpu().numpy(), bsc.cpu().numpy()
+    N, K = bp_h.shape[0], bp_h.shape[1] // 3 * 4
+    t0 = time.perf_counter()
+    co.gemm_f32(ap_h, bp_h, asc_h, bsc_h, 2, 2)
+    dt = time.perf_counter() - t0
+    return {
+        "value": 2.0 * M_sample * N * K / dt / 1e12,
+        "unit": "TFLOPS",
+        "cores": co.num_threads(),
+        "kind": "port",
+        "sample": f"first {M_sample} of 8192 rows of A against all 8192 rows of B, K=8192 (dequantise + fp32 matmul, {dt:.2f} s)",
+    }
+
+
+def main():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=100)
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--cpu-rows", type=int, default=2048)
+    args = p.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures ONE GPU (a single-GPU operator; sharding is by N or M with no exchange). Run with --gpus 1.")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import hipkittensp_amd as hk
+    from hipkittensp_amd import _lib
+
+    _lib.lib()  # fail loudly if the HIP library is missing
+
+    # ---- headline: configs[1], 8192^3 e2m3 x e2m3 -> bf16
+    M = N = K = 8192
+    inputs = make_inputs(hk, torch, M, N, K, 2, 2, seed=1, sets=3)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    wall, ev_ms, ev_min = timed_loop(hk, torch, inputs, C, args.steps, args.warmup)
+    flops = 2.0 * M * N * K
+    ms_per_step = wall / args.steps * 1e3
+    value = flops / (wall / args.steps) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": "gemm_tiled_kernel (256x256x128 tiles, v_mfma_scale_f32_32x32x64_f8f6f4)",
+        "bound": "mfma",
+        "achieved": achieved,
+        "peak": MFMA_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": achieved / MFMA_PEAK_TFLOPS,
+        "traffic": TILED_TRAFFIC_BYTES,
+        "launch_ms_mean": ev_ms,
+        "launch_ms_min": ev_min,
+        "algorithmic_flops_per_launch": flops,
+        "algorithmic_bytes_per_launch": algorithmic_bytes(M, N, K),
+        "hbm_bound_ms": algorithmic_bytes(M, N, K) / (HBM_PEAK_GBS * 1e9) * 1e3,
+    }
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(inputs[0], args.cpu_rows)
+    del inputs, C
+    torch.cuda.empty_cache()
+
+    # ---- decode shape: configs[3], M=16, N=8192, K=28672, weights N(0, 0.02); five weight sets
+    # (5 x 184 MB > the 256 MB last-level cache) so that the rate is HBM's, not the cache's
+    dM, dN, dK = 16, 8192, 28672
+    dinputs = make_inputs(hk, torch, dM, dN, dK, 2, 2, seed=3, sets=5, std_b=0.02)
+    dC = torch.empty(dM, dN, dtype=torch.bfloat16, device="cuda")
+    dwall, dev_ms, dev_min = timed_loop(hk, torch, dinputs, dC, args.steps, args.warmup)
+    dbytes = algorithmic_bytes(dM, dN, dK)
+    d_achieved = dbytes / (dev_ms * 1e-3) / 1e9
+    decode = {
+        "metric": "MXFP6 decode GEMM achieved GB/s @M=16,N=8192,K=28672",
+        "value": dbytes / (dwall / args.steps) / 1e9,
+        "unit": "GB/s",
+        "ms_per_step": dwall / args.steps * 1e3,
+        "roofline": {
+            "kernel": "gemm_skinny_kernel",
+            "bound": "hbm",
+            "achieved": d_achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": d_achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "launch_ms_mean": dev_ms,
+            "launch_ms_min": dev_min,
+            "algorithmic_bytes_per_launch": dbytes,
+        },
+    }
+
+    line = {
+        "metric": "MXFP6 GEMM TFLOPS @8192^3 (% of MFMA peak); GB/s @M=16 decode",
+        "value": value,
+        "unit": "TFLOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": value / PUBLISHED_FP6_8192,
+        "dtype": "mxfp6 e2m3 x e2m3 (E8M0 block scales), f32 accumulate, bf16 out",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: square MXFP6 e2m3 GEMM C=A.B^T, M=N=K=8192, N(0,1) sources quantised per 32-block, bf16 output",
+            "M": M, "N": N, "K": K, "fmt_a": "e2m3", "fmt_b": "e2m3", "input_sets": 3,
+        },
+        "pct_of_mfma_peak": 100.0 * value / MFMA_PEAK_TFLOPS,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "decode": decode,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
