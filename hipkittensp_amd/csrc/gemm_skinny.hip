@@ -4,8 +4,8 @@
 // into the MFMA source registers (16-byte loads of the packed rows; no unpacking, no LDS staging:
 // with M <= 32 a B element meets the tensor core once).  A (the few activation rows) is re-read
 // from L2 by every wave.  One workgroup owns 32 consecutive rows of B (32 output columns) and
-// splits K over its 16 waves; the 16 partial 32x32 tiles are summed through LDS, so no global
-// scratch and no atomics are needed.  Each wave keeps three K-tiles (3 x 48 bytes per lane per
+// splits K over its 8 waves; the 8 partial 32x32 tiles are summed through LDS, so no global
+// scratch and no atomics are needed.  Each wave keeps four K-tiles (4 x 48 bytes per lane per
 // operand) in flight, about 100 KB per CU, which is what HBM latency x bandwidth asks for.
 //
 // The reference has no kernel for this shape (its GEMMs need M, N multiples of the 256 tile,
@@ -16,12 +16,41 @@
 
 namespace mxfp6 {
 
-constexpr int kSkinnyWaves = 16;
-constexpr int kPF = 3;  // K-tiles in flight per wave
+constexpr int kSkinnyWaves = 8;
+constexpr int kPF = 4;  // K-tiles in flight per wave
 
 struct Frag {
   v4i b[3], a[3];  // the lane's 48 bytes (two 32-element K-blocks) of its B row and A row
+  int sb, sa;      // the two E8M0 bytes of those K-blocks, B and A
 };
+
+// Loads are issued from inline assembly and waited for by hand: the compiler's own counter
+// placement drains the whole queue once per loop iteration, which leaves HBM idle while the
+// MFMAs run.  The wait takes the stage's registers as read-write operands so that no use can be
+// scheduled above it.
+__device__ __forceinline__ v4i load128_stream(const __amdgpu_buffer_rsrc_t& r, uint32_t voff, int soff) {
+  v4i d;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
+  return d;
+}
+__device__ __forceinline__ v4i load128(const __amdgpu_buffer_rsrc_t& r, uint32_t voff, int soff) {
+  v4i d;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
+  return d;
+}
+__device__ __forceinline__ int load16(const __amdgpu_buffer_rsrc_t& r, uint32_t voff, int soff) {
+  int d;
+  asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
+  return d;
+}
+constexpr int kLoadsPerStage = 8;
+template <int N>
+__device__ __forceinline__ void wait_stage(Frag& f) {
+  asm volatile("s_waitcnt vmcnt(%8)"
+               : "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.sb), "+v"(f.sa)
+               : "n"(N)
+               : "memory");
+}
 
 template <int FA, int FB, typename Out>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A,
@@ -51,15 +80,16 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const ui
   const uint32_t vbs = n < N ? (uint32_t)n * sbytes + 2 * h : kOob;
   const uint32_t vas = r32 < M ? (uint32_t)r32 * sbytes + 2 * h : kOob;
 
-  auto load = [&](Frag& f, int& sb, int& sa, int t) {
+  auto load = [&](Frag& f, int t) {
+    const int so = __builtin_amdgcn_readfirstlane(t * 96), ss = __builtin_amdgcn_readfirstlane(t * 4);
+    // B is streamed once: non-temporal; A is shared by every wave: default policy
 #pragma unroll
     for (int c = 0; c < 3; c++) {
-      // B is streamed once: non-temporal; A is shared by every wave: default policy
-      f.b[c] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rB, vb, t * 96 + 16 * c, 2));
-      f.a[c] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rA, va, t * 96 + 16 * c, 0));
+      f.b[c] = load128_stream(rB, vb, so + 16 * c);
+      f.a[c] = load128(rA, va, so + 16 * c);
     }
-    sb = __builtin_amdgcn_raw_buffer_load_b16(rBs, vbs, t * 4, 0);
-    sa = __builtin_amdgcn_raw_buffer_load_b16(rAs, vas, t * 4, 0);
+    f.sb = load16(rBs, vbs, ss);
+    f.sa = load16(rAs, vas, ss);
   };
 
   v16f acc;
@@ -67,38 +97,59 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const ui
   for (int e = 0; e < 16; e++) acc[e] = 0.f;
 
   Frag f[kPF];
-  int sb[kPF], sa[kPF];
+  auto use = [&](Frag& g) {
+    const v8i b0 = __builtin_shufflevector(g.b[0], g.b[1], 0, 1, 2, 3, 4, 5, -1, -1);
+    const v8i b1 = __builtin_shufflevector(g.b[1], g.b[2], 2, 3, 4, 5, 6, 7, -1, -1);
+    const v8i a0 = __builtin_shufflevector(g.a[0], g.a[1], 0, 1, 2, 3, 4, 5, -1, -1);
+    const v8i a1 = __builtin_shufflevector(g.a[1], g.a[2], 2, 3, 4, 5, 6, 7, -1, -1);
+    acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, g.sb, g.sa);
+    acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, g.sb, g.sa);
+  };
+  const int nt = t1 - t0;
+  int t = 0;
+  if (nt >= 2 * kPF) {
+    // prologue, then a steady state in which every stage is consumed and at once refilled with
+    // the tile kPF ahead: kPF-1 stages (3 x 8 loads) are always in flight
 #pragma unroll
-  for (int s = 0; s < kPF; s++)
-    if (t0 + s < t1) load(f[s], sb[s], sa[s], t0 + s);
-
-  for (int t = t0; t < t1; t += kPF) {
+    for (int s = 0; s < kPF; s++) load(f[s], t0 + s);
+    for (; t + 2 * kPF <= nt; t += kPF) {
 #pragma unroll
-    for (int s = 0; s < kPF; s++) {
-      if (t + s < t1) {
-        const v8i b0 = __builtin_shufflevector(f[s].b[0], f[s].b[1], 0, 1, 2, 3, 4, 5, -1, -1);
-        const v8i b1 = __builtin_shufflevector(f[s].b[1], f[s].b[2], 2, 3, 4, 5, 6, 7, -1, -1);
-        const v8i a0 = __builtin_shufflevector(f[s].a[0], f[s].a[1], 0, 1, 2, 3, 4, 5, -1, -1);
-        const v8i a1 = __builtin_shufflevector(f[s].a[1], f[s].a[2], 2, 3, 4, 5, 6, 7, -1, -1);
-        const int csb = sb[s], csa = sa[s];
-        if (t + s + kPF < t1) load(f[s], sb[s], sa[s], t + s + kPF);
-        acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, csb, csa);
-        acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, csb, csa);
+      for (int s = 0; s < kPF; s++) {
+        wait_stage<(kPF - 1) * kLoadsPerStage>(f[s]);
+        use(f[s]);
+        load(f[s], t0 + t + kPF + s);
       }
     }
+    // drain the kPF stages still in flight
+    wait_stage<3 * kLoadsPerStage>(f[0]); use(f[0]);
+    wait_stage<2 * kLoadsPerStage>(f[1]); use(f[1]);
+    wait_stage<1 * kLoadsPerStage>(f[2]); use(f[2]);
+    wait_stage<0>(f[3]); use(f[3]);
+    static_assert(kPF == 4, "drain sequence is written for four stages");
+    t += kPF;
+  }
+  // remainder (and short K): one tile at a time
+  for (; t < nt; t++) {
+    load(f[0], t0 + t);
+    wait_stage<0>(f[0]);
+    use(f[0]);
   }
 
-  // sum the 16 K-slices: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4]
+  // sum the K-slices: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4]
 #pragma unroll
   for (int e = 0; e < 16; e++) part[wave][e][lane] = acc[e];
   __syncthreads();
-  const int e = tid >> 6;  // 1024 threads = 16 registers x 64 lanes
-  float s = 0.f;
+  // 512 threads, 1024 outputs: thread handles registers e and e + 8 of its lane
 #pragma unroll
-  for (int w = 0; w < kSkinnyWaves; w++) s += part[w][e][lane];
-  const int m = lane & 31;
-  const long nn = (long)blockIdx.x * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-  if (m < M && nn < N) store1(C + (long)m * N + nn, s);
+  for (int half = 0; half < 2; half++) {
+    const int e = (tid >> 6) + 8 * half;
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kSkinnyWaves; w++) s += part[w][e][lane];
+    const int m = lane & 31;
+    const long nn = (long)blockIdx.x * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+    if (m < M && nn < N) store1(C + (long)m * N + nn, s);
+  }
 }
 
 bool gemm_skinny_supports(const GemmArgs& g) {
