@@ -1,164 +1,212 @@
-// Skinny-M (decode-shaped) MXFP6 GEMM for gfx950: M <= 32, HBM-bound.
+// Skinny-M (decode-shaped) MXFP6 GEMM for gfx950: M <= 32, bound by HBM.
 //
-// Every byte of B (weights) and of its scales is read exactly once, straight from global memory
-// into the MFMA source registers (16-byte loads of the packed rows; no unpacking, no LDS staging:
-// with M <= 32 a B element meets the tensor core once).  A (the few activation rows) is re-read
-// from L2 by every wave.  One workgroup owns 32 consecutive rows of B (32 output columns) and
-// splits K over its 8 waves; the 8 partial 32x32 tiles are summed through LDS, so no global
-// scratch and no atomics are needed.  Each wave keeps four K-tiles (4 x 48 bytes per lane per
-// operand) in flight, about 100 KB per CU, which is what HBM latency x bandwidth asks for.
+// Every byte of B (weights) is read from HBM once.  One workgroup owns 32 consecutive rows of B
+// (32 output columns) and splits K over its waves in chunks of four K-tiles (4 x 128 elements =
+// 384 bytes per row = three whole 128-byte lines), dealt round-robin: wave w takes chunks w, w+NW, ...
+// so the workgroup streams one contiguous K range of its 32 rows and no cache line is shared
+// between chunks.  Each wave owns a private 4-stage LDS ring (one stage per K-tile of a chunk):
+//   global --buffer_load_dwordx4 ... lds--> LDS --ds_read_b128--> MFMA sources
+// with the same lane->address map as the tiled kernel (consecutive lanes fetch consecutive 16-byte
+// pieces of a row; row-major 96-byte LDS rows with a pair swap that makes the reads conflict-free).
+// Staging through LDS is what lets the loads be coalesced: the MFMA wants lane = row, the memory
+// system wants lane = consecutive bytes.  A's rows (M <= 32) are staged the same way from L2.  The
+// E8M0 bytes of a chunk are 16 bytes per row: one 16-byte load per lane per chunk, kept in VGPRs.
+// All loads are issued from inline assembly and waited for with hand-counted vmcnt, four K-tiles
+// ahead.  The partial 32x32 tiles of the waves are summed through LDS: no scratch, no atomics.
 //
 // The reference has no kernel for this shape (its GEMMs need M, N multiples of the 256 tile,
-// analysis/bf16_gemm/mi325x/kernel_8192.cpp:24-32); the MFMA operand conventions are those of the
-// tiled kernel.  Algorithmic bytes per launch: 0.75*K*(M+N) + (K/32)*(M+N) + 2*M*N.
+// analysis/bf16_gemm/mi325x/kernel_8192.cpp:24-32).  Algorithmic bytes per launch:
+// 0.75*K*(M+N) + (K/32)*(M+N) + 2*M*N.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace mxfp6 {
 
-constexpr int kSkinnyWaves = 8;
-constexpr int kPF = 4;  // K-tiles in flight per wave
+namespace {
 
-struct Frag {
-  v4i b[3], a[3];  // the lane's 48 bytes (two 32-element K-blocks) of its B row and A row
-  int sb, sa;      // the two E8M0 bytes of those K-blocks, B and A
-};
+constexpr int kStagesSk = 4;  // = K-tiles per chunk
 
-// Loads are issued from inline assembly and waited for by hand: the compiler's own counter
-// placement drains the whole queue once per loop iteration, which leaves HBM idle while the
-// MFMAs run.  The wait takes the stage's registers as read-write operands so that no use can be
-// scheduled above it.
-__device__ __forceinline__ v4i load128_stream(const __amdgpu_buffer_rsrc_t& r, uint32_t voff, int soff) {
-  v4i d;
-  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
-  return d;
+__device__ __forceinline__ void dma16_sk(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
 }
-__device__ __forceinline__ v4i load128(const __amdgpu_buffer_rsrc_t& r, uint32_t voff, int soff) {
+__device__ __forceinline__ v4i load128_sk(const __amdgpu_buffer_rsrc_t& r, int voff, int soff) {
   v4i d;
   asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
   return d;
 }
-__device__ __forceinline__ int load16(const __amdgpu_buffer_rsrc_t& r, uint32_t voff, int soff) {
-  int d;
-  asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
-  return d;
-}
-constexpr int kLoadsPerStage = 8;
+// wait until at most N of this wave's loads are outstanding; the scale registers ride along as
+// read-write operands so that no use of them can be scheduled above the wait
 template <int N>
-__device__ __forceinline__ void wait_stage(Frag& f) {
-  asm volatile("s_waitcnt vmcnt(%8)"
-               : "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.sb), "+v"(f.sa)
-               : "n"(N)
-               : "memory");
+__device__ __forceinline__ void wait_loads(v4i& s0, v4i& s1) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(s0), "+v"(s1) : "n"(N) : "memory");
 }
 
-template <int FA, int FB, typename Out>
-__global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A,
-                                                                        const uint8_t* __restrict__ B,
-                                                                        const uint8_t* __restrict__ As,
-                                                                        const uint8_t* __restrict__ Bs,
-                                                                        typename Out::type* __restrict__ C, int M, int N, int K) {
-  __shared__ float part[kSkinnyWaves][16][64];
+}  // namespace
+
+// AR = rows of A staged per K-tile (16 or 32); NW = waves per workgroup
+template <int FA, int FB, typename Out, int AR, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                              const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
+                                                              typename Out::type* __restrict__ C, int M, int N, int K) {
+  constexpr int kBTile = 32 * 96, kATile = AR * 96, kStage = kBTile + kATile, kRing = kStagesSk * kStage;
+  constexpr int kADma = (kATile + 1023) / 1024;  // direct loads per A tile (the last one half full when AR = 16)
+  constexpr int kDmaPerTile = 3 + kADma;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kRing];
+  static_assert(NW * kRing <= 163840 && NW * kRing >= NW * 16 * 64 * 4, "LDS budget (ring doubles as the reduction buffer)");
+
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, r32 = lane & 31;
   const int nkt = K / 128, sbytes = K / 32, rowbytes = K / 4 * 3;
-  const long n = (long)blockIdx.x * 32 + r32;
-  // K-tiles [t0, t1) of this wave
-  const int per = (nkt + kSkinnyWaves - 1) / kSkinnyWaves;
-  const int t0 = min(wave * per, nkt), t1 = min(t0 + per, nkt);
+  const int n0 = blockIdx.x * 32;
+  const int nrows = min(32, N - n0);
 
-  // buffer resources bound the operands: a lane whose row does not exist (n >= N, m >= M) points
-  // past the end and reads zeros -- no divergent control flow around the loads
-  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B, (uint32_t)N * (uint32_t)rowbytes);
-  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, (uint32_t)M * (uint32_t)rowbytes);
-  const __amdgpu_buffer_rsrc_t rBs = make_rsrc(Bs, (uint32_t)N * (uint32_t)sbytes);
-  const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * (uint32_t)sbytes);
-  const uint32_t kOob = 0xFFFFFF00u;
-  const uint32_t vb = n < N ? (uint32_t)n * rowbytes + 48 * h : kOob;
-  const uint32_t va = r32 < M ? (uint32_t)r32 * rowbytes + 48 * h : kOob;
-  const uint32_t vbs = n < N ? (uint32_t)n * sbytes + 2 * h : kOob;
-  const uint32_t vas = r32 < M ? (uint32_t)r32 * sbytes + 2 * h : kOob;
+  // rows that do not exist (n >= N, m >= M) lie past the end of the resource and read as zeros
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, (uint32_t)M * rowbytes);
+  const __amdgpu_buffer_rsrc_t rBs = make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
+  const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * sbytes);
 
-  auto load = [&](Frag& f, int t) {
-    const int so = __builtin_amdgcn_readfirstlane(t * 96), ss = __builtin_amdgcn_readfirstlane(t * 4);
-    // B is streamed once: non-temporal; A is shared by every wave: default policy
+  // direct-load address map: LDS slot o (16 bytes) of a tile holds chunk (o%6) ^ ((row>>3)&1) of row o/6
+  int voff[3];
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
-      f.b[c] = load128_stream(rB, vb, so + 16 * c);
-      f.a[c] = load128(rA, va, so + 16 * c);
+  for (int i = 0; i < 3; i++) {
+    const int o = i * 64 + lane, r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
+    voff[i] = r * rowbytes + c * 16;
+  }
+  const int voff_bs = r32 * sbytes, voff_as = (AR == 16 ? (r32 & 15) : r32) * sbytes;
+
+  const uint32_t ring = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kRing;
+  const uint8_t* ringp = smem + wave * kRing;
+  const int sw = (r32 >> 3) & 1;
+  int b_rd[3], a_rd[3];
+#pragma unroll
+  for (int c = 0; c < 3; c++) {
+    b_rd[c] = r32 * 96 + ((3 * h + c) ^ sw) * 16;
+    const int ra = AR == 16 ? (r32 & 15) : r32;  // AR = 16: lanes 16-31 mirror rows 0-15 (their outputs are never stored)
+    a_rd[c] = kBTile + ra * 96 + ((3 * h + c) ^ ((ra >> 3) & 1)) * 16;
+  }
+
+  // chunks of this wave: wave, wave + NW, ...
+  const int nchunks = (nkt + 3) / 4;
+  const int mine = wave < nchunks ? (nchunks - wave + NW - 1) / NW : 0;
+
+  v4i sc_b_next, sc_a_next, sc_b, sc_a;
+  sc_b_next = sc_a_next = sc_b = sc_a = v4i{0, 0, 0, 0};
+
+  auto issue_scales = [&](int chunk) {  // 16 scale bytes per row: the chunk's four K-tiles
+    const int so = __builtin_amdgcn_readfirstlane(chunk * 16);
+    sc_b_next = load128_sk(rBs, voff_bs, so);
+    sc_a_next = load128_sk(rAs, voff_as, so);
+  };
+  auto issue_tile = [&](int chunk, int u) {  // K-tile u of a chunk into stage u
+    const int t = min(chunk * 4 + u, nkt - 1);  // past-the-end tiles re-read the last one and are never multiplied
+    const int so = __builtin_amdgcn_readfirstlane(t * 96);
+    const uint32_t dst = ring + u * kStage;
+#pragma unroll
+    for (int i = 0; i < 3; i++) dma16_sk(rB, dst + i * 1024, voff[i], so);
+    dma16_sk(rA, dst + kBTile, voff[0], so);
+    if constexpr (kADma == 2) {
+      if (lane < 32) dma16_sk(rA, dst + kBTile + 1024, voff[1], so);
+    } else {
+      dma16_sk(rA, dst + kBTile + 1024, voff[1], so);
+      dma16_sk(rA, dst + kBTile + 2048, voff[2], so);
     }
-    f.sb = load16(rBs, vbs, ss);
-    f.sa = load16(rAs, vas, ss);
   };
 
   v16f acc;
 #pragma unroll
   for (int e = 0; e < 16; e++) acc[e] = 0.f;
 
-  Frag f[kPF];
-  auto use = [&](Frag& g) {
-    const v8i b0 = __builtin_shufflevector(g.b[0], g.b[1], 0, 1, 2, 3, 4, 5, -1, -1);
-    const v8i b1 = __builtin_shufflevector(g.b[1], g.b[2], 2, 3, 4, 5, 6, 7, -1, -1);
-    const v8i a0 = __builtin_shufflevector(g.a[0], g.a[1], 0, 1, 2, 3, 4, 5, -1, -1);
-    const v8i a1 = __builtin_shufflevector(g.a[1], g.a[2], 2, 3, 4, 5, 6, 7, -1, -1);
-    acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, g.sb, g.sa);
-    acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, g.sb, g.sa);
+  auto consume = [&](int chunk, int u) {
+    if (chunk * 4 + u >= nkt) return;
+    const uint8_t* st = ringp + u * kStage;
+    v4i fb[3], fa[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      fb[c] = *reinterpret_cast<const v4i*>(st + b_rd[c]);
+      fa[c] = *reinterpret_cast<const v4i*>(st + a_rd[c]);
+    }
+    const int sb = (uint32_t)sc_b[u] >> (16 * h), sa = (uint32_t)sc_a[u] >> (16 * h);
+    const v8i b0 = __builtin_shufflevector(fb[0], fb[1], 0, 1, 2, 3, 4, 5, -1, -1);
+    const v8i b1 = __builtin_shufflevector(fb[1], fb[2], 2, 3, 4, 5, 6, 7, -1, -1);
+    const v8i a0 = __builtin_shufflevector(fa[0], fa[1], 0, 1, 2, 3, 4, 5, -1, -1);
+    const v8i a1 = __builtin_shufflevector(fa[1], fa[2], 2, 3, 4, 5, 6, 7, -1, -1);
+    acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, sb, sa);
+    acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, sb, sa);
+    // the stage is about to be refilled: its reads must have left LDS
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   };
-  const int nt = t1 - t0;
-  int t = 0;
-  if (nt >= 2 * kPF) {
-    // prologue, then a steady state in which every stage is consumed and at once refilled with
-    // the tile kPF ahead: kPF-1 stages (3 x 8 loads) are always in flight
+
+  if (mine > 0) {
+    issue_scales(wave);
 #pragma unroll
-    for (int s = 0; s < kPF; s++) load(f[s], t0 + s);
-    for (; t + 2 * kPF <= nt; t += kPF) {
+    for (int u = 0; u < 4; u++) issue_tile(wave, u);
+    int j = 0;
+    // steady state: waiting for tile (j,u) leaves the direct loads of the next three tiles in flight,
+    // plus the two scale loads of chunk j+1 once they have been issued (u >= 1)
+    for (; j + 1 < mine; j++) {
+      const int chunk = wave + j * NW, next = chunk + NW;
+      wait_loads<3 * kDmaPerTile>(sc_b_next, sc_a_next);
+      sc_b = sc_b_next;
+      sc_a = sc_a_next;
+      consume(chunk, 0);
+      issue_scales(next);
+      issue_tile(next, 0);
 #pragma unroll
-      for (int s = 0; s < kPF; s++) {
-        wait_stage<(kPF - 1) * kLoadsPerStage>(f[s]);
-        use(f[s]);
-        load(f[s], t0 + t + kPF + s);
+      for (int u = 1; u < 4; u++) {
+        wait_loads<3 * kDmaPerTile + 2>(sc_b_next, sc_a_next);
+        consume(chunk, u);
+        issue_tile(next, u);
       }
     }
-    // drain the kPF stages still in flight
-    wait_stage<3 * kLoadsPerStage>(f[0]); use(f[0]);
-    wait_stage<2 * kLoadsPerStage>(f[1]); use(f[1]);
-    wait_stage<1 * kLoadsPerStage>(f[2]); use(f[2]);
-    wait_stage<0>(f[3]); use(f[3]);
-    static_assert(kPF == 4, "drain sequence is written for four stages");
-    t += kPF;
-  }
-  // remainder (and short K): one tile at a time
-  for (; t < nt; t++) {
-    load(f[0], t0 + t);
-    wait_stage<0>(f[0]);
-    use(f[0]);
+    // last chunk: nothing more to issue
+    const int chunk = wave + j * NW;
+    wait_loads<3 * kDmaPerTile>(sc_b_next, sc_a_next);
+    sc_b = sc_b_next;
+    sc_a = sc_a_next;
+    consume(chunk, 0);
+    wait_loads<2 * kDmaPerTile>(sc_b_next, sc_a_next);
+    consume(chunk, 1);
+    wait_loads<1 * kDmaPerTile>(sc_b_next, sc_a_next);
+    consume(chunk, 2);
+    wait_loads<0>(sc_b_next, sc_a_next);
+    consume(chunk, 3);
   }
 
-  // sum the K-slices: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4]
-#pragma unroll
-  for (int e = 0; e < 16; e++) part[wave][e][lane] = acc[e];
+  // sum the K-slices: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4].
+  // The ring doubles as the reduction buffer once every wave has drained its loads.
   __syncthreads();
-  // 512 threads, 1024 outputs: thread handles registers e and e + 8 of its lane
+  float* part = reinterpret_cast<float*>(smem);
 #pragma unroll
-  for (int half = 0; half < 2; half++) {
-    const int e = (tid >> 6) + 8 * half;
+  for (int e = 0; e < 16; e++) part[(wave * 16 + e) * 64 + lane] = acc[e];
+  __syncthreads();
+  for (int idx = tid; idx < 1024; idx += NW * 64) {
+    const int e = idx >> 6, l = idx & 63;
     float s = 0.f;
 #pragma unroll
-    for (int w = 0; w < kSkinnyWaves; w++) s += part[w][e][lane];
-    const int m = lane & 31;
-    const long nn = (long)blockIdx.x * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+    for (int w = 0; w < NW; w++) s += part[(w * 16 + e) * 64 + l];
+    const int m = l & 31;
+    const long nn = (long)n0 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
     if (m < M && nn < N) store1(C + (long)m * N + nn, s);
   }
 }
 
 bool gemm_skinny_supports(const GemmArgs& g) {
-  return g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 128 && g.K % 128 == 0 && (long)g.N * (g.K / 4 * 3) < 0xFFFFFF00L;
+  // K % 512: chunks of four K-tiles are whole (three 128-byte lines per row, 16 scale bytes per row)
+  return g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  gemm_skinny_kernel<FA, FB, Out><<<(g.N + 31) / 32, kSkinnyWaves * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K);
+  const unsigned grid = (g.N + 31) / 32;
+  if (g.M <= 16)
+    gemm_skinny_kernel<FA, FB, Out, 16, 8><<<grid, 8 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K);
+  else
+    gemm_skinny_kernel<FA, FB, Out, 32, 6><<<grid, 6 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K);
   return hipGetLastError();
 }
 

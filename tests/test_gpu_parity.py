@@ -83,10 +83,10 @@ def one_hot_b(K):
 
 
 # ------------------------------------------------------------------ decode: bit exact
-@pytest.mark.parametrize("kernel,M", [(1, 64), (1, 37), (2, 256), (3, 16), (3, 32)])
+@pytest.mark.parametrize("kernel,M", [(1, 64), (1, 37), (2, 256), (3, 16), (3, 32), (3, 5)])
 @pytest.mark.parametrize("fmt", [2, 3])
 def test_decode_bit_exact_through_the_mfma(hk, kernel, M, fmt):
-    K = 256
+    K = 512 if kernel == 3 else 256
     rng = np.random.default_rng(fmt * 10 + kernel)
     codes = rng.integers(0, 64, size=(M, K), dtype=np.uint8)
     codes[0, :64] = np.arange(64)  # every code of the format at least once
@@ -139,14 +139,20 @@ def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb):
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
-def test_tiled_rejects_shapes_it_cannot_take(hk):
+def test_forced_kernels_reject_shapes_they_cannot_take(hk):
     ap, asc, bp, bsc = operands(64, 64, 64, 2, 2, seed=1)
     with pytest.raises(RuntimeError, match="bad shape"):
         gemm(hk, ap, bp, asc, bsc, kernel=2)
+    with pytest.raises(RuntimeError, match="bad shape"):
+        gemm(hk, ap, bp, asc, bsc, kernel=3)          # M > 32
+    ap, asc, bp, bsc = operands(16, 64, 384, 2, 2, seed=1)
+    with pytest.raises(RuntimeError, match="bad shape"):
+        gemm(hk, ap, bp, asc, bsc, kernel=3)          # K % 512
+    check(gemm(hk, ap, bp, asc, bsc, kernel=0), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)  # automatic: generic
 
 
 # ------------------------------------------------------------------ skinny kernel
-@pytest.mark.parametrize("M,N,K", [(16, 64, 128), (1, 32, 256), (7, 100, 2048), (16, 512, 3584), (32, 96, 1152), (13, 33, 128 * 17)])
+@pytest.mark.parametrize("M,N,K", [(16, 64, 512), (1, 32, 1024), (7, 100, 2048), (16, 512, 3584), (32, 96, 1536), (13, 33, 512 * 9), (17, 31, 512 * 13), (16, 1000, 512 * 20)])
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
 def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + 2 * N + K, kind_b="weights")
