@@ -57,12 +57,18 @@ __device__ __forceinline__ void wait_vmcnt_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void barrier_only() { asm volatile("s_barrier" ::: "memory"); }
+
 template <int FA, int FB, typename Out, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                  const uint8_t* __restrict__ As,
                                                                  const uint8_t* __restrict__ Bs,
                                                                  typename Out::type* __restrict__ C, int M, int N, int K,
-                                                                 int tiles_m, int tiles_n, int dev_mode) {
+                                                                 int tiles_m, int tiles_n, int dev_mode, int sched) {
   constexpr int NW = WM * WN;
   constexpr int TM = 8 / WM, TN = 8 / WN;  // 32x32 MFMA tiles per wave in M and N
   constexpr int OPS = 24 / NW;             // operand DMA instructions per wave per operand per K-tile
@@ -138,13 +144,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
   // ---- DMA issue slot of K-tile t: its operand loads, then (every fourth tile) the scales of the
   // four K-tiles starting at t + 2.  Every slot therefore ends with at most a scale load, and a
   // wait that leaves 2*OPS loads outstanding always covers the whole previous slot.
-  auto issue_scales = [&](int grp) {
+  auto issue_scales = [&](int grp) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + (wave & 3) * 1024;
     const int soff = grp * 16;
     if (NW == 4 || wave < 4) dma16(rSA, dst, voff_s, soff);
     if (NW == 4 || wave >= 4) dma16(rSB, dst + kScStage, voff_s, soff);
   };
-  auto issue_slot = [&](int t) {
+  auto issue_slot = [&](int t) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + (t % kStages) * kStage + wave * (OPS * 1024);
     const int soff = dev_mode == 3 ? t * 24576 : t * 96;
 #pragma unroll
@@ -154,22 +160,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
     if ((t & 3) == 2 && t + 2 < nkt) issue_scales((t + 2) >> 2);
   };
 
-  // ---- prologue: scales of the first four K-tiles, then K-tiles 0 and 1
-  issue_scales(0);
-  issue_slot(0);
-  if (nkt > 1) issue_slot(1);
-
-  for (int kt = 0; kt < nkt; kt++) {
-    // tile kt has landed (this wave's share) once at most the next slot's 2*OPS loads are pending;
-    // the barrier publishes every wave's share and retires the ring slot tile kt+2 will overwrite
-    if (kt + 1 < nkt) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();
-    if (kt + 2 < nkt && dev_mode != 1) issue_slot(kt + 2);
-    if (dev_mode >= 2) continue;
-
+  // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
+  v4i fa[TM][3], fb[TN][3];
+  int sca[TM], scb[TN];
+  auto read_tile = [&](int kt) __attribute__((always_inline)) {
     const uint8_t* st = smem + (kt % kStages) * kStage;
     const uint8_t* sc = smem + ((kt >> 2) & 1) * kScaleBuf + (kt & 3) * 4;
-    v4i fa[TM][3], fb[TN][3];
-    int sca[TM], scb[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -182,9 +178,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
       for (int c = 0; c < 3; c++) fa[i][c] = *reinterpret_cast<const v4i*>(st + a_rd[c] + i * 3072);
       sca[i] = *reinterpret_cast<const uint16_t*>(sc + sa_rd + i * 512);
     }
-    // first K-block of every lane for all tiles, then the second: two MFMAs into the same
-    // accumulator are TM*TN instructions apart.  First source = B rows (index n), second = A rows
-    // (index m): a lane ends up owning 4 consecutive n of one m, which keeps the C store wide.
+  };
+  // first K-block of every lane for all tiles, then the second: two MFMAs into the same accumulator
+  // are TM*TN instructions apart.  First source = B rows (index n), second = A rows (index m): a
+  // lane ends up owning 4 consecutive n of one m, which keeps the C store wide.
+  auto mma_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const v8i a0 = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, -1, -1);
@@ -203,27 +201,112 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
         acc[i][j] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[i][j], scb[j], sca[i]);
       }
     }
+  };
+
+  // ---- prologue: scales of the first four K-tiles, then K-tiles 0 and 1
+  issue_scales(0);
+  issue_slot(0);
+  if (nkt > 1) issue_slot(1);
+
+  if (sched == 0) {
+    // plain schedule: one barrier per K-tile, every wave loads then multiplies
+    for (int kt = 0; kt < nkt; kt++) {
+      // tile kt has landed (this wave's share) once at most the next slot's 2*OPS loads are pending;
+      // the barrier publishes every wave's share and retires the ring slot tile kt+2 will overwrite
+      if (kt + 1 < nkt) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();
+      if (kt + 2 < nkt && dev_mode != 1) issue_slot(kt + 2);
+      if (dev_mode >= 2) continue;
+      read_tile(kt);
+      mma_tile();
+    }
+  } else {
+    // ping-pong (the reference's 8-wave pattern, analysis/bf16_gemm/mi325x/kernel_8192.cpp:75-153):
+    // waves 0-3 and waves 4-7 (one of each per SIMD) run half a K-tile out of phase, so that on
+    // every SIMD one wave issues MFMAs while the other reads LDS and issues the next loads.
+    // Barrier n is common to all waves; between barriers 2k and 2k+1 the first group is in its
+    // memory cluster for tile k, between 2k+1 and 2k+2 in its compute cluster; the second group
+    // does the same one barrier later.  A ring slot is refilled (tile k+2 over tile k-1) only after
+    // the barrier by which both groups have finished reading it, and each wave waits for its own
+    // share of tile k+1 before the barrier that precedes the first read of that tile.
+    constexpr int SCL = 1;  // scale loads per wave per slot that carries scales (8 waves)
+    auto wait_next_tile = [&](int kt) __attribute__((always_inline)) {
+      if (kt + 2 < nkt) {  // slot kt+2 was issued in this iteration and may stay in flight
+        if ((kt & 3) == 0 && kt + 4 < nkt) wait_vmcnt<2 * OPS + SCL>(); else wait_vmcnt<2 * OPS>();
+      } else {
+        wait_vmcnt<0>();
+      }
+    };
+    if (nkt > 1) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();  // tile 0 landed everywhere
+    if (wm == 1) barrier_only();                                                // phase offset
+    for (int kt = 0; kt < nkt; kt++) {
+      if (kt + 2 < nkt && dev_mode != 1 && dev_mode < 4) issue_slot(kt + 2);
+      if (dev_mode < 2 || dev_mode == 5) read_tile(kt);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this tile's LDS reads are done before anyone may refill its slot
+      if (wm == 1) wait_next_tile(kt);
+      __builtin_amdgcn_sched_barrier(0);
+      barrier_only();
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(1);
+      if (dev_mode < 2 || dev_mode == 4) mma_tile();
+      __builtin_amdgcn_s_setprio(0);
+      if (wm == 0) wait_next_tile(kt);
+      __builtin_amdgcn_sched_barrier(0);
+      barrier_only();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (wm == 0) barrier_only();  // every wave executes the same number of barriers
   }
 
-  // ---- epilogue: lane owns C[m][n .. n+3] for 4 values of n per 32x32 tile
-  typename Out::type* cbase = C + ((size_t)pm * kBM + wm * (TM * 32) + r32) * (size_t)N + (size_t)pn * kBN + wn * (TN * 32) + 4 * h;
+  // ---- epilogue.  A lane owns C[m][n .. n+3] for four values of n per 32x32 tile, i.e. 8 bytes of
+  // bf16 per store: written straight to global memory those are partial-line writes (measured 1.4x
+  // the output in HBM write traffic and a visible tail after every tile).  The bf16 tile (128 KB)
+  // is therefore staged through LDS, which is free once the K loop is over, and written out in
+  // whole rows: one wave store = two rows x 512 contiguous bytes.
+  if constexpr (sizeof(typename Out::type) == 2) {
+    constexpr int kRowPitch = 512 + 16;  // bytes; the pad spreads the 32 rows of a store over the banks
+    static_assert(256 * kRowPitch <= (int)sizeof(smem), "C tile fits the ring");
+    __syncthreads();  // every wave is done reading the ring
+    uint8_t* cs = smem + (wm * (TM * 32) + r32) * kRowPitch + (wn * (TN * 32) + 4 * h) * 2;
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+      for (int j = 0; j < TN; j++)
 #pragma unroll
-      for (int g = 0; g < 4; g++)
-        store4(cbase + (size_t)i * 32 * N + j * 32 + 8 * g, acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-               acc[i][j][4 * g + 3]);
+        for (int g = 0; g < 4; g++) {
+          const u32x2 v = {pack_bf16x2(acc[i][j][4 * g], acc[i][j][4 * g + 1]), pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
+          *reinterpret_cast<u32x2*>(cs + i * 32 * kRowPitch + (j * 32 + 8 * g) * 2) = v;
+        }
+    __syncthreads();
+    const int chunk = tid & 31, row0 = tid >> 5;  // 32 lanes cover one 512-byte row
+    uint8_t* cg = reinterpret_cast<uint8_t*>(C) + ((size_t)pm * kBM + row0) * (size_t)N * 2 + (size_t)pn * kBN * 2 + chunk * 16;
+    constexpr int kRowsPerPass = NW * 2;
+#pragma unroll 4
+    for (int r = 0; r < 256; r += kRowsPerPass) {
+      const v4i v = *reinterpret_cast<const v4i*>(smem + (row0 + r) * kRowPitch + chunk * 16);
+      *reinterpret_cast<v4i*>(cg + (size_t)r * N * 2) = v;
+    }
+  } else {
+    typename Out::type* cbase = C + ((size_t)pm * kBM + wm * (TM * 32) + r32) * (size_t)N + (size_t)pn * kBN + wn * (TN * 32) + 4 * h;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+          store4(cbase + (size_t)i * 32 * N + j * 32 + 8 * g, acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                 acc[i][j][4 * g + 3]);
+  }
 }
 
 bool gemm_tiled_supports(const GemmArgs& g) {
   return g.M > 0 && g.N > 0 && g.K > 0 && g.M % kBM == 0 && g.N % kBN == 0 && g.K % kBK == 0 &&
-         (long)kBM * (g.K / 4 * 3) < (1L << 31) && ((uintptr_t)g.C % (g.f32out ? 16 : 8)) == 0;
+         (long)kBM * (g.K / 4 * 3) < (1L << 31) && ((uintptr_t)g.C % 16) == 0;
 }
 
 static int g_tiled_waves = 8;
 static int g_dev_mode = 0;
+static int g_sched = 1;
+void set_sched(int v) { g_sched = v; }
 void set_dev_mode(int m) { g_dev_mode = m; }
 void set_tiled_waves(int w) { g_tiled_waves = w; }
 
@@ -231,9 +314,9 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int tm = g.M / kBM, tn = g.N / kBN;
   if (g_tiled_waves == 4)
-    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode);
+    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0);
   else
-    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode);
+    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0);
   return hipGetLastError();
 }
 
