@@ -23,10 +23,14 @@ int check_device() {
 }
 
 int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
-                int fmt_b, bool f32out, void* stream) {
+                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream) {
   if (M < 0 || N < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
   if ((fmt_a != MXFP6_FMT_E2M3 && fmt_a != MXFP6_FMT_E3M2) || (fmt_b != MXFP6_FMT_E2M3 && fmt_b != MXFP6_FMT_E3M2))
     return MXFP6_EINVAL_FMT;
+  if ((layout_a != MXFP6_LAYOUT_ROW && layout_a != MXFP6_LAYOUT_TILE) || (layout_b != MXFP6_LAYOUT_ROW && layout_b != MXFP6_LAYOUT_TILE))
+    return MXFP6_EINVAL_LAYOUT;
+  if ((layout_a == MXFP6_LAYOUT_TILE && (M % 32 || K % 128)) || (layout_b == MXFP6_LAYOUT_TILE && (N % 32 || K % 128)))
+    return MXFP6_EINVAL_SHAPE;
   if (M == 0 || N == 0) return MXFP6_OK;
   if (!C) return MXFP6_EINVAL_PTR;
   if (K > 0 && (!A || !B || !As || !Bs)) return MXFP6_EINVAL_PTR;
@@ -39,7 +43,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     hipError_t e = mxfp6::launch_fill_zero(C, (size_t)M * N * (f32out ? 4 : 2), s);
     return e == hipSuccess ? MXFP6_OK : (int)e;
   }
-  mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out};
+  mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out, layout_a, layout_b};
   const int force = g_force.load(std::memory_order_relaxed);
   hipError_t e;
   if (force == 1) {
@@ -67,12 +71,28 @@ extern "C" {
 
 int mxfp6_gemm(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
                int fmt_b, void* stream) {
-  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, stream);
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, 0, 0, stream);
 }
 
 int mxfp6_gemm_f32out(const void* A, const void* B, const void* As, const void* Bs, float* C, int M, int N, int K,
                       int fmt_a, int fmt_b, void* stream) {
-  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, true, stream);
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, true, 0, 0, stream);
+}
+
+int mxfp6_gemm_ex(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
+                  int fmt_b, int layout_a, int layout_b, int out_f32, void* stream) {
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, out_f32 != 0, layout_a, layout_b, stream);
+}
+
+int mxfp6_tile_operand(const void* src, void* dst, int rows, int K, int tile, void* stream) {
+  if (rows < 0 || K < 0 || rows % 32 || K % 128) return MXFP6_EINVAL_SHAPE;
+  if (rows == 0 || K == 0) return MXFP6_OK;
+  if (!src || !dst) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return MXFP6_EINVAL_ALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  hipError_t e = mxfp6::launch_tile_operand((const uint8_t*)src, (uint8_t*)dst, rows, K, tile, (hipStream_t)stream);
+  return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
 int mxfp6_set_kernel(int which) {
@@ -81,14 +101,20 @@ int mxfp6_set_kernel(int which) {
 }
 
 int mxfp6_quantize(const float* X, void* packed, void* scales, int rows, int K, int fmt, void* stream) {
+  return mxfp6_quantize_ex(X, packed, scales, rows, K, fmt, MXFP6_LAYOUT_ROW, stream);
+}
+
+int mxfp6_quantize_ex(const float* X, void* packed, void* scales, int rows, int K, int fmt, int layout, void* stream) {
   if (rows < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
+  if (layout != MXFP6_LAYOUT_ROW && layout != MXFP6_LAYOUT_TILE) return MXFP6_EINVAL_LAYOUT;
+  if (layout == MXFP6_LAYOUT_TILE && (rows % 32 || K % 128)) return MXFP6_EINVAL_SHAPE;
   if (fmt != MXFP6_FMT_E2M3 && fmt != MXFP6_FMT_E3M2) return MXFP6_EINVAL_FMT;
   if (rows == 0 || K == 0) return MXFP6_OK;
   if (!X || !packed || !scales) return MXFP6_EINVAL_PTR;
   if (((uintptr_t)X & 15) || ((uintptr_t)packed & 3)) return MXFP6_EINVAL_ALIGN;
   int rc = check_device();
   if (rc) return rc;
-  hipError_t e = mxfp6::launch_quantize(X, (uint8_t*)packed, (uint8_t*)scales, rows, K, fmt, (hipStream_t)stream);
+  hipError_t e = mxfp6::launch_quantize(X, (uint8_t*)packed, (uint8_t*)scales, rows, K, fmt, layout, (hipStream_t)stream);
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
@@ -100,13 +126,14 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_EINVAL_FMT: return "mxfp6: format must be 2 (e2m3) or 3 (e3m2)";
     case MXFP6_EINVAL_ALIGN: return "mxfp6: pointer alignment (packed operands 4 bytes, fp32 input 16 bytes)";
     case MXFP6_ENODEVICE: return "mxfp6: the current device is not gfx950 (MI355X)";
+    case MXFP6_EINVAL_LAYOUT: return "mxfp6: layout must be 0 (row-major) or 1 (tile-major)";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 100; }
+int mxfp6_abi_version(void) { return 101; }
 
 // development knob (not part of the ABI header)
 int mxfp6_dev_set(const char* name, int value) {

@@ -55,4 +55,12 @@ __device__ __forceinline__ v16f mfma_fp6(v8i sa, v8i sb, v16f acc, int scale_sa,
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(sa, sb, acc, FMT_SA, FMT_SB, OPA, scale_sa, OPB, scale_sb);
 }
 
+// Byte offset, inside a tile-major operand, of byte `b` (0 .. 3K/4) of row `row`; nkt = K / 128.
+// Tiles are 32 rows x 96 bytes in the kernels' LDS image order (16-byte pieces, pairs swapped in
+// rows with bit 3 set).
+__host__ __device__ __forceinline__ size_t tile_major_offset(int row, int b, int nkt) {
+  const int kt = b / 96, in = b - kt * 96, c = in >> 4, r = row & 31;
+  return ((size_t)(row >> 5) * nkt + kt) * 3072 + (size_t)((r * 6 + (c ^ ((r >> 3) & 1))) * 16 + (in & 15));
+}
+
 }  // namespace mxfp6

@@ -11,7 +11,8 @@ namespace mxfp6 {
 template <int FA, int FB, typename Out>
 __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                           const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
-                                                          typename Out::type* __restrict__ C, int M, int N, int K) {
+                                                          typename Out::type* __restrict__ C, int M, int N, int K, int layout_a,
+                                                          int layout_b) {
   const int lane = threadIdx.x, h = lane >> 5, r = lane & 31;
   const long m = (long)blockIdx.y * 32 + r, n = (long)blockIdx.x * 32 + r;
   const int nkb = K / 32;
@@ -29,11 +30,13 @@ __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restr
     v8i a = {0, 0, 0, 0, 0, 0, 0, 0}, b = {0, 0, 0, 0, 0, 0, 0, 0};
     int sa = 127, sb = 127;
     if (kv && mv) {
-      for (int i = 0; i < 6; i++) a[i] = (int)arow[kb * 6 + i];
+      for (int i = 0; i < 6; i++)
+        a[i] = layout_a ? *reinterpret_cast<const int*>(A + tile_major_offset((int)m, kb * 24 + 4 * i, nkb / 4)) : (int)arow[kb * 6 + i];
       sa = asr[kb];
     }
     if (kv && nv) {
-      for (int i = 0; i < 6; i++) b[i] = (int)brow[kb * 6 + i];
+      for (int i = 0; i < 6; i++)
+        b[i] = layout_b ? *reinterpret_cast<const int*>(B + tile_major_offset((int)n, kb * 24 + 4 * i, nkb / 4)) : (int)brow[kb * 6 + i];
       sb = bsr[kb];
     }
     // rows of the first source index n (B), columns index m (A): each lane then owns 4 consecutive n
@@ -52,7 +55,7 @@ __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restr
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   dim3 grid((g.N + 31) / 32, (g.M + 31) / 32);
-  gemm_generic_kernel<FA, FB, Out><<<grid, 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K);
+  gemm_generic_kernel<FA, FB, Out><<<grid, 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_a, g.layout_b);
   return hipGetLastError();
 }
 

@@ -4,7 +4,7 @@
 // (32 output columns) and splits K over its waves in chunks of four K-tiles (4 x 128 elements =
 // 384 bytes per row = three whole 128-byte lines), dealt round-robin: wave w takes chunks w, w+NW, ...
 // so the workgroup streams one contiguous K range of its 32 rows and no cache line is shared
-// between chunks.  Each wave owns a private 4-stage LDS ring (one stage per K-tile of a chunk):
+// between chunks.  With a tile-major B the 32 rows x K of a workgroup are one contiguous run of HBM.  Each wave owns a private 4-stage LDS ring (one stage per K-tile of a chunk):
 //   global --buffer_load_dwordx4 ... lds--> LDS --ds_read_b128--> MFMA sources
 // with the same lane->address map as the tiled kernel (consecutive lanes fetch consecutive 16-byte
 // pieces of a row; row-major 96-byte LDS rows with a pair swap that makes the reads conflict-free).
@@ -50,7 +50,7 @@ __device__ __forceinline__ void wait_loads(v4i& s0, v4i& s1) {
 template <int FA, int FB, typename Out, int AR, int NW>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
-                                                              typename Out::type* __restrict__ C, int M, int N, int K, int dev) {
+                                                              typename Out::type* __restrict__ C, int M, int N, int K, int layout_b) {
   constexpr int kBTile = 32 * 96, kATile = AR * 96, kStage = kBTile + kATile, kRing = kStagesSk * kStage;
   constexpr int kADma = (kATile + 1023) / 1024;  // direct loads per A tile (the last one half full when AR = 16)
   constexpr int kDmaPerTile = 3 + kADma;
@@ -77,8 +77,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     const int o = i * 64 + lane, r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
     voff[i] = r * rowbytes + c * 16;
   }
-  int voffc[3];
-  for (int i = 0; i < 3; i++) voffc[i] = dev == 3 ? (i * 64 + lane) * 16 : voff[i];
+  // tile-major B: the 32-row tile is stored in LDS image order, a load is one contiguous KiB
+  int voff_bt[3];
+#pragma unroll
+  for (int i = 0; i < 3; i++) voff_bt[i] = layout_b ? (i * 64 + lane) * 16 : voff[i];
   const int voff_bs = r32 * sbytes, voff_as = (AR == 16 ? (r32 & 15) : r32) * sbytes;
 
   const uint32_t ring = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kRing;
@@ -107,11 +109,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   auto issue_tile = [&](int chunk, int u) {  // K-tile u of a chunk into stage u
     const int t = min(chunk * 4 + u, nkt - 1);  // past-the-end tiles re-read the last one and are never multiplied
     const int so = __builtin_amdgcn_readfirstlane(t * 96);
-    const int soc = __builtin_amdgcn_readfirstlane(dev == 3 ? t * 3072 : t * 96);
+    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? t * 3072 : t * 96);
     const uint32_t dst = ring + u * kStage;
 #pragma unroll
-    for (int i = 0; i < 3; i++) dma16_sk(dev == 2 ? rA : rB, dst + i * 1024, voffc[i], soc);
-    dma16_sk(dev == 1 ? rB : rA, dst + kBTile, voff[0], so);
+    for (int i = 0; i < 3; i++) dma16_sk(rB, dst + i * 1024, voff_bt[i], sob);
+    dma16_sk(rA, dst + kBTile, voff[0], so);
     if constexpr (kADma == 2) {
       if (lane < 32) dma16_sk(rA, dst + kBTile + 1024, voff[1], so);
     } else {
@@ -200,19 +202,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 
 bool gemm_skinny_supports(const GemmArgs& g) {
   // K % 512: chunks of four K-tiles are whole (three 128-byte lines per row, 16 scale bytes per row)
-  return g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
+  return g.layout_a == 0 && g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
 }
 
-static int g_skinny_dev = 0;
-void set_skinny_dev(int v) { g_skinny_dev = v; }
+void set_skinny_dev(int) {}
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const unsigned grid = (g.N + 31) / 32;
   if (g.M <= 16)
-    gemm_skinny_kernel<FA, FB, Out, 16, 8><<<grid, 8 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g_skinny_dev);
+    gemm_skinny_kernel<FA, FB, Out, 16, 8><<<grid, 8 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b);
   else
-    gemm_skinny_kernel<FA, FB, Out, 32, 6><<<grid, 6 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g_skinny_dev);
+    gemm_skinny_kernel<FA, FB, Out, 32, 6><<<grid, 6 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b);
   return hipGetLastError();
 }
 

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
                                                                  const uint8_t* __restrict__ As,
                                                                  const uint8_t* __restrict__ Bs,
                                                                  typename Out::type* __restrict__ C, int M, int N, int K,
-                                                                 int tiles_m, int tiles_n, int dev_mode, int sched) {
+                                                                 int tiles_m, int tiles_n, int dev_mode, int sched, int layout_a, int layout_b) {
   constexpr int NW = WM * WN;
   constexpr int TM = 8 / WM, TN = 8 / WN;  // 32x32 MFMA tiles per wave in M and N
   constexpr int OPS = 24 / NW;             // operand DMA instructions per wave per operand per K-tile
@@ -109,15 +109,22 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
   const __amdgpu_buffer_rsrc_t rSA = make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)kBM * sbytes);
   const __amdgpu_buffer_rsrc_t rSB = make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)kBN * sbytes);
 
-  // per-lane global byte offsets of the OPS direct loads (identical for A and B: same row pitch)
-  int voff[OPS];
+  // per-lane global byte offsets of the OPS direct loads.  Load q = wave*OPS + i fills LDS bytes
+  // [q*1024, q*1024 + 1024) of the operand tile.  Row-major operand: slot o holds piece
+  // (o%6) ^ ((row>>3)&1) of row o/6, K-tile t starts at byte 96 t of a row.  Tile-major operand:
+  // the 3072-byte tile of 32 rows is stored in exactly this order, so the load is one contiguous
+  // KiB, row-tiles are (K/128)*3072 bytes apart and K-tile t starts at byte 3072 t.
+  int voff_a[OPS], voff_b[OPS];
 #pragma unroll
   for (int i = 0; i < OPS; i++) {
-    const int o = (wave * OPS + i) * 64 + lane;  // linear 16-byte slot inside the LDS image
+    const int q = wave * OPS + i, o = q * 64 + lane;  // linear 16-byte slot inside the LDS image
     const int r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
-    voff[i] = r * rowbytes + c * 16;
-    if (dev_mode == 3) voff[i] = o * 16;
+    const int vrow = r * rowbytes + c * 16;
+    const int vtile = (q / 3) * (nkt * 3072) + (q % 3) * 1024 + lane * 16;
+    voff_a[i] = layout_a ? vtile : vrow;
+    voff_b[i] = layout_b ? vtile : vrow;
   }
+  const int kstep_a = layout_a ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
   // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; with 4 waves every wave
   // loads 64 rows of A and of B, with 8 waves waves 0-3 load A and waves 4-7 load B
   const int voff_s = ((wave & 3) * 64 + lane) * sbytes;
@@ -152,11 +159,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
   };
   auto issue_slot = [&](int t) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + (t % kStages) * kStage + wave * (OPS * 1024);
-    const int soff = dev_mode == 3 ? t * 24576 : t * 96;
+    const int soff_a = t * kstep_a, soff_b = t * kstep_b;
 #pragma unroll
-    for (int i = 0; i < OPS; i++) dma16(rA, dst + i * 1024, voff[i], soff);
+    for (int i = 0; i < OPS; i++) dma16(rA, dst + i * 1024, voff_a[i], soff_a);
 #pragma unroll
-    for (int i = 0; i < OPS; i++) dma16(rB, dst + kOpStage + i * 1024, voff[i], soff);
+    for (int i = 0; i < OPS; i++) dma16(rB, dst + kOpStage + i * 1024, voff_b[i], soff_b);
     if ((t & 3) == 2 && t + 2 < nkt) issue_scales((t + 2) >> 2);
   };
 
@@ -314,9 +321,9 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int tm = g.M / kBM, tn = g.N / kBN;
   if (g_tiled_waves == 4)
-    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0);
+    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0, g.layout_a, g.layout_b);
   else
-    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0);
+    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0, g.layout_a, g.layout_b);
   return hipGetLastError();
 }
 

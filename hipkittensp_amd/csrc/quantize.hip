@@ -39,7 +39,7 @@ __device__ __forceinline__ uint32_t quantise_mag(float a) {
 
 template <int FMT>
 __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ X, uint8_t* __restrict__ packed,
-                                                       uint8_t* __restrict__ scales, long nblocks) {
+                                                       uint8_t* __restrict__ scales, long nblocks, int nkb, int layout) {
   constexpr int MB = FMT == 2 ? 3 : 2, BIAS = FMT == 2 ? 1 : 3, EB = FMT == 2 ? 2 : 3, EMAX = FMT == 2 ? 2 : 4;
   const long b = (long)blockIdx.x * 256 + threadIdx.x;
   if (b >= nblocks) return;
@@ -80,19 +80,45 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
     w[d] |= g << sh;
     if (sh > 8) w[d + 1] |= g >> (32 - sh);
   }
-  uint32_t* dst = reinterpret_cast<uint32_t*>(packed + b * 24);
+  if (layout == 0) {
+    uint32_t* dst = reinterpret_cast<uint32_t*>(packed + b * 24);
 #pragma unroll
-  for (int i = 0; i < 6; i++) dst[i] = w[i];
+    for (int i = 0; i < 6; i++) dst[i] = w[i];
+  } else {
+    const int row = (int)(b / nkb), kb = (int)(b - (long)row * nkb);
+#pragma unroll
+    for (int i = 0; i < 6; i++) *reinterpret_cast<uint32_t*>(packed + tile_major_offset(row, kb * 24 + 4 * i, nkb / 4)) = w[i];
+  }
   scales[b] = (uint8_t)sb;
 }
 
-hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, hipStream_t s) {
+hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s) {
   const long nblocks = (long)rows * (K / 32);
   const unsigned grid = (unsigned)((nblocks + 255) / 256);
   if (fmt == 2)
-    quantize_kernel<2><<<grid, 256, 0, s>>>(X, packed, scales, nblocks);
+    quantize_kernel<2><<<grid, 256, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
   else
-    quantize_kernel<3><<<grid, 256, 0, s>>>(X, packed, scales, nblocks);
+    quantize_kernel<3><<<grid, 256, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
+  return hipGetLastError();
+}
+
+// row-major <-> tile-major: one lane moves one 16-byte piece
+__global__ __launch_bounds__(256) void tile_operand_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, long npieces,
+                                                          int nkt, int tile) {
+  const long s = (long)blockIdx.x * 256 + threadIdx.x;
+  if (s >= npieces) return;
+  // s indexes the row-major pieces: row = s / (6 nkt), piece p of the row
+  const int per_row = 6 * nkt;
+  const int row = (int)(s / per_row), p = (int)(s - (long)row * per_row);
+  const size_t rm = (size_t)s * 16, tm = tile_major_offset(row, p * 16, nkt);
+  const v4i v = *reinterpret_cast<const v4i*>(src + (tile ? rm : tm));
+  *reinterpret_cast<v4i*>(dst + (tile ? tm : rm)) = v;
+}
+
+hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s) {
+  const long npieces = (long)rows * (K / 128) * 6;
+  if (npieces == 0) return hipSuccess;
+  tile_operand_kernel<<<(unsigned)((npieces + 255) / 256), 256, 0, s>>>(src, dst, npieces, K / 128, tile);
   return hipGetLastError();
 }
 

@@ -17,6 +17,9 @@ adds the checks a packed format needs (dtype, packed width, scale shape).
     B_scale  uint8 [N, K/32]
     C        bfloat16 [M, N]   (a float32 C receives the accumulators before the bf16 rounding)
     fmt_*    2 = e2m3, 3 = e3m2
+    layout_* LAYOUT_ROW (as above) or LAYOUT_TILE: the same bytes regrouped into 32-row x 128-element
+             tiles in the kernels' LDS order (tile_operand() converts; quantize(..., layout=LAYOUT_TILE)
+             emits it directly); loads of a tile-major operand are contiguous
 
 PyTorch is used for tensor storage and the current stream only; the work is done by the HIP
 library behind include/mxfp6_gemm.h.
@@ -27,6 +30,8 @@ from . import _lib
 
 E2M3 = 2
 E3M2 = 3
+LAYOUT_ROW = 0
+LAYOUT_TILE = 1
 
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_TILED, KERNEL_SKINNY = 0, 1, 2, 3
 
@@ -61,7 +66,8 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3) -> None:
+def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, layout_a: int = LAYOUT_ROW,
+                   layout_b: int = LAYOUT_ROW) -> None:
     import torch
 
     A, B = _as_tensor(A, "A"), _as_tensor(B, "B")
@@ -74,6 +80,8 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
         raise RuntimeError(f"C: expected dtype bfloat16 (or float32 for unrounded output), got {C.dtype}")
     if fmt_a not in (E2M3, E3M2) or fmt_b not in (E2M3, E3M2):
         raise RuntimeError("fmt_a / fmt_b must be 2 (e2m3) or 3 (e3m2)")
+    if layout_a not in (LAYOUT_ROW, LAYOUT_TILE) or layout_b not in (LAYOUT_ROW, LAYOUT_TILE):
+        raise RuntimeError("layout_a / layout_b must be LAYOUT_ROW (0) or LAYOUT_TILE (1)")
     M, wa = _rows_cols(A, "A")
     N, wb = _rows_cols(B, "B")
     if wa != wb:
@@ -90,15 +98,19 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
     devs = {t.device for t in (A, B, A_scale, B_scale, C)}
     if len(devs) != 1:
         raise RuntimeError(f"all tensors must be on one device, got {sorted(map(str, devs))}")
+    for rows, lay, name in ((M, layout_a, "A"), (N, layout_b, "B")):
+        if lay == LAYOUT_TILE and (rows % 32 or K % 128):
+            raise RuntimeError(f"{name}: a tile-major operand needs rows % 32 == 0 and K % 128 == 0")
     L = _lib.lib()
-    fn = L.mxfp6_gemm if C.dtype == torch.bfloat16 else L.mxfp6_gemm_f32out
     with torch.cuda.device(C.device):
-        rc = fn(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K, fmt_a, fmt_b, _stream())
+        rc = L.mxfp6_gemm_ex(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
+                             fmt_a, fmt_b, layout_a, layout_b, int(C.dtype == torch.float32), _stream())
     _lib.check(rc, "dispatch_micro")
 
 
-def quantize(X, fmt: int = E2M3):
-    """fp32 [rows, K] on the GPU -> (packed uint8 [rows, 3K/4], scales uint8 [rows, K/32])."""
+def quantize(X, fmt: int = E2M3, layout: int = LAYOUT_ROW):
+    """fp32 [rows, K] on the GPU -> (packed uint8 [rows, 3K/4], scales uint8 [rows, K/32]).
+    With layout=LAYOUT_TILE the packed bytes are written tile-major (rows % 32 == 0, K % 128 == 0)."""
     import torch
 
     X = _as_tensor(X, "X")
@@ -112,9 +124,26 @@ def quantize(X, fmt: int = E2M3):
     packed = torch.empty(*X.shape[:-1], K // 4 * 3, dtype=torch.uint8, device=X.device)
     scales = torch.empty(*X.shape[:-1], K // 32, dtype=torch.uint8, device=X.device)
     with torch.cuda.device(X.device):
-        rc = _lib.lib().mxfp6_quantize(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, _stream())
+        rc = _lib.lib().mxfp6_quantize_ex(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, layout, _stream())
     _lib.check(rc, "quantize")
     return packed, scales
+
+
+def tile_operand(packed, untile: bool = False):
+    """Row-major packed operand [rows, 3K/4] -> tile-major (same shape, regrouped bytes), or back."""
+    import torch
+
+    packed = _as_tensor(packed, "packed")
+    if packed.dtype != torch.uint8:
+        raise RuntimeError(f"packed: expected dtype uint8, got {packed.dtype}")
+    rows, w = _rows_cols(packed, "packed")
+    if w % 96 or rows % 32:
+        raise RuntimeError("tile-major layout needs rows % 32 == 0 and K % 128 == 0")
+    out = torch.empty_like(packed)
+    with torch.cuda.device(packed.device):
+        rc = _lib.lib().mxfp6_tile_operand(packed.data_ptr(), out.data_ptr(), rows, w // 3 * 4, 0 if untile else 1, _stream())
+    _lib.check(rc, "tile_operand")
+    return out
 
 
 def set_kernel(which: int) -> int:

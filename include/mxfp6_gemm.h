@@ -38,6 +38,7 @@ extern "C" {
 #define MXFP6_EINVAL_FMT (-3)   /* format code is not 2 (e2m3) or 3 (e3m2)                     */
 #define MXFP6_EINVAL_ALIGN (-4) /* a pointer violates the stated alignment                     */
 #define MXFP6_ENODEVICE (-5)    /* current device is not gfx950                                */
+#define MXFP6_EINVAL_LAYOUT (-6) /* layout code is not MXFP6_LAYOUT_ROW / MXFP6_LAYOUT_TILE    */
 
 /*
  * The operator.  Replaces the reference's dispatch_micro(A, B, C) launcher
@@ -78,6 +79,35 @@ int mxfp6_set_kernel(int which);
  * the same way (kernels/gemm/bf16fp32/utils.py:28-34).
  */
 int mxfp6_quantize(const float *X, void *packed, void *scales, int rows, int K, int fmt, void *hip_stream);
+
+/*
+ * Tile-major operand layout ("pre-shuffled" operands; rows % 32 == 0, K % 128 == 0).  The packed bytes
+ * of an operand are regrouped into tiles of 32 rows x 128 elements (3072 bytes), tile (rt, kt) at byte
+ * ((rt * (K/128)) + kt) * 3072; inside a tile, the 16-byte piece c (0..5) of row r (0..31) sits at
+ * (r*6 + (c ^ ((r >> 3) & 1))) * 16.  This is exactly the image the kernels keep in LDS, so their
+ * direct-to-LDS loads become fully contiguous (one 1 KiB run per load instead of ~11 row pieces);
+ * scale tensors are unchanged.  The reference applies its LDS swizzle to the global address of every
+ * load (include/ops/warp/memory/tile/global_to_shared.cuh:46-59); this applies it to the data once,
+ * which suits weights (converted offline) and activations (the quantiser can emit it directly).
+ */
+#define MXFP6_LAYOUT_ROW 0  /* [rows, 3K/4], K contiguous: the layout of mxfp6_gemm                */
+#define MXFP6_LAYOUT_TILE 1 /* tile-major, see above                                                */
+
+/* Row-major packed operand -> tile-major (tile != 0) or back (tile == 0); src and dst must not overlap. */
+int mxfp6_tile_operand(const void *src, void *dst, int rows, int K, int tile, void *hip_stream);
+
+/*
+ * mxfp6_gemm / mxfp6_gemm_f32out with a layout per operand (MXFP6_LAYOUT_*) and out_f32 != 0 for
+ * the fp32 output.  With both layouts MXFP6_LAYOUT_ROW it is exactly those two entry points.
+ * A tile-major operand needs rows % 32 == 0 and K % 128 == 0 (MXFP6_EINVAL_SHAPE otherwise).
+ */
+int mxfp6_gemm_ex(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, void *C,
+                  int M, int N, int K, int fmt_a, int fmt_b, int layout_a, int layout_b, int out_f32,
+                  void *hip_stream);
+
+/* mxfp6_quantize writing the packed operand in the given layout (scales are always [rows, K/32]). */
+int mxfp6_quantize_ex(const float *X, void *packed, void *scales, int rows, int K, int fmt, int layout,
+                      void *hip_stream);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

@@ -155,6 +155,24 @@ def unpack_fp6(packed: np.ndarray) -> np.ndarray:
     return out.reshape(rows, nb // 3 * 4)
 
 
+def tile_operand(packed: np.ndarray) -> np.ndarray:
+    """Row-major packed [rows, 3K/4] -> tile-major bytes (same shape): tiles of 32 rows x 96 bytes, tile
+    (rt, kt) at ((rt * K/128) + kt) * 3072; inside, 16-byte piece c of row r at (r*6 + (c ^ ((r>>3)&1))) * 16.
+    Defines the layout of include/mxfp6_gemm.h (MXFP6_LAYOUT_TILE) independently of the GPU converter."""
+    p = np.asarray(packed, dtype=np.uint8)
+    rows, w = p.shape
+    if rows % 32 or w % 96:
+        raise ValueError("rows % 32 == 0 and K % 128 == 0 required")
+    nkt = w // 96
+    x = p.reshape(rows // 32, 32, nkt, 6, 16)                      # [rt, r, kt, c, byte]
+    out = np.empty((rows // 32, nkt, 32, 6, 16), dtype=np.uint8)     # [rt, kt, r, slot, byte]
+    for r in range(32):
+        sw = (r >> 3) & 1
+        for c in range(6):
+            out[:, :, r, c ^ sw, :] = x[:, r, :, c, :]
+    return out.reshape(rows, w)
+
+
 def dequantise(packed: np.ndarray, scales: np.ndarray, fmt: int, dtype=np.float32) -> np.ndarray:
     """packed [rows, 3K/4] + scales [rows, K/32] -> values [rows, K] = table[code] * 2^(scale-127).
     Exact in fp32 whenever the result is a normal fp32 number."""

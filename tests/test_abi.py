@@ -30,7 +30,8 @@ def built_lib():
 
 def test_header_declares_the_operator():
     names = _declared_functions()
-    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_quantize", "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel"):
+    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_tile_operand",
+                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel"):
         assert want in names
 
 
@@ -47,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 100
+    assert L.mxfp6_abi_version() == 101
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -75,6 +76,15 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     assert L.mxfp6_quantize(one, one, one, 4, 40, 2, None) == -2
     assert L.mxfp6_quantize(one, one, one, 4, 64, 5, None) == -3
     assert L.mxfp6_quantize(one, one, one, 0, 64, 2, None) == 0
+    L.mxfp6_gemm_ex.restype = ci
+    L.mxfp6_gemm_ex.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp]
+    assert L.mxfp6_gemm_ex(one, one, one, one, one, 32, 32, 128, 2, 2, 2, 0, 0, None) == -6      # unknown layout
+    assert L.mxfp6_gemm_ex(one, one, one, one, one, 48, 32, 128, 2, 2, 1, 0, 0, None) == -2      # tile-major rows % 32
+    assert L.mxfp6_gemm_ex(one, one, one, one, one, 32, 32, 96, 2, 2, 0, 1, 0, None) == -2       # tile-major K % 128
+    L.mxfp6_tile_operand.restype = ci
+    L.mxfp6_tile_operand.argtypes = [vp, vp, ci, ci, ci, vp]
+    assert L.mxfp6_tile_operand(one, one, 33, 128, 1, None) == -2
+    assert L.mxfp6_tile_operand(one, None, 32, 128, 1, None) == -1
 
 
 def test_python_operator_rejects_like_the_reference():

@@ -163,6 +163,74 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
+# ------------------------------------------------------------------ tile-major operand layout
+@pytest.mark.parametrize("rows,K", [(32, 128), (64, 512), (256, 1152), (96, 8192)])
+def test_tile_operand_matches_format_definition(hk, rows, K):
+    rng = np.random.default_rng(rows + K)
+    p = rng.integers(0, 256, size=(rows, K // 4 * 3), dtype=np.uint8)
+    t = hk.tile_operand(dev(p))
+    torch.cuda.synchronize()
+    assert np.array_equal(t.cpu().numpy(), o.tile_operand(p))                       # bit exact vs the CPU definition
+    assert np.array_equal(hk.tile_operand(t, untile=True).cpu().numpy(), p)         # and back
+    x = o.make_source("normal", (rows, K), rng)
+    pt, st = hk.quantize(dev(x), 2, layout=hk.LAYOUT_TILE)                          # quantiser emitting it directly
+    pr, sr = co.quantise(x, 2)
+    assert np.array_equal(pt.cpu().numpy(), o.tile_operand(pr)) and np.array_equal(st.cpu().numpy(), sr)
+
+
+@pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (2, 256, 512, 640), (2, 512, 256, 2048), (3, 16, 128, 1024), (3, 7, 64, 512), (0, 32, 32, 128)])
+@pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
+def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
+    if kernel == 3 and la == 1:
+        pytest.skip("the skinny kernel takes a row-major A (M need not be a multiple of 32)")
+    fa, fb = 3, 2
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + N + K + la, kind_a="laplace", kind_b="weights")
+    if la == 1 and M % 32:
+        pytest.skip("tile-major needs rows % 32 == 0")
+    ref = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel)
+    A = hk.tile_operand(dev(ap)) if la else dev(ap)
+    B = hk.tile_operand(dev(bp)) if lb else dev(bp)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    prev = hk.tk_kernel.set_kernel(kernel)
+    try:
+        hk.dispatch_micro(A, B, dev(asc), dev(bsc), C, fa, fb, layout_a=la, layout_b=lb)
+        torch.cuda.synchronize()
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+    assert np.array_equal(C.cpu().numpy(), ref)      # same kernel, same arithmetic order: bit for bit
+    check(ref, o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64), fa, fb)
+
+
+def test_tile_major_rejects_bad_shapes(hk):
+    ap, asc, bp, bsc = operands(48, 32, 128, 2, 2, seed=3)
+    C = torch.empty(48, 32, dtype=torch.float32, device="cuda")
+    with pytest.raises(RuntimeError, match="tile-major"):
+        hk.dispatch_micro(dev(ap), dev(bp), dev(asc), dev(bsc), C, layout_a=hk.LAYOUT_TILE)
+    with pytest.raises(RuntimeError, match="layout"):
+        hk.dispatch_micro(dev(ap), dev(bp), dev(asc), dev(bsc), C, layout_b=7)
+
+
+def test_cfg1_and_cfg3_tile_major_full_size(hk):
+    M = N = K = 8192
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=1)
+    dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    Ct = torch.empty_like(C)
+    hk.dispatch_micro(dA, dB, dAs, dBs, C)
+    hk.dispatch_micro(hk.tile_operand(dA), hk.tile_operand(dB), dAs, dBs, Ct, layout_a=1, layout_b=1)
+    assert torch.equal(C, Ct)
+    del dA, dB, C, Ct
+    M, N, K = 16, 8192, 28672
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=3, kind_b="weights")
+    dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    Ct = torch.empty_like(C)
+    hk.dispatch_micro(dA, dB, dAs, dBs, C)
+    hk.dispatch_micro(dA, hk.tile_operand(dB), dAs, dBs, Ct, layout_b=1)
+    torch.cuda.synchronize()
+    assert torch.equal(C, Ct)
+
+
 # ------------------------------------------------------------------ edge cases
 def test_empty_and_degenerate(hk):
     z = lambda *s: torch.zeros(*s, dtype=torch.uint8, device="cuda")

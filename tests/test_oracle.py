@@ -159,6 +159,24 @@ def test_pack_roundtrip_and_bit_positions():
         assert v == codes[2, j]
 
 
+def test_tile_major_layout_definition():
+    # hand-checked placements: 64 rows, K = 256 (2 K-tiles): piece c of row r, K-tile kt
+    p = np.zeros((64, 192), np.uint8)
+    def piece(r, kt, c):
+        return p[r, kt * 96 + c * 16 : kt * 96 + c * 16 + 16]
+    piece(0, 0, 0)[:] = 1      # row 0: no swap -> slot 0 of tile (0,0): byte 0
+    piece(0, 1, 5)[:] = 2      # K-tile 1 -> tile (0,1) at 3072; slot 5 -> 3072 + 80
+    piece(9, 0, 2)[:] = 3      # row 9 has bit 3 set: piece 2 <-> slot 3 -> (9*6+3)*16 = 912
+    piece(40, 1, 1)[:] = 4     # row 40 = row-tile 1 row 8 (bit 3 set): tile (1,1) at (1*2+1)*3072 = 9216; slot 0 -> 9216 + 8*96
+    t = o.tile_operand(p).reshape(-1)
+    assert t[0] == 1 and t[3072 + 80] == 2 and t[912] == 3 and t[9216 + 768] == 4
+    assert int(t.astype(np.int64).sum()) == 16 * (1 + 2 + 3 + 4)
+    rng = np.random.default_rng(1)
+    q = rng.integers(0, 256, size=(96, 384), dtype=np.uint8)
+    tq = o.tile_operand(q)
+    assert sorted(tq.reshape(-1).tolist()) == sorted(q.reshape(-1).tolist())
+
+
 # ------------------------------------------------------------------ numpy vs C, end to end
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("kind", ["normal", "weights_outliers", "laplace"])
