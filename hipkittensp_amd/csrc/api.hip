@@ -135,14 +135,5 @@ const char* mxfp6_strerror(int code) {
 
 int mxfp6_abi_version(void) { return 101; }
 
-// development knob (not part of the ABI header)
-int mxfp6_dev_set(const char* name, int value) {
-  if (!__builtin_strcmp(name, "tiled_waves")) { mxfp6::set_tiled_waves(value); return 0; }
-  if (!__builtin_strcmp(name, "dev_mode")) { mxfp6::set_dev_mode(value); return 0; }
-  if (!__builtin_strcmp(name, "sched")) { mxfp6::set_sched(value); return 0; }
-  if (!__builtin_strcmp(name, "skinny_dev")) { mxfp6::set_skinny_dev(value); return 0; }
-  return -1;
-}
-
 #pragma GCC visibility pop
 }  // extern "C"

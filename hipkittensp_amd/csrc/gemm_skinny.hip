@@ -205,8 +205,6 @@ bool gemm_skinny_supports(const GemmArgs& g) {
   return g.layout_a == 0 && g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
 }
 
-void set_skinny_dev(int) {}
-
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const unsigned grid = (g.N + 31) / 32;

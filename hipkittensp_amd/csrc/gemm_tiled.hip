@@ -1,34 +1,38 @@
-// LDS-tiled MXFP6 GEMM for gfx950: 256x256 output tile per workgroup, K-tile 128.
+// LDS-tiled MXFP6 GEMM for gfx950: 256x256 output tile per workgroup, K-tile 128, 8 waves.
 //
 // Data path (no operand byte ever passes through a VGPR on its way to LDS):
 //   global --buffer_load_dwordx4 ... lds--> LDS (3-stage ring) --ds_read_b128--> MFMA source VGPRs
 //   v_mfma_scale_f32_32x32x64_f8f6f4 (fp32 accumulate, E8M0 block scales applied by the instruction)
-//   accumulators --v_cvt_pk_bf16_f32--> global
+//   accumulators --v_cvt_pk_bf16_f32--> LDS --> whole rows to global
 //
-// LDS image of one operand tile (256 rows x 96 bytes = 6 chunks of 16 B per row): row-major, 96 bytes
-// per row, with chunks 2p and 2p+1 exchanged in every row whose bit 3 is set:
-//     chunk c of row r lives at  r * 96 + (c ^ ((r >> 3) & 1)) * 16.
+// LDS image of one operand tile (256 rows x 96 bytes = 6 pieces of 16 B per row): row-major, 96 bytes
+// per row, with pieces 2p and 2p+1 exchanged in every row whose bit 3 is set:
+//     piece c of row r lives at  r * 96 + (c ^ ((r >> 3) & 1)) * 16.
 // A direct-to-LDS load writes lane l's 16 bytes at base + 16*l, so the image is produced by choosing
 // which global bytes each lane fetches (the same idea as the reference's swizzled global offsets,
 // include/ops/warp/memory/tile/global_to_shared.cuh:46-72).  Consecutive lanes fetch consecutive
-// 16-byte pieces of one row, so the texture-address unit sees 64..96 contiguous bytes per 4..6 lanes.
-// The pair exchange is what makes the reads conflict-free: a ds_read_b128 executes in 16-lane phases
-// ({0-3,12-15,20-23,24-27}, {4-11,16-19,28-31}, ... measured in
+// pieces of one row.  The pair exchange is what makes the reads conflict-free: a ds_read_b128
+// executes in 16-lane phases ({0-3,12-15,20-23,24-27}, {4-11,16-19,28-31}, ... measured in
 // analysis/paper_experiments/phases/ds_read_b128/phase_results.txt:4-7); with a 96-byte pitch rows r
-// and r+8 would share banks, and every phase holds each (r mod 8) once with bit 3 clear and once set.
+// and r+8 would share banks, and every phase holds each (r mod 8) once with bit 3 clear and once set
+// (measured here: 199 B/clk/CU with the exchange, 126 without).
+// A tile-major operand (MXFP6_LAYOUT_TILE) is stored in global memory in exactly this order, which
+// turns every load into one contiguous KiB.
 //
 // MFMA operand mapping: lane l of a 32x32x64 MFMA supplies row l%32 and one 32-element K-block.  Lanes
 // 0-31 take K-blocks {0,1} of the K-tile and lanes 32-63 take K-blocks {2,3}: each lane reads its row's
-// 48 contiguous bytes (three aligned 16-byte chunks) once and feeds two MFMAs (K-blocks {0,2} then {1,3}).
+// 48 contiguous bytes (three aligned 16-byte pieces) once and feeds two MFMAs (K-blocks {0,2} then {1,3}).
 // Any assignment of K-blocks to lane halves is legal as long as both operands use the same one.
 //
 // E8M0 scales ride in LDS too: 16 bytes per row cover four K-tiles, fetched by one dwordx4 direct
 // load per 64 rows per four K-tiles; a lane reads the 2 bytes it needs with ds_read_u16 and the MFMA's
 // op_sel picks byte 0 / byte 1.
 //
-// Schedule: all waves are consumers (the reference measures all-consumer above producer/consumer,
-// analysis/paper_experiments/producer_consumer_micro/plot.py:26-30); one s_barrier per K-tile; DMA for
-// tile k+2 is issued right after the barrier that publishes tile k.
+// Schedule: 8-wave ping-pong (the reference's pattern, analysis/bf16_gemm/mi325x/kernel_8192.cpp:75-153):
+// waves 0-3 and waves 4-7 (one of each per SIMD) run half a K-tile out of phase, so that on every SIMD
+// one wave issues MFMAs while the other reads LDS and issues the next loads.  All waves are consumers
+// (the reference measures all-consumer above producer/consumer,
+// analysis/paper_experiments/producer_consumer_micro/plot.py:26-30).
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -39,44 +43,42 @@ constexpr int kOpStage = 256 * 96;  // bytes of one operand tile
 constexpr int kScStage = 256 * 16;  // bytes of one operand's scales for four K-tiles
 constexpr int kGroupM = 4;          // tile rows per raster group
 constexpr int kStages = 3;          // operand ring depth
+constexpr int kStage = 2 * kOpStage, kScaleBase = kStages * kStage, kScaleBuf = 2 * kScStage;
+constexpr int kLdsBytes = kScaleBase + 2 * kScaleBuf;
+constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile 128 x 64
+constexpr int TM = 8 / WM, TN = 8 / WN;      // 32x32 MFMA tiles per wave in M and N
+constexpr int OPS = 24 / NW;                 // operand direct loads per wave per operand per K-tile
+constexpr int SCL = 1;                       // scale direct loads per wave per slot that carries scales
+static_assert(kLdsBytes <= 163840, "LDS budget");
 
 // One direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff and the hardware
 // writes them at LDS address lds_base + 16 * lane.  Issued from inline assembly so that the VMEM
-// counter is managed by hand (wait_tile below): the ring keeps two K-tiles in flight across
-// barriers, which the compiler's automatic waits would serialise.  M0 is used by nothing else here.
+// counter is managed by hand: the ring keeps two K-tiles in flight across barriers, which the
+// compiler's automatic waits would serialise.  M0 is used by nothing else in this kernel.
 __device__ __forceinline__ void dma16(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory");
 }
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_barrier() {
-  // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
-}
-
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
-__device__ __forceinline__ void barrier_only() { asm volatile("s_barrier" ::: "memory"); }
+__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
 
-template <int FA, int FB, typename Out, int WM, int WN>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
-                                                                 const uint8_t* __restrict__ As,
-                                                                 const uint8_t* __restrict__ Bs,
-                                                                 typename Out::type* __restrict__ C, int M, int N, int K,
-                                                                 int tiles_m, int tiles_n, int dev_mode, int sched, int layout_a, int layout_b) {
-  constexpr int NW = WM * WN;
-  constexpr int TM = 8 / WM, TN = 8 / WN;  // 32x32 MFMA tiles per wave in M and N
-  constexpr int OPS = 24 / NW;             // operand DMA instructions per wave per operand per K-tile
-  static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+template <int FA, int FB, typename Out>
+__global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                             const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
+                                                             typename Out::type* __restrict__ C, int M, int N, int K,
+                                                             int tiles_m, int tiles_n, int layout_a, int layout_b) {
   // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
-  constexpr int kStage = 2 * kOpStage, kScaleBase = kStages * kStage, kScaleBuf = 2 * kScStage;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[kScaleBase + 2 * kScaleBuf];
-  static_assert(sizeof(smem) <= 163840, "LDS budget");
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
 
   // ---- workgroup -> output tile: undo the round-robin XCD placement, then a grouped raster.
@@ -125,11 +127,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
     voff_b[i] = layout_b ? vtile : vrow;
   }
   const int kstep_a = layout_a ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
-  // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; with 4 waves every wave
-  // loads 64 rows of A and of B, with 8 waves waves 0-3 load A and waves 4-7 load B
+  // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; waves 0-3 load A's, 4-7 B's
   const int voff_s = ((wave & 3) * 64 + lane) * sbytes;
 
-  // per-lane LDS read offsets (bytes from the start of a stage): the lane's three chunks 3h..3h+2
+  // per-lane LDS read offsets (bytes from the start of a stage): the lane's three pieces 3h..3h+2
   const int sw = (r32 >> 3) & 1;
   int a_rd[3], b_rd[3];
 #pragma unroll
@@ -148,31 +149,29 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-  // ---- DMA issue slot of K-tile t: its operand loads, then (every fourth tile) the scales of the
-  // four K-tiles starting at t + 2.  Every slot therefore ends with at most a scale load, and a
-  // wait that leaves 2*OPS loads outstanding always covers the whole previous slot.
+  // ---- loads.  The issue slot of K-tile t holds its 2*OPS operand loads and, when t % 4 == 2, the
+  // scale load for the four K-tiles starting at t + 2 (at the end, so that a wait that leaves a
+  // whole slot in flight also covers the scales of the slot before).
   auto issue_scales = [&](int grp) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + (wave & 3) * 1024;
     const int soff = grp * 16;
-    if (NW == 4 || wave < 4) dma16(rSA, dst, voff_s, soff);
-    if (NW == 4 || wave >= 4) dma16(rSB, dst + kScStage, voff_s, soff);
+    if (wave < 4) dma16(rSA, dst, voff_s, soff); else dma16(rSB, dst + kScStage, voff_s, soff);
   };
-  auto issue_slot = [&](int t) __attribute__((always_inline)) {
-    const uint32_t dst = lds0 + (t % kStages) * kStage + wave * (OPS * 1024);
+  auto issue_ops = [&](int t, int stage) __attribute__((always_inline)) {
+    const uint32_t dst = lds0 + stage * kStage + wave * (OPS * 1024);
     const int soff_a = t * kstep_a, soff_b = t * kstep_b;
 #pragma unroll
     for (int i = 0; i < OPS; i++) dma16(rA, dst + i * 1024, voff_a[i], soff_a);
 #pragma unroll
     for (int i = 0; i < OPS; i++) dma16(rB, dst + kOpStage + i * 1024, voff_b[i], soff_b);
-    if ((t & 3) == 2 && t + 2 < nkt) issue_scales((t + 2) >> 2);
   };
 
   // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
   v4i fa[TM][3], fb[TN][3];
   int sca[TM], scb[TN];
-  auto read_tile = [&](int kt) __attribute__((always_inline)) {
-    const uint8_t* st = smem + (kt % kStages) * kStage;
-    const uint8_t* sc = smem + ((kt >> 2) & 1) * kScaleBuf + (kt & 3) * 4;
+  auto read_tile = [&](int stage, int sc_off) __attribute__((always_inline)) {
+    const uint8_t* st = smem + stage * kStage;
+    const uint8_t* sc = smem + sc_off;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -188,7 +187,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
   };
   // first K-block of every lane for all tiles, then the second: two MFMAs into the same accumulator
   // are TM*TN instructions apart.  First source = B rows (index n), second = A rows (index m): a
-  // lane ends up owning 4 consecutive n of one m, which keeps the C store wide.
+  // lane ends up owning 4 consecutive n of one m.
   auto mma_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
@@ -210,58 +209,72 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
     }
   };
 
-  // ---- prologue: scales of the first four K-tiles, then K-tiles 0 and 1
-  issue_scales(0);
-  issue_slot(0);
-  if (nkt > 1) issue_slot(1);
-
-  if (sched == 0) {
-    // plain schedule: one barrier per K-tile, every wave loads then multiplies
-    for (int kt = 0; kt < nkt; kt++) {
-      // tile kt has landed (this wave's share) once at most the next slot's 2*OPS loads are pending;
-      // the barrier publishes every wave's share and retires the ring slot tile kt+2 will overwrite
-      if (kt + 1 < nkt) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();
-      if (kt + 2 < nkt && dev_mode != 1) issue_slot(kt + 2);
-      if (dev_mode >= 2) continue;
-      read_tile(kt);
-      mma_tile();
+  // ---- the K loop.  Barrier n is common to all waves; between barriers 2k and 2k+1 group 0 (waves
+  // 0-3) is in its memory cluster for tile k and between 2k+1 and 2k+2 in its compute cluster; group 1
+  // (waves 4-7) does the same one barrier later.  A ring slot is refilled (tile k+2 over tile k-1)
+  // only after the barrier by which both groups have finished reading it, and each wave waits for
+  // its own share of tile k+1 before the barrier that precedes the first read of that tile.
+  // The body is instantiated per group (GRP) and per k mod 4 (KM), so the steady state carries no
+  // branch: STEADY means tiles k+2 and (for the scales) k+4 exist.
+  int stage = 0, stage2 = 2;  // ring slots of tile k and tile k+2
+  auto step = [&]<int GRP, int KM, bool STEADY>(int kt) __attribute__((always_inline)) {
+    const bool has2 = STEADY || kt + 2 < nkt;            // tile kt+2 exists
+    const bool has_sc = STEADY || kt + 4 < nkt;           // and so do the scales its slot would carry
+    if (has2) {
+      issue_ops(kt + 2, stage2);
+      if (KM == 0 && has_sc) issue_scales((kt + 4) >> 2);
     }
-  } else {
-    // ping-pong (the reference's 8-wave pattern, analysis/bf16_gemm/mi325x/kernel_8192.cpp:75-153):
-    // waves 0-3 and waves 4-7 (one of each per SIMD) run half a K-tile out of phase, so that on
-    // every SIMD one wave issues MFMAs while the other reads LDS and issues the next loads.
-    // Barrier n is common to all waves; between barriers 2k and 2k+1 the first group is in its
-    // memory cluster for tile k, between 2k+1 and 2k+2 in its compute cluster; the second group
-    // does the same one barrier later.  A ring slot is refilled (tile k+2 over tile k-1) only after
-    // the barrier by which both groups have finished reading it, and each wave waits for its own
-    // share of tile k+1 before the barrier that precedes the first read of that tile.
-    constexpr int SCL = 1;  // scale loads per wave per slot that carries scales (8 waves)
-    auto wait_next_tile = [&](int kt) __attribute__((always_inline)) {
-      if (kt + 2 < nkt) {  // slot kt+2 was issued in this iteration and may stay in flight
-        if ((kt & 3) == 0 && kt + 4 < nkt) wait_vmcnt<2 * OPS + SCL>(); else wait_vmcnt<2 * OPS>();
+    read_tile(stage, ((kt >> 2) & 1) * kScaleBuf + KM * 4);
+    wait_lds_reads();  // this tile's LDS reads are done before anyone may refill its slot
+    auto wait_next = [&]() __attribute__((always_inline)) {  // own share of tile kt+1 has landed
+      if (has2) {
+        if (KM == 0 && has_sc) wait_vmcnt<2 * OPS + SCL>(); else wait_vmcnt<2 * OPS>();
       } else {
         wait_vmcnt<0>();
       }
     };
-    if (nkt > 1) wait_vmcnt_barrier<2 * OPS>(); else wait_vmcnt_barrier<0>();  // tile 0 landed everywhere
-    if (wm == 1) barrier_only();                                                // phase offset
-    for (int kt = 0; kt < nkt; kt++) {
-      if (kt + 2 < nkt && dev_mode != 1 && dev_mode < 4) issue_slot(kt + 2);
-      if (dev_mode < 2 || dev_mode == 5) read_tile(kt);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this tile's LDS reads are done before anyone may refill its slot
-      if (wm == 1) wait_next_tile(kt);
-      __builtin_amdgcn_sched_barrier(0);
-      barrier_only();
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_setprio(1);
-      if (dev_mode < 2 || dev_mode == 4) mma_tile();
-      __builtin_amdgcn_s_setprio(0);
-      if (wm == 0) wait_next_tile(kt);
-      __builtin_amdgcn_sched_barrier(0);
-      barrier_only();
-      __builtin_amdgcn_sched_barrier(0);
+    if (GRP == 1) wait_next();
+    barrier();
+    __builtin_amdgcn_s_setprio(1);
+    mma_tile();
+    __builtin_amdgcn_s_setprio(0);
+    if (GRP == 0) wait_next();
+    barrier();
+    stage = stage == kStages - 1 ? 0 : stage + 1;
+    stage2 = stage2 == kStages - 1 ? 0 : stage2 + 1;
+  };
+  auto k_loop = [&]<int GRP>() __attribute__((always_inline)) {
+    int kt = 0;
+    for (; kt + 8 <= nkt; kt += 4) {  // four tiles per trip, all of them with tiles kt+2 .. kt+7 in range
+      step.template operator()<GRP, 0, true>(kt);
+      step.template operator()<GRP, 1, true>(kt + 1);
+      step.template operator()<GRP, 2, true>(kt + 2);
+      step.template operator()<GRP, 3, true>(kt + 3);
     }
-    if (wm == 0) barrier_only();  // every wave executes the same number of barriers
+    for (; kt < nkt; kt += 4) {  // last (up to seven) tiles: same body with the range checks
+      step.template operator()<GRP, 0, false>(kt);
+      if (kt + 1 < nkt) step.template operator()<GRP, 1, false>(kt + 1);
+      if (kt + 2 < nkt) step.template operator()<GRP, 2, false>(kt + 2);
+      if (kt + 3 < nkt) step.template operator()<GRP, 3, false>(kt + 3);
+    }
+  };
+
+  // prologue: scales of the first four K-tiles, K-tiles 0 and 1; tile 0 must have landed everywhere
+  issue_scales(0);
+  issue_ops(0, 0);
+  if (nkt > 1) {
+    issue_ops(1, 1);
+    wait_vmcnt<2 * OPS>();
+  } else {
+    wait_vmcnt<0>();
+  }
+  barrier();
+  if (wm == 0) {
+    k_loop.template operator()<0>();
+    barrier();  // every wave executes the same number of barriers
+  } else {
+    barrier();  // phase offset of group 1
+    k_loop.template operator()<1>();
   }
 
   // ---- epilogue.  A lane owns C[m][n .. n+3] for four values of n per 32x32 tile, i.e. 8 bytes of
@@ -271,7 +284,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_tiled_kernel(const uint8_t* 
   // whole rows: one wave store = two rows x 512 contiguous bytes.
   if constexpr (sizeof(typename Out::type) == 2) {
     constexpr int kRowPitch = 512 + 16;  // bytes; the pad spreads the 32 rows of a store over the banks
-    static_assert(256 * kRowPitch <= (int)sizeof(smem), "C tile fits the ring");
+    static_assert(256 * kRowPitch <= kLdsBytes, "C tile fits the ring");
     __syncthreads();  // every wave is done reading the ring
     uint8_t* cs = smem + (wm * (TM * 32) + r32) * kRowPitch + (wn * (TN * 32) + 4 * h) * 2;
 #pragma unroll
@@ -310,20 +323,11 @@ bool gemm_tiled_supports(const GemmArgs& g) {
          (long)kBM * (g.K / 4 * 3) < (1L << 31) && ((uintptr_t)g.C % 16) == 0;
 }
 
-static int g_tiled_waves = 8;
-static int g_dev_mode = 0;
-static int g_sched = 1;
-void set_sched(int v) { g_sched = v; }
-void set_dev_mode(int m) { g_dev_mode = m; }
-void set_tiled_waves(int w) { g_tiled_waves = w; }
-
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int tm = g.M / kBM, tn = g.N / kBN;
-  if (g_tiled_waves == 4)
-    gemm_tiled_kernel<FA, FB, Out, 2, 2><<<tm * tn, 256, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0, g.layout_a, g.layout_b);
-  else
-    gemm_tiled_kernel<FA, FB, Out, 2, 4><<<tm * tn, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn, g_dev_mode, g_tiled_waves == 8 ? g_sched : 0, g.layout_a, g.layout_b);
+  gemm_tiled_kernel<FA, FB, Out><<<tm * tn, NW * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn,
+                                                            g.layout_a, g.layout_b);
   return hipGetLastError();
 }
 

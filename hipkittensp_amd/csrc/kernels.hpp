@@ -17,10 +17,6 @@ struct GemmArgs {
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
-void set_tiled_waves(int w);
-void set_dev_mode(int m);
-void set_skinny_dev(int v);
-void set_sched(int v);
 bool gemm_skinny_supports(const GemmArgs& g);
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);
