@@ -106,10 +106,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   const int h = lane >> 5, r32 = lane & 31;
 
   const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK;
-  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A + (size_t)pm * kBM * rowbytes, (uint32_t)kBM * rowbytes);
-  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)pn * kBN * rowbytes, (uint32_t)kBN * rowbytes);
-  const __amdgpu_buffer_rsrc_t rSA = make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)kBM * sbytes);
-  const __amdgpu_buffer_rsrc_t rSB = make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)kBN * sbytes);
+  // edge tiles: rows past M (or N) lie beyond the end of the buffer resource and read as zeros
+  const int rows_a = min(kBM, M - pm * kBM), rows_b = min(kBN, N - pn * kBN);
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+  const __amdgpu_buffer_rsrc_t rSA = make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)rows_a * sbytes);
+  const __amdgpu_buffer_rsrc_t rSB = make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)rows_b * sbytes);
 
   // per-lane global byte offsets of the OPS direct loads.  Load q = wave*OPS + i fills LDS bytes
   // [q*1024, q*1024 + 1024) of the operand tile.  Row-major operand: slot o holds piece
@@ -300,10 +302,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
     const int chunk = tid & 31, row0 = tid >> 5;  // 32 lanes cover one 512-byte row
     uint8_t* cg = reinterpret_cast<uint8_t*>(C) + ((size_t)pm * kBM + row0) * (size_t)N * 2 + (size_t)pn * kBN * 2 + chunk * 16;
     constexpr int kRowsPerPass = NW * 2;
+    const bool col_ok = chunk * 8 < rows_b;  // N % 8 == 0: a 16-byte piece is inside or outside as a whole
 #pragma unroll 4
     for (int r = 0; r < 256; r += kRowsPerPass) {
       const v4i v = *reinterpret_cast<const v4i*>(smem + (row0 + r) * kRowPitch + chunk * 16);
-      *reinterpret_cast<v4i*>(cg + (size_t)r * N * 2) = v;
+      if (col_ok && row0 + r < rows_a) *reinterpret_cast<v4i*>(cg + (size_t)r * N * 2) = v;
     }
   } else {
     typename Out::type* cbase = C + ((size_t)pm * kBM + wm * (TM * 32) + r32) * (size_t)N + (size_t)pn * kBN + wn * (TN * 32) + 4 * h;
@@ -313,19 +316,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
       for (int j = 0; j < TN; j++)
 #pragma unroll
         for (int g = 0; g < 4; g++)
-          store4(cbase + (size_t)i * 32 * N + j * 32 + 8 * g, acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                 acc[i][j][4 * g + 3]);
+          if (wm * (TM * 32) + i * 32 + r32 < rows_a && wn * (TN * 32) + j * 32 + 8 * g + 4 * h < rows_b)
+            store4(cbase + (size_t)i * 32 * N + j * 32 + 8 * g, acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                   acc[i][j][4 * g + 3]);
   }
 }
 
 bool gemm_tiled_supports(const GemmArgs& g) {
-  return g.M > 0 && g.N > 0 && g.K > 0 && g.M % kBM == 0 && g.N % kBN == 0 && g.K % kBK == 0 &&
-         (long)kBM * (g.K / 4 * 3) < (1L << 31) && ((uintptr_t)g.C % 16) == 0;
+  // any M; N % 8 keeps every 16-byte output piece whole and aligned; K in whole K-tiles
+  return g.M > 0 && g.N > 0 && g.K > 0 && g.N % 8 == 0 && g.K % kBK == 0 && (long)kBM * (g.K / 4 * 3) < (1L << 31) &&
+         ((uintptr_t)g.C % 16) == 0;
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  const int tm = g.M / kBM, tn = g.N / kBN;
+  const int tm = (g.M + kBM - 1) / kBM, tn = (g.N + kBN - 1) / kBN;
   gemm_tiled_kernel<FA, FB, Out><<<tm * tn, NW * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn,
                                                             g.layout_a, g.layout_b);
   return hipGetLastError();

@@ -128,7 +128,8 @@ def test_generic_kernel_any_shape(hk, M, N, K, fa, fb):
 
 
 # ------------------------------------------------------------------ tiled kernel
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (256, 512, 384), (512, 256, 1664), (768, 1024, 1024)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (256, 512, 384), (512, 256, 1664), (768, 1024, 1024),
+                                   (300, 264, 256), (257, 8, 128), (100, 1000, 384), (33, 520, 640), (1, 256, 128)])  # edge tiles too
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
 def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M * 3 + N + K, kind_a="laplace" if fa == 3 else "normal", kind_b="weights")
@@ -148,6 +149,10 @@ def test_forced_kernels_reject_shapes_they_cannot_take(hk):
     ap, asc, bp, bsc = operands(16, 64, 384, 2, 2, seed=1)
     with pytest.raises(RuntimeError, match="bad shape"):
         gemm(hk, ap, bp, asc, bsc, kernel=3)          # K % 512
+    check(gemm(hk, ap, bp, asc, bsc, kernel=0), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)  # automatic: tiled
+    ap, asc, bp, bsc = operands(40, 36, 96, 2, 2, seed=2)
+    with pytest.raises(RuntimeError, match="bad shape"):
+        gemm(hk, ap, bp, asc, bsc, kernel=2)          # N % 8, K % 128
     check(gemm(hk, ap, bp, asc, bsc, kernel=0), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)  # automatic: generic
 
 
@@ -178,7 +183,7 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
     assert np.array_equal(pt.cpu().numpy(), o.tile_operand(pr)) and np.array_equal(st.cpu().numpy(), sr)
 
 
-@pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (2, 256, 512, 640), (2, 512, 256, 2048), (3, 16, 128, 1024), (3, 7, 64, 512), (0, 32, 32, 128)])
+@pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (3, 16, 128, 1024), (3, 7, 64, 512), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
     if kernel == 3 and la == 1:
