@@ -32,9 +32,11 @@ sys.path.insert(0, ROOT)
 MFMA_PEAK_TFLOPS = 10066.0  # MI355X dense MXFP6: 256 CU x 4 SIMD x 4096 FLOP/clk x 2.4 GHz
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 PUBLISHED_FP6_8192 = 2861.52  # reference's own FP6 GEMM at 8192^3 on MI355X
-# HBM bytes per launch of the 8192^3 tiled kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a
-# copy kernel of known size (profiles/); None until that measurement exists.
-TILED_TRAFFIC_BYTES = None
+# Fabric bytes per launch (L2 fills + write-backs) from rocprofv3 FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the
+# factors calibrated on an elementwise kernel of known size in the same runs
+# (profiles/bench_gemm_tiled_8192_gemm_skinny_m16.md): tiled 8192^3 = 614 832 + 131 072 KiB, skinny cfg3 = 190 658 + 256 KiB.
+TILED_TRAFFIC_BYTES = (614832 + 131072) * 1024
+SKINNY_TRAFFIC_BYTES = (190658 + 256) * 1024
 
 
 def algorithmic_bytes(M, N, K):
@@ -60,23 +62,24 @@ def make_inputs(hk, torch, M, N, K, fmt_a, fmt_b, seed, sets, std_b=1.0):
 
 
 def timed_loop(hk, torch, inputs, C, steps, warmup, layout_a=0, layout_b=0):
-    """W untimed + K timed launches; returns (wall seconds for K steps, mean per-launch event ms)."""
+    """W untimed + K timed launches.  Returns (wall seconds for the K steps between two device
+    synchronisations, mean per-launch milliseconds from one pair of device events recorded on the
+    launch stream around the K back-to-back launches)."""
     n = len(inputs)
     for i in range(warmup):
         ap, bp, asc, bsc = inputs[i % n]
         hk.dispatch_micro(ap, bp, asc, bsc, C, layout_a=layout_a, layout_b=layout_b)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    e0.record()
     for i in range(steps):
         ap, bp, asc, bsc = inputs[i % n]
-        ev[i][0].record()
         hk.dispatch_micro(ap, bp, asc, bsc, C, layout_a=layout_a, layout_b=layout_b)
-        ev[i][1].record()
+    e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    per = [a.elapsed_time(b) for a, b in ev]
-    return wall, sum(per) / len(per), min(per)
+    return wall, e0.elapsed_time(e1) / steps
 
 
 def cpu_baseline(inputs, M_sample):
@@ -107,6 +110,7 @@ def main():
     p.add_argument("--warmup", type=int, default=100)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-rows", type=int, default=8192)
+    p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the tile-major extras (used for profiling one layout)")
     args = p.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU (a single-GPU operator; sharding is by N or M with no exchange). Run with --gpus 1.")
@@ -124,7 +128,7 @@ def main():
     M = N = K = 8192
     inputs = make_inputs(hk, torch, M, N, K, 2, 2, seed=1, sets=3)
     C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
-    wall, ev_ms, ev_min = timed_loop(hk, torch, inputs, C, args.steps, args.warmup)
+    wall, ev_ms = timed_loop(hk, torch, inputs, C, args.steps, args.warmup)
     flops = 2.0 * M * N * K
     ms_per_step = wall / args.steps * 1e3
     value = flops / (wall / args.steps) / 1e12
@@ -138,7 +142,6 @@ def main():
         "frac": achieved / MFMA_PEAK_TFLOPS,
         "traffic": TILED_TRAFFIC_BYTES,
         "launch_ms_mean": ev_ms,
-        "launch_ms_min": ev_min,
         "algorithmic_flops_per_launch": flops,
         "algorithmic_bytes_per_launch": algorithmic_bytes(M, N, K),
         "hbm_bound_ms": algorithmic_bytes(M, N, K) / (HBM_PEAK_GBS * 1e9) * 1e3,
@@ -150,16 +153,21 @@ def main():
 
     # same workload with both operands pre-arranged tile-major (MXFP6_LAYOUT_TILE): reported beside the
     # headline, never as `value` (configs[1] asks for row-major operands)
-    tinputs = [(hk.tile_operand(ap), hk.tile_operand(bp), asc, bsc) for ap, bp, asc, bsc in inputs]
-    del inputs
-    twall, tev_ms, tev_min = timed_loop(hk, torch, tinputs, C, args.steps, args.warmup, 1, 1)
-    tile_major = {
-        "what": "same 8192^3 workload, operands in tile-major layout (mxfp6_tile_operand / quantiser output)",
-        "value": flops / (twall / args.steps) / 1e12, "unit": "TFLOPS",
-        "achieved": flops / (tev_ms * 1e-3) / 1e12, "frac": flops / (tev_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
-        "launch_ms_mean": tev_ms, "launch_ms_min": tev_min,
-    }
-    del tinputs, C
+    tile_major = None
+    if args.layouts == "both":
+        tinputs = [(hk.tile_operand(ap), hk.tile_operand(bp), asc, bsc) for ap, bp, asc, bsc in inputs]
+        del inputs
+        twall, tev_ms = timed_loop(hk, torch, tinputs, C, args.steps, args.warmup, 1, 1)
+        tile_major = {
+            "what": "same 8192^3 workload, operands in tile-major layout (mxfp6_tile_operand / quantiser output)",
+            "value": flops / (twall / args.steps) / 1e12, "unit": "TFLOPS",
+            "achieved": flops / (tev_ms * 1e-3) / 1e12, "frac": flops / (tev_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
+            "launch_ms_mean": tev_ms,
+        }
+        del tinputs
+    else:
+        del inputs
+    del C
     torch.cuda.empty_cache()
 
     # ---- decode shape: configs[3], M=16, N=8192, K=28672, weights N(0, 0.02); five weight sets
@@ -167,12 +175,19 @@ def main():
     dM, dN, dK = 16, 8192, 28672
     dinputs = make_inputs(hk, torch, dM, dN, dK, 2, 2, seed=3, sets=5, std_b=0.02)
     dC = torch.empty(dM, dN, dtype=torch.bfloat16, device="cuda")
-    dwall, dev_ms, dev_min = timed_loop(hk, torch, dinputs, dC, args.steps, args.warmup)
+    dwall, dev_ms = timed_loop(hk, torch, dinputs, dC, args.steps, args.warmup)
     dbytes = algorithmic_bytes(dM, dN, dK)
     d_achieved = dbytes / (dev_ms * 1e-3) / 1e9
-    dtin = [(ap, hk.tile_operand(bp), asc, bsc) for ap, bp, asc, bsc in dinputs]
-    dtwall, dtev_ms, dtev_min = timed_loop(hk, torch, dtin, dC, args.steps, args.warmup, 0, 1)
-    del dtin
+    dtile = None
+    if args.layouts == "both":
+        dtin = [(ap, hk.tile_operand(bp), asc, bsc) for ap, bp, asc, bsc in dinputs]
+        dtwall, dtev_ms = timed_loop(hk, torch, dtin, dC, args.steps, args.warmup, 0, 1)
+        del dtin
+        dtile = {
+            "what": "same decode workload, weights (B) tile-major",
+            "achieved": dbytes / (dtev_ms * 1e-3) / 1e9, "unit": "GB/s", "frac": dbytes / (dtev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "launch_ms_mean": dtev_ms,
+        }
     decode = {
         "metric": "MXFP6 decode GEMM achieved GB/s @M=16,N=8192,K=28672",
         "value": dbytes / (dwall / args.steps) / 1e9,
@@ -185,16 +200,11 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": d_achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": SKINNY_TRAFFIC_BYTES,
             "launch_ms_mean": dev_ms,
-            "launch_ms_min": dev_min,
             "algorithmic_bytes_per_launch": dbytes,
         },
-        "tile_major_weights": {
-            "what": "same decode workload, weights (B) tile-major",
-            "achieved": dbytes / (dtev_ms * 1e-3) / 1e9, "unit": "GB/s", "frac": dbytes / (dtev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "launch_ms_mean": dtev_ms, "launch_ms_min": dtev_min,
-        },
+        "tile_major_weights": dtile,
     }
 
     line = {
