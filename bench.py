@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 
 MFMA_PEAK_TFLOPS = 10066.0  # MI355X dense MXFP6: 256 CU x 4 SIMD x 4096 FLOP/clk x 2.4 GHz
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
-PUBLISHED_FP6_8192 = 2861.52  # reference's own FP6 GEMM at 8192^3 on MI355X
+PUBLISHED_FP6_8192 = 2861.52  # reference's published FP6 GEMM at 8192^3 on MI355X (analysis/fp6_gemm/mi355x_fp6_gemm.json:5)
 # Fabric bytes per launch (L2 fills + write-backs) from rocprofv3 FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the
 # factors calibrated on an elementwise kernel of known size in the same runs
 # (profiles/bench_gemm_tiled_8192_gemm_skinny_m16.md): tiled 8192^3 = 614 832 + 131 072 KiB, skinny cfg3 = 190 658 + 256 KiB.
