@@ -30,9 +30,14 @@
 //
 // Schedule: 8-wave ping-pong (the reference's pattern, analysis/bf16_gemm/mi325x/kernel_8192.cpp:75-153):
 // waves 0-3 and waves 4-7 (one of each per SIMD) run half a K-tile out of phase, so that on every SIMD
-// one wave issues MFMAs while the other reads LDS and issues the next loads.  All waves are consumers
-// (the reference measures all-consumer above producer/consumer,
-// analysis/paper_experiments/producer_consumer_micro/plot.py:26-30).
+// one wave issues MFMAs while the other reads LDS.  All waves are consumers (the reference measures
+// all-consumer above producer/consumer, analysis/paper_experiments/producer_consumer_micro/plot.py:26-30).
+// The direct loads are split between the two clusters: a load issued while four waves queue theirs at the
+// same time stalls the wave for ~100 clocks (row-major operands; ~45 for contiguous ones), which is cheap
+// between two MFMAs and expensive in front of the LDS reads, so kLoadsInCompute of a tile's six loads per
+// wave ride in the compute cluster, one after every second MFMA, and the rest follow the LDS reads of the
+// memory cluster (measured: memory cluster 1110 -> 720 clocks, 7 % / 11 % less time per GEMM for
+// row-major / tile-major operands).
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -49,6 +54,8 @@ constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile 128 x 64
 constexpr int TM = 8 / WM, TN = 8 / WN;      // 32x32 MFMA tiles per wave in M and N
 constexpr int OPS = 24 / NW;                 // operand direct loads per wave per operand per K-tile
 constexpr int SCL = 1;                       // scale direct loads per wave per slot that carries scales
+constexpr int kLoadsInCompute = 4;           // of the 2*OPS operand loads per wave and K-tile: issued between MFMAs
+static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= 2 * OPS && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
 static_assert(kLdsBytes <= 163840, "LDS budget");
 
 // One direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff and the hardware
@@ -151,21 +158,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-  // ---- loads.  The issue slot of K-tile t holds its 2*OPS operand loads and, when t % 4 == 2, the
-  // scale load for the four K-tiles starting at t + 2 (at the end, so that a wait that leaves a
-  // whole slot in flight also covers the scales of the slot before).
+  // ---- loads.  A wave's batch for K-tile t is its 2*OPS operand loads (n = 0..OPS-1: A, then B) and,
+  // when t % 4 == 2, the scale load for the four K-tiles starting at t + 2 (at the end of the batch, so
+  // that a wait that leaves a whole batch in flight also covers the scales of the batch before).
   auto issue_scales = [&](int grp) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + (wave & 3) * 1024;
     const int soff = grp * 16;
     if (wave < 4) dma16(rSA, dst, voff_s, soff); else dma16(rSB, dst + kScStage, voff_s, soff);
   };
-  auto issue_ops = [&](int t, int stage) __attribute__((always_inline)) {
-    const uint32_t dst = lds0 + stage * kStage + wave * (OPS * 1024);
-    const int soff_a = t * kstep_a, soff_b = t * kstep_b;
+  auto issue_one = [&](int t, int slot, int n) __attribute__((always_inline)) {
+    const uint32_t dst = lds0 + slot * kStage + wave * (OPS * 1024);
+    if (n < OPS) dma16(rA, dst + n * 1024, voff_a[n], t * kstep_a);
+    else dma16(rB, dst + kOpStage + (n - OPS) * 1024, voff_b[n - OPS], t * kstep_b);
+  };
+  auto issue_ops = [&](int t, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < OPS; i++) dma16(rA, dst + i * 1024, voff_a[i], soff_a);
-#pragma unroll
-    for (int i = 0; i < OPS; i++) dma16(rB, dst + kOpStage + i * 1024, voff_b[i], soff_b);
+    for (int n = 0; n < 2 * OPS; n++) issue_one(t, slot, n);
   };
 
   // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
@@ -189,8 +197,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   };
   // first K-block of every lane for all tiles, then the second: two MFMAs into the same accumulator
   // are TM*TN instructions apart.  First source = B rows (index n), second = A rows (index m): a
-  // lane ends up owning 4 consecutive n of one m.
-  auto mma_tile = [&]() __attribute__((always_inline)) {
+  // lane ends up owning 4 consecutive n of one m.  between(i) runs after the i-th MFMA.
+  auto mma_tile = [&](auto&& between) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const v8i a0 = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, -1, -1);
@@ -198,6 +206,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
       for (int j = 0; j < TN; j++) {
         const v8i b0 = __builtin_shufflevector(fb[j][0], fb[j][1], 0, 1, 2, 3, 4, 5, -1, -1);
         acc[i][j] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[i][j], scb[j], sca[i]);
+        between(i * TN + j);
       }
     }
 #pragma unroll
@@ -207,28 +216,40 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
       for (int j = 0; j < TN; j++) {
         const v8i b1 = __builtin_shufflevector(fb[j][1], fb[j][2], 2, 3, 4, 5, 6, 7, -1, -1);
         acc[i][j] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[i][j], scb[j], sca[i]);
+        between(TM * TN + i * TN + j);
       }
     }
   };
 
   // ---- the K loop.  Barrier n is common to all waves; between barriers 2k and 2k+1 group 0 (waves
   // 0-3) is in its memory cluster for tile k and between 2k+1 and 2k+2 in its compute cluster; group 1
-  // (waves 4-7) does the same one barrier later.  A ring slot is refilled (tile k+2 over tile k-1)
-  // only after the barrier by which both groups have finished reading it, and each wave waits for
-  // its own share of tile k+1 before the barrier that precedes the first read of that tile.
+  // (waves 4-7) does the same one barrier later.  A ring slot is refilled only after the barrier by
+  // which both groups have finished reading it, and each wave waits for its own share of tile k+1
+  // before the barrier that precedes the first read of that tile.
+  // Loads of step k.  Memory cluster, after the LDS reads, both groups: loads kLoadsInCompute.. of tile
+  // k+2 (slot of tile k-1, free since barrier 2k) and the scales.  Compute cluster: loads
+  // 0..kLoadsInCompute-1, for group 0 of the same tile k+2, for group 1 of tile k+3, whose slot is the
+  // one of tile k: group 1's compute cluster starts at barrier 2k+2, by which both groups have read
+  // tile k.  In program order every tile's batch is contiguous for both groups, so one wait count
+  // serves both: everything older than the newest batch has landed.
   // The body is instantiated per group (GRP) and per k mod 4 (KM), so the steady state carries no
-  // branch: STEADY means tiles k+2 and (for the scales) k+4 exist.
+  // branch: STEADY means tiles k+2, k+3 and (for the scales) k+4 exist.
   int stage = 0, stage2 = 2;  // ring slots of tile k and tile k+2
   auto step = [&]<int GRP, int KM, bool STEADY>(int kt) __attribute__((always_inline)) {
-    const bool has2 = STEADY || kt + 2 < nkt;            // tile kt+2 exists
-    const bool has_sc = STEADY || kt + 4 < nkt;           // and so do the scales its slot would carry
+    constexpr int AHEAD = GRP == 0 ? 2 : 3;
+    const bool has2 = STEADY || kt + 2 < nkt;             // tile kt+2 exists
+    const bool hasx = STEADY || kt + AHEAD < nkt;         // the tile the compute-cluster loads belong to exists
+    const bool has_sc = STEADY || kt + 4 < nkt;           // the scales this step's batch would carry exist
+    const int slotx = GRP == 0 ? stage2 : stage;
+    read_tile(stage, ((kt >> 2) & 1) * kScaleBuf + KM * 4);
+    __builtin_amdgcn_sched_barrier(0);
     if (has2) {
-      issue_ops(kt + 2, stage2);
+#pragma unroll
+      for (int n = kLoadsInCompute; n < 2 * OPS; n++) issue_one(kt + 2, stage2, n);
       if (KM == 0 && has_sc) issue_scales((kt + 4) >> 2);
     }
-    read_tile(stage, ((kt >> 2) & 1) * kScaleBuf + KM * 4);
     wait_lds_reads();  // this tile's LDS reads are done before anyone may refill its slot
-    auto wait_next = [&]() __attribute__((always_inline)) {  // own share of tile kt+1 has landed
+    auto wait_next = [&]() __attribute__((always_inline)) {  // own share of tile kt+1 has landed; tile kt+2's batch may be in flight
       if (has2) {
         if (KM == 0 && has_sc) wait_vmcnt<2 * OPS + SCL>(); else wait_vmcnt<2 * OPS>();
       } else {
@@ -238,7 +259,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
     if (GRP == 1) wait_next();
     barrier();
     __builtin_amdgcn_s_setprio(1);
-    mma_tile();
+    mma_tile([&](int i) __attribute__((always_inline)) {
+      if (hasx && (i & 1) && i / 2 < kLoadsInCompute) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_one(kt + AHEAD, slotx, i / 2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
     __builtin_amdgcn_s_setprio(0);
     if (GRP == 0) wait_next();
     barrier();
@@ -261,11 +288,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
     }
   };
 
-  // prologue: scales of the first four K-tiles, K-tiles 0 and 1; tile 0 must have landed everywhere
+  // prologue: scales of the first four K-tiles, K-tiles 0 and 1 and, for group 1, the loads of tile 2
+  // that its compute cluster of "step -1" would have issued; tile 0 must have landed everywhere
   issue_scales(0);
   issue_ops(0, 0);
-  if (nkt > 1) {
-    issue_ops(1, 1);
+  if (nkt > 1) issue_ops(1, 1);
+  if (wm == 1 && nkt > 2 && kLoadsInCompute > 0) {
+#pragma unroll
+    for (int n = 0; n < kLoadsInCompute; n++) issue_one(2, 2, n);
+    wait_vmcnt<2 * OPS + kLoadsInCompute>();
+  } else if (nkt > 1) {
     wait_vmcnt<2 * OPS>();
   } else {
     wait_vmcnt<0>();
