@@ -5,6 +5,7 @@
 
 namespace mxfp6 {
 
+typedef int v12i __attribute__((ext_vector_type(12)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));

@@ -177,7 +177,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   };
 
   // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
-  v4i fa[TM][3], fb[TN][3];
+  // a lane's 48 bytes of one 32-row tile live in 12 consecutive VGPRs: dwords 0-5 are the operand of the
+  // first MFMA, 6-11 of the second
+  v12i fa[TM], fb[TN];
   int sca[TM], scb[TN];
   auto read_tile = [&](int stage, int sc_off) __attribute__((always_inline)) {
     const uint8_t* st = smem + stage * kStage;
@@ -185,13 +187,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
-      for (int c = 0; c < 3; c++) fb[j][c] = *reinterpret_cast<const v4i*>(st + b_rd[c] + j * 3072);
+      for (int c = 0; c < 3; c++) {
+        const v4i p = *reinterpret_cast<const v4i*>(st + b_rd[c] + j * 3072);
+#pragma unroll
+        for (int e = 0; e < 4; e++) fb[j][4 * c + e] = p[e];
+      }
       scb[j] = *reinterpret_cast<const uint16_t*>(sc + sb_rd + j * 512);
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
-      for (int c = 0; c < 3; c++) fa[i][c] = *reinterpret_cast<const v4i*>(st + a_rd[c] + i * 3072);
+      for (int c = 0; c < 3; c++) {
+        const v4i p = *reinterpret_cast<const v4i*>(st + a_rd[c] + i * 3072);
+#pragma unroll
+        for (int e = 0; e < 4; e++) fa[i][4 * c + e] = p[e];
+      }
       sca[i] = *reinterpret_cast<const uint16_t*>(sc + sa_rd + i * 512);
     }
   };
@@ -201,20 +211,20 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   auto mma_tile = [&](auto&& between) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      const v8i a0 = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, -1, -1);
+      const v8i a0 = __builtin_shufflevector(fa[i], fa[i], 0, 1, 2, 3, 4, 5, -1, -1);
 #pragma unroll
       for (int j = 0; j < TN; j++) {
-        const v8i b0 = __builtin_shufflevector(fb[j][0], fb[j][1], 0, 1, 2, 3, 4, 5, -1, -1);
+        const v8i b0 = __builtin_shufflevector(fb[j], fb[j], 0, 1, 2, 3, 4, 5, -1, -1);
         acc[i][j] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[i][j], scb[j], sca[i]);
         between(i * TN + j);
       }
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      const v8i a1 = __builtin_shufflevector(fa[i][1], fa[i][2], 2, 3, 4, 5, 6, 7, -1, -1);
+      const v8i a1 = __builtin_shufflevector(fa[i], fa[i], 6, 7, 8, 9, 10, 11, -1, -1);
 #pragma unroll
       for (int j = 0; j < TN; j++) {
-        const v8i b1 = __builtin_shufflevector(fb[j][1], fb[j][2], 2, 3, 4, 5, 6, 7, -1, -1);
+        const v8i b1 = __builtin_shufflevector(fb[j], fb[j], 6, 7, 8, 9, 10, 11, -1, -1);
         acc[i][j] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[i][j], scb[j], sca[i]);
         between(TM * TN + i * TN + j);
       }
@@ -249,6 +259,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
       if (KM == 0 && has_sc) issue_scales((kt + 4) >> 2);
     }
     wait_lds_reads();  // this tile's LDS reads are done before anyone may refill its slot
+    // the middle 16-byte piece straddles the two operands; naming each fragment as one 384-bit value here
+    // makes the register allocator keep it in one tuple, and the MFMAs read sub-tuples of it instead of
+    // copies (24 v_mov per K-tile otherwise)
+#pragma unroll
+    for (int i = 0; i < TM; i++) asm volatile("" : "+v"(fa[i]));
+#pragma unroll
+    for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
     auto wait_next = [&]() __attribute__((always_inline)) {  // own share of tile kt+1 has landed; tile kt+2's batch may be in flight
       if (has2) {
         if (KM == 0 && has_sc) wait_vmcnt<2 * OPS + SCL>(); else wait_vmcnt<2 * OPS>();
