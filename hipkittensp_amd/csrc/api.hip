@@ -95,6 +95,17 @@ int mxfp6_tile_operand(const void* src, void* dst, int rows, int K, int tile, vo
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
+int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, void* stream) {
+  if (rows < 0 || K < 0 || rows % 32 || K % 128) return MXFP6_EINVAL_SHAPE;
+  if (rows == 0 || K == 0) return MXFP6_OK;
+  if (!src || !dst) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)src & 3) || ((uintptr_t)dst & 3)) return MXFP6_EINVAL_ALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  hipError_t e = mxfp6::launch_tile_scales((const uint8_t*)src, (uint8_t*)dst, rows, K, tile, (hipStream_t)stream);
+  return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
 int mxfp6_set_kernel(int which) {
   if (which < 0 || which > 3) return g_force.load();
   return g_force.exchange(which);
@@ -133,7 +144,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 101; }
+int mxfp6_abi_version(void) { return 102; }
 
 #pragma GCC visibility pop
 }  // extern "C"

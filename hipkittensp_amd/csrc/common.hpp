@@ -64,4 +64,11 @@ __host__ __device__ __forceinline__ size_t tile_major_offset(int row, int b, int
   return ((size_t)(row >> 5) * nkt + kt) * 3072 + (size_t)((r * 6 + (c ^ ((r >> 3) & 1))) * 16 + (in & 15));
 }
 
+// Byte offset, inside tile-major scales, of the E8M0 byte of K-block kb (32 elements) of row `row`; nk4 =
+// ceil(K / 512).  The 16 scale bytes one row has for four K-tiles stay together, and the 32 rows of a row-tile
+// are adjacent: 512-byte chunk (rt, g) at ((rt * nk4) + g) * 512, row r of the tile at r * 16 inside it.
+__host__ __device__ __forceinline__ size_t tile_major_scale_offset(int row, int kb, int nk4) {
+  return ((size_t)(row >> 5) * nk4 + (kb >> 4)) * 512 + (size_t)((row & 31) * 16 + (kb & 15));
+}
+
 }  // namespace mxfp6

@@ -32,12 +32,12 @@ __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restr
     if (kv && mv) {
       for (int i = 0; i < 6; i++)
         a[i] = layout_a ? *reinterpret_cast<const int*>(A + tile_major_offset((int)m, kb * 24 + 4 * i, nkb / 4)) : (int)arow[kb * 6 + i];
-      sa = asr[kb];
+      sa = layout_a ? As[tile_major_scale_offset((int)m, kb, (nkb + 15) / 16)] : asr[kb];
     }
     if (kv && nv) {
       for (int i = 0; i < 6; i++)
         b[i] = layout_b ? *reinterpret_cast<const int*>(B + tile_major_offset((int)n, kb * 24 + 4 * i, nkb / 4)) : (int)brow[kb * 6 + i];
-      sb = bsr[kb];
+      sb = layout_b ? Bs[tile_major_scale_offset((int)n, kb, (nkb + 15) / 16)] : bsr[kb];
     }
     // rows of the first source index n (B), columns index m (A): each lane then owns 4 consecutive n
     acc = mfma_fp6<FB, FA, 0, 0>(b, a, acc, sb, sa);

@@ -67,7 +67,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   // rows that do not exist (n >= N, m >= M) lie past the end of the resource and read as zeros
   const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, (uint32_t)M * rowbytes);
-  const __amdgpu_buffer_rsrc_t rBs = make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
+  // tile-major B: this workgroup's 32 rows are one row-tile, whose scales are nk4 chunks of 512 bytes (row r at r * 16)
+  const int nk4 = (nkt + 3) / 4;
+  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)blockIdx.x * nk4 * 512, (uint32_t)nk4 * 512)
+                                              : make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
   const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * sbytes);
 
   // direct-load address map: LDS slot o (16 bytes) of a tile holds chunk (o%6) ^ ((row>>3)&1) of row o/6
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   int voff_bt[3];
 #pragma unroll
   for (int i = 0; i < 3; i++) voff_bt[i] = layout_b ? (i * 64 + lane) * 16 : voff[i];
-  const int voff_bs = r32 * sbytes, voff_as = (AR == 16 ? (r32 & 15) : r32) * sbytes;
+  const int voff_bs = layout_b ? r32 * 16 : r32 * sbytes, voff_as = (AR == 16 ? (r32 & 15) : r32) * sbytes;
 
   const uint32_t ring = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kRing;
   const uint8_t* ringp = smem + wave * kRing;
@@ -103,7 +106,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 
   auto issue_scales = [&](int chunk) {  // 16 scale bytes per row: the chunk's four K-tiles
     const int so = __builtin_amdgcn_readfirstlane(chunk * 16);
-    sc_b_next = load128_sk(rBs, voff_bs, so);
+    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * 512 : chunk * 16);
+    sc_b_next = load128_sk(rBs, voff_bs, sob);
     sc_a_next = load128_sk(rAs, voff_as, so);
   };
   auto issue_tile = [&](int chunk, int u) {  // K-tile u of a chunk into stage u

@@ -17,7 +17,8 @@
 // and r+8 would share banks, and every phase holds each (r mod 8) once with bit 3 clear and once set
 // (measured here: 199 B/clk/CU with the exchange, 126 without).
 // A tile-major operand (MXFP6_LAYOUT_TILE) is stored in global memory in exactly this order, which
-// turns every load into one contiguous KiB.
+// turns every load into one contiguous KiB; its scales are stored as the 512-byte chunks the scale
+// loads fetch (32 rows x 16 bytes), 4 cache lines per 32 rows instead of 32.
 //
 // MFMA operand mapping: lane l of a 32x32x64 MFMA supplies row l%32 and one 32-element K-block.  Lanes
 // 0-31 take K-blocks {0,1} of the K-tile and lanes 32-63 take K-blocks {2,3}: each lane reads its row's
@@ -117,8 +118,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   const int rows_a = min(kBM, M - pm * kBM), rows_b = min(kBN, N - pn * kBN);
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
   const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
-  const __amdgpu_buffer_rsrc_t rSA = make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)rows_a * sbytes);
-  const __amdgpu_buffer_rsrc_t rSB = make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)rows_b * sbytes);
+  // tile-major scales: the 16 bytes a row has for four K-tiles, 32 rows adjacent (512-byte chunks, nk4 per row-tile)
+  const int nk4 = (nkt + 3) / 4;
+  const __amdgpu_buffer_rsrc_t rSA = layout_a ? make_rsrc(As + (size_t)pm * (kBM / 32) * nk4 * 512, (uint32_t)((rows_a + 31) / 32) * nk4 * 512)
+                                              : make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)rows_a * sbytes);
+  const __amdgpu_buffer_rsrc_t rSB = layout_b ? make_rsrc(Bs + (size_t)pn * (kBN / 32) * nk4 * 512, (uint32_t)((rows_b + 31) / 32) * nk4 * 512)
+                                              : make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)rows_b * sbytes);
 
   // per-lane global byte offsets of the OPS direct loads.  Load q = wave*OPS + i fills LDS bytes
   // [q*1024, q*1024 + 1024) of the operand tile.  Row-major operand: slot o holds piece
@@ -137,7 +142,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   }
   const int kstep_a = layout_a ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
   // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; waves 0-3 load A's, 4-7 B's
-  const int voff_s = ((wave & 3) * 64 + lane) * sbytes;
+  const int srow = (wave & 3) * 64 + lane, slay = wave < 4 ? layout_a : layout_b;
+  const int voff_s = slay ? (srow >> 5) * nk4 * 512 + (srow & 31) * 16 : srow * sbytes;
+  const int sstep = slay ? 512 : 16;  // bytes between consecutive groups of four K-tiles
 
   // per-lane LDS read offsets (bytes from the start of a stage): the lane's three pieces 3h..3h+2
   const int sw = (r32 >> 3) & 1;
@@ -163,7 +170,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   // that a wait that leaves a whole batch in flight also covers the scales of the batch before).
   auto issue_scales = [&](int grp) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + (wave & 3) * 1024;
-    const int soff = grp * 16;
+    const int soff = grp * sstep;
     if (wave < 4) dma16(rSA, dst, voff_s, soff); else dma16(rSB, dst + kScStage, voff_s, soff);
   };
   auto issue_one = [&](int t, int slot, int n) __attribute__((always_inline)) {

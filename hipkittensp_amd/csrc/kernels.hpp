@@ -11,7 +11,7 @@ struct GemmArgs {
   int M, N, K;
   int fmt_a, fmt_b;  // 2 = e2m3, 3 = e3m2
   bool f32out;
-  int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (32 rows x 128 elements, LDS image order)
+  int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (operand: 32 rows x 128 elements in LDS image order; scales: 32 rows x 16 bytes)
 };
 
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
@@ -21,6 +21,7 @@ bool gemm_skinny_supports(const GemmArgs& g);
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);
 hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);
+hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);
 hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 
 }  // namespace mxfp6

@@ -88,6 +88,8 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
     const int row = (int)(b / nkb), kb = (int)(b - (long)row * nkb);
 #pragma unroll
     for (int i = 0; i < 6; i++) *reinterpret_cast<uint32_t*>(packed + tile_major_offset(row, kb * 24 + 4 * i, nkb / 4)) = w[i];
+    scales[tile_major_scale_offset(row, kb, (nkb + 15) / 16)] = (uint8_t)sb;
+    return;
   }
   scales[b] = (uint8_t)sb;
 }
@@ -119,6 +121,33 @@ hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K
   const long npieces = (long)rows * (K / 128) * 6;
   if (npieces == 0) return hipSuccess;
   tile_operand_kernel<<<(unsigned)((npieces + 255) / 256), 256, 0, s>>>(src, dst, npieces, K / 128, tile);
+  return hipGetLastError();
+}
+
+// scales [rows, K/32] row-major <-> tile-major: one lane moves the (up to) 16 bytes one row has for four K-tiles;
+// K-blocks past K (K % 512 != 0) are written as zero in the tile-major direction
+__global__ __launch_bounds__(256) void tile_scales_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, long nchunks,
+                                                         int nkb, int nk4, int tile) {
+  const long s = (long)blockIdx.x * 256 + threadIdx.x;
+  if (s >= nchunks) return;
+  const int row = (int)(s / nk4), g = (int)(s - (long)row * nk4);
+  const int nvalid = min(16, nkb - g * 16);  // a multiple of 4: K % 128 == 0
+  const size_t rm = (size_t)row * nkb + (size_t)g * 16, tm = tile_major_scale_offset(row, g * 16, nk4);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if (tile) {
+      *reinterpret_cast<uint32_t*>(dst + tm + 4 * i) = 4 * i < nvalid ? *reinterpret_cast<const uint32_t*>(src + rm + 4 * i) : 0u;
+    } else if (4 * i < nvalid) {
+      *reinterpret_cast<uint32_t*>(dst + rm + 4 * i) = *reinterpret_cast<const uint32_t*>(src + tm + 4 * i);
+    }
+  }
+}
+
+hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s) {
+  const int nkb = K / 32, nk4 = (nkb + 15) / 16;
+  const long nchunks = (long)rows * nk4;
+  if (nchunks == 0) return hipSuccess;
+  tile_scales_kernel<<<(unsigned)((nchunks + 255) / 256), 256, 0, s>>>(src, dst, nchunks, nkb, nk4, tile);
   return hipGetLastError();
 }
 

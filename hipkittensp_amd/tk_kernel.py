@@ -18,8 +18,10 @@ adds the checks a packed format needs (dtype, packed width, scale shape).
     C        bfloat16 [M, N]   (a float32 C receives the accumulators before the bf16 rounding)
     fmt_*    2 = e2m3, 3 = e3m2
     layout_* LAYOUT_ROW (as above) or LAYOUT_TILE: the same bytes regrouped into 32-row x 128-element
-             tiles in the kernels' LDS order (tile_operand() converts; quantize(..., layout=LAYOUT_TILE)
-             emits it directly); loads of a tile-major operand are contiguous
+             tiles in the kernels' LDS order, with the scales regrouped into 32-row x 16-byte chunks
+             (shape [rows, ceil(K/512) * 16]); tile_operand() / tile_scales() convert and
+             quantize(..., layout=LAYOUT_TILE) emits both directly; loads of a tile-major operand and
+             of its scales are contiguous
 
 PyTorch is used for tensor storage and the current stream only; the work is done by the HIP
 library behind include/mxfp6_gemm.h.
@@ -66,6 +68,11 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+def scale_width(K: int, layout: int = LAYOUT_ROW) -> int:
+    """Bytes of scales per row: K/32, or ceil(K/512) * 16 for tile-major scales."""
+    return K // 32 if layout == LAYOUT_ROW else (K + 511) // 512 * 16
+
+
 def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, layout_a: int = LAYOUT_ROW,
                    layout_b: int = LAYOUT_ROW) -> None:
     import torch
@@ -89,18 +96,18 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
     if wa % 24:
         raise RuntimeError(f"packed width {wa} is not a whole number of 32-element blocks (24 bytes each)")
     K = wa // 3 * 4
-    if _rows_cols(A_scale, "A_scale") != (M, K // 32):
-        raise RuntimeError(f"A_scale: expected shape [{M}, {K // 32}], got {tuple(A_scale.shape)}")
-    if _rows_cols(B_scale, "B_scale") != (N, K // 32):
-        raise RuntimeError(f"B_scale: expected shape [{N}, {K // 32}], got {tuple(B_scale.shape)}")
+    for rows, lay, name in ((M, layout_a, "A"), (N, layout_b, "B")):
+        if lay == LAYOUT_TILE and (rows % 32 or K % 128):
+            raise RuntimeError(f"{name}: a tile-major operand needs rows % 32 == 0 and K % 128 == 0")
+    for t, rows, lay, name in ((A_scale, M, layout_a, "A_scale"), (B_scale, N, layout_b, "B_scale")):
+        want = (rows, scale_width(K, lay))
+        if _rows_cols(t, name) != want:
+            raise RuntimeError(f"{name}: expected shape [{want[0]}, {want[1]}], got {tuple(t.shape)}")
     if _rows_cols(C, "C") != (M, N):
         raise RuntimeError(f"C: expected shape [{M}, {N}], got {tuple(C.shape)}")
     devs = {t.device for t in (A, B, A_scale, B_scale, C)}
     if len(devs) != 1:
         raise RuntimeError(f"all tensors must be on one device, got {sorted(map(str, devs))}")
-    for rows, lay, name in ((M, layout_a, "A"), (N, layout_b, "B")):
-        if lay == LAYOUT_TILE and (rows % 32 or K % 128):
-            raise RuntimeError(f"{name}: a tile-major operand needs rows % 32 == 0 and K % 128 == 0")
     L = _lib.lib()
     with torch.cuda.device(C.device):
         rc = L.mxfp6_gemm_ex(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
@@ -110,7 +117,8 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
 
 def quantize(X, fmt: int = E2M3, layout: int = LAYOUT_ROW):
     """fp32 [rows, K] on the GPU -> (packed uint8 [rows, 3K/4], scales uint8 [rows, K/32]).
-    With layout=LAYOUT_TILE the packed bytes are written tile-major (rows % 32 == 0, K % 128 == 0)."""
+    With layout=LAYOUT_TILE packed bytes and scales are written tile-major (rows % 32 == 0, K % 128 == 0;
+    scales [rows, ceil(K/512) * 16], padding zero)."""
     import torch
 
     X = _as_tensor(X, "X")
@@ -122,7 +130,11 @@ def quantize(X, fmt: int = E2M3, layout: int = LAYOUT_ROW):
     if K % 32:
         raise RuntimeError(f"K = {K} is not a multiple of 32")
     packed = torch.empty(*X.shape[:-1], K // 4 * 3, dtype=torch.uint8, device=X.device)
-    scales = torch.empty(*X.shape[:-1], K // 32, dtype=torch.uint8, device=X.device)
+    if layout not in (LAYOUT_ROW, LAYOUT_TILE):
+        raise RuntimeError("layout must be LAYOUT_ROW (0) or LAYOUT_TILE (1)")
+    sw = scale_width(K, layout)
+    alloc = torch.zeros if sw != K // 32 else torch.empty  # the quantiser does not write padding bytes
+    scales = alloc(*X.shape[:-1], sw, dtype=torch.uint8, device=X.device)
     with torch.cuda.device(X.device):
         rc = _lib.lib().mxfp6_quantize_ex(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, layout, _stream())
     _lib.check(rc, "quantize")
@@ -143,6 +155,26 @@ def tile_operand(packed, untile: bool = False):
     with torch.cuda.device(packed.device):
         rc = _lib.lib().mxfp6_tile_operand(packed.data_ptr(), out.data_ptr(), rows, w // 3 * 4, 0 if untile else 1, _stream())
     _lib.check(rc, "tile_operand")
+    return out
+
+
+def tile_scales(scales, K: int, untile: bool = False):
+    """Row-major scales [rows, K/32] -> tile-major [rows, ceil(K/512) * 16], or back (K = elements per row)."""
+    import torch
+
+    scales = _as_tensor(scales, "scales")
+    if scales.dtype != torch.uint8:
+        raise RuntimeError(f"scales: expected dtype uint8, got {scales.dtype}")
+    rows, w = _rows_cols(scales, "scales")
+    if K % 128 or rows % 32:
+        raise RuntimeError("tile-major layout needs rows % 32 == 0 and K % 128 == 0")
+    src_w, dst_w = (scale_width(K, LAYOUT_TILE), K // 32) if untile else (K // 32, scale_width(K, LAYOUT_TILE))
+    if w != src_w:
+        raise RuntimeError(f"scales: expected {src_w} bytes per row for K = {K}, got {w}")
+    out = torch.empty(*scales.shape[:-1], dst_w, dtype=torch.uint8, device=scales.device)
+    with torch.cuda.device(scales.device):
+        rc = _lib.lib().mxfp6_tile_scales(scales.data_ptr(), out.data_ptr(), rows, K, 0 if untile else 1, _stream())
+    _lib.check(rc, "tile_scales")
     return out
 
 

@@ -85,8 +85,13 @@ int mxfp6_quantize(const float *X, void *packed, void *scales, int rows, int K, 
  * of an operand are regrouped into tiles of 32 rows x 128 elements (3072 bytes), tile (rt, kt) at byte
  * ((rt * (K/128)) + kt) * 3072; inside a tile, the 16-byte piece c (0..5) of row r (0..31) sits at
  * (r*6 + (c ^ ((r >> 3) & 1))) * 16.  This is exactly the image the kernels keep in LDS, so their
- * direct-to-LDS loads become fully contiguous (one 1 KiB run per load instead of ~11 row pieces);
- * scale tensors are unchanged.  The reference applies its LDS swizzle to the global address of every
+ * direct-to-LDS loads become fully contiguous (one 1 KiB run per load instead of ~11 row pieces).
+ * The scales of a tile-major operand are tile-major too: the 16 scale bytes one row has for four K-tiles
+ * (512 elements) stay together and the 32 rows of a row-tile are adjacent, i.e. 512-byte chunk (rt, g) at
+ * ((rt * nk4) + g) * 512 with nk4 = ceil(K / 512), the byte of K-block kb of row r at (r % 32) * 16 + kb % 16
+ * inside chunk (r / 32, kb / 16).  The scale tensor then holds rows * nk4 * 16 bytes (= rows * K/32 when
+ * K % 512 == 0; the bytes of K-blocks past K are padding).  A kernel's scale load of 32 rows is 4 cache
+ * lines instead of 32.  The reference applies its LDS swizzle to the global address of every
  * load (include/ops/warp/memory/tile/global_to_shared.cuh:46-59); this applies it to the data once,
  * which suits weights (converted offline) and activations (the quantiser can emit it directly).
  */
@@ -97,15 +102,24 @@ int mxfp6_quantize(const float *X, void *packed, void *scales, int rows, int K, 
 int mxfp6_tile_operand(const void *src, void *dst, int rows, int K, int tile, void *hip_stream);
 
 /*
+ * Scales [rows, K/32] row-major -> tile-major (tile != 0; rows * ceil(K/512) * 16 bytes, padding written as 0)
+ * or back (tile == 0); rows % 32 == 0, K % 128 == 0; src and dst must not overlap.  No counterpart in the
+ * reference (its operands carry no scales); part of the tile-major operand format above.
+ */
+int mxfp6_tile_scales(const void *src, void *dst, int rows, int K, int tile, void *hip_stream);
+
+/*
  * mxfp6_gemm / mxfp6_gemm_f32out with a layout per operand (MXFP6_LAYOUT_*) and out_f32 != 0 for
  * the fp32 output.  With both layouts MXFP6_LAYOUT_ROW it is exactly those two entry points.
- * A tile-major operand needs rows % 32 == 0 and K % 128 == 0 (MXFP6_EINVAL_SHAPE otherwise).
+ * A tile-major operand comes with tile-major scales and needs rows % 32 == 0 and K % 128 == 0
+ * (MXFP6_EINVAL_SHAPE otherwise).
  */
 int mxfp6_gemm_ex(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, void *C,
                   int M, int N, int K, int fmt_a, int fmt_b, int layout_a, int layout_b, int out_f32,
                   void *hip_stream);
 
-/* mxfp6_quantize writing the packed operand in the given layout (scales are always [rows, K/32]). */
+/* mxfp6_quantize writing the packed operand and its scales in the given layout (tile-major scales: rows *
+ * ceil(K/512) * 16 bytes, of which the padding bytes are not written). */
 int mxfp6_quantize_ex(const float *X, void *packed, void *scales, int rows, int K, int fmt, int layout,
                       void *hip_stream);
 

@@ -173,6 +173,22 @@ def tile_operand(packed: np.ndarray) -> np.ndarray:
     return out.reshape(rows, w)
 
 
+def tile_scales(scales: np.ndarray) -> np.ndarray:
+    """Row-major scales [rows, K/32] -> tile-major [rows, nk4 * 16] (nk4 = ceil(K/512)): the 16 bytes a row has
+    for four K-tiles stay together, the 32 rows of a row-tile are adjacent: chunk (rt, g) of 512 bytes at
+    ((rt * nk4) + g) * 512, row r at (r % 32) * 16 inside it; K-blocks past K are zero.  Defines the scale half of
+    MXFP6_LAYOUT_TILE (include/mxfp6_gemm.h) independently of the GPU converter."""
+    s = np.asarray(scales, dtype=np.uint8)
+    rows, nkb = s.shape
+    if rows % 32 or nkb % 4:
+        raise ValueError("rows % 32 == 0 and K % 128 == 0 required")
+    nk4 = (nkb + 15) // 16
+    padded = np.zeros((rows, nk4 * 16), dtype=np.uint8)
+    padded[:, :nkb] = s
+    x = padded.reshape(rows // 32, 32, nk4, 16)           # [rt, r, g, byte]
+    return np.ascontiguousarray(x.transpose(0, 2, 1, 3)).reshape(rows, nk4 * 16)
+
+
 def dequantise(packed: np.ndarray, scales: np.ndarray, fmt: int, dtype=np.float32) -> np.ndarray:
     """packed [rows, 3K/4] + scales [rows, K/32] -> values [rows, K] = table[code] * 2^(scale-127).
     Exact in fp32 whenever the result is a normal fp32 number."""

@@ -30,7 +30,7 @@ def built_lib():
 
 def test_header_declares_the_operator():
     names = _declared_functions()
-    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_tile_operand",
+    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_tile_operand", "mxfp6_tile_scales",
                  "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel"):
         assert want in names
 
@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 101
+    assert L.mxfp6_abi_version() == 102
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -85,6 +85,11 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     L.mxfp6_tile_operand.argtypes = [vp, vp, ci, ci, ci, vp]
     assert L.mxfp6_tile_operand(one, one, 33, 128, 1, None) == -2
     assert L.mxfp6_tile_operand(one, None, 32, 128, 1, None) == -1
+    L.mxfp6_tile_scales.restype = ci
+    L.mxfp6_tile_scales.argtypes = [vp, vp, ci, ci, ci, vp]
+    assert L.mxfp6_tile_scales(one, one, 32, 96, 1, None) == -2
+    assert L.mxfp6_tile_scales(None, one, 32, 128, 1, None) == -1
+    assert L.mxfp6_tile_scales(one, one, 0, 128, 1, None) == 0
 
 
 def test_python_operator_rejects_like_the_reference():

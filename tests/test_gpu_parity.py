@@ -169,7 +169,7 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
 
 
 # ------------------------------------------------------------------ tile-major operand layout
-@pytest.mark.parametrize("rows,K", [(32, 128), (64, 512), (256, 1152), (96, 8192)])
+@pytest.mark.parametrize("rows,K", [(32, 128), (64, 512), (256, 1152), (96, 8192), (64, 640)])
 def test_tile_operand_matches_format_definition(hk, rows, K):
     rng = np.random.default_rng(rows + K)
     p = rng.integers(0, 256, size=(rows, K // 4 * 3), dtype=np.uint8)
@@ -180,10 +180,14 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
     x = o.make_source("normal", (rows, K), rng)
     pt, st = hk.quantize(dev(x), 2, layout=hk.LAYOUT_TILE)                          # quantiser emitting it directly
     pr, sr = co.quantise(x, 2)
-    assert np.array_equal(pt.cpu().numpy(), o.tile_operand(pr)) and np.array_equal(st.cpu().numpy(), sr)
+    assert np.array_equal(pt.cpu().numpy(), o.tile_operand(pr)) and np.array_equal(st.cpu().numpy(), o.tile_scales(sr))
+    ts = hk.tile_scales(dev(sr), K)                                                 # scale converter, both ways
+    assert np.array_equal(ts.cpu().numpy(), o.tile_scales(sr))
+    assert np.array_equal(hk.tile_scales(ts, K, untile=True).cpu().numpy(), sr)
 
 
-@pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (3, 16, 128, 1024), (3, 7, 64, 512), (0, 32, 32, 128)])
+@pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
+                                          (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
     if kernel == 3 and la == 1:
@@ -195,10 +199,12 @@ def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb)
     ref = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel)
     A = hk.tile_operand(dev(ap)) if la else dev(ap)
     B = hk.tile_operand(dev(bp)) if lb else dev(bp)
+    As = hk.tile_scales(dev(asc), K) if la else dev(asc)
+    Bs = hk.tile_scales(dev(bsc), K) if lb else dev(bsc)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     prev = hk.tk_kernel.set_kernel(kernel)
     try:
-        hk.dispatch_micro(A, B, dev(asc), dev(bsc), C, fa, fb, layout_a=la, layout_b=lb)
+        hk.dispatch_micro(A, B, As, Bs, C, fa, fb, layout_a=la, layout_b=lb)
         torch.cuda.synchronize()
     finally:
         hk.tk_kernel.set_kernel(prev)
@@ -222,7 +228,7 @@ def test_cfg1_and_cfg3_tile_major_full_size(hk):
     C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     Ct = torch.empty_like(C)
     hk.dispatch_micro(dA, dB, dAs, dBs, C)
-    hk.dispatch_micro(hk.tile_operand(dA), hk.tile_operand(dB), dAs, dBs, Ct, layout_a=1, layout_b=1)
+    hk.dispatch_micro(hk.tile_operand(dA), hk.tile_operand(dB), hk.tile_scales(dAs, K), hk.tile_scales(dBs, K), Ct, layout_a=1, layout_b=1)
     assert torch.equal(C, Ct)
     del dA, dB, C, Ct
     M, N, K = 16, 8192, 28672
@@ -231,7 +237,7 @@ def test_cfg1_and_cfg3_tile_major_full_size(hk):
     C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     Ct = torch.empty_like(C)
     hk.dispatch_micro(dA, dB, dAs, dBs, C)
-    hk.dispatch_micro(dA, hk.tile_operand(dB), dAs, dBs, Ct, layout_b=1)
+    hk.dispatch_micro(dA, hk.tile_operand(dB), dAs, hk.tile_scales(dBs, K), Ct, layout_b=1)
     torch.cuda.synchronize()
     assert torch.equal(C, Ct)
 

@@ -177,6 +177,24 @@ def test_tile_major_layout_definition():
     assert sorted(tq.reshape(-1).tolist()) == sorted(q.reshape(-1).tolist())
 
 
+def test_tile_major_scale_layout_definition():
+    # hand-checked placements: 64 rows, K = 1152 (36 K-blocks -> nk4 = 3 chunks per row-tile, last one a quarter full)
+    s = np.zeros((64, 36), np.uint8)
+    s[0, 0] = 1       # row-tile 0, chunk 0, row 0, byte 0 -> 0
+    s[5, 17] = 2      # chunk 1 (blocks 16..31), row 5, byte 1 -> 512 + 5*16 + 1
+    s[40, 35] = 3     # row-tile 1 (chunks 3..5), chunk 2, row 8, byte 3 -> (3 + 2)*512 + 8*16 + 3
+    t = o.tile_scales(s)
+    assert t.shape == (64, 48)
+    f = t.reshape(-1)
+    assert f[0] == 1 and f[512 + 81] == 2 and f[5 * 512 + 131] == 3 and int(f.astype(np.int64).sum()) == 6
+    rng = np.random.default_rng(2)
+    q = rng.integers(1, 256, size=(96, 32), dtype=np.uint8)   # K = 1024: a pure permutation
+    tq = o.tile_scales(q)
+    assert tq.shape == q.shape and sorted(tq.reshape(-1).tolist()) == sorted(q.reshape(-1).tolist())
+    # the 16 bytes of one row and one group of four K-tiles stay contiguous
+    assert np.array_equal(tq.reshape(-1)[(1 * 2 + 1) * 512 + 7 * 16:(1 * 2 + 1) * 512 + 8 * 16], q[39, 16:32])
+
+
 # ------------------------------------------------------------------ numpy vs C, end to end
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("kind", ["normal", "weights_outliers", "laplace"])
