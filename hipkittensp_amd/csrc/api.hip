@@ -54,8 +54,13 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 3) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_skinny(g, s);
+  } else if (force == 4) {
+    if (!mxfp6::gemm_mid_supports(g)) return MXFP6_EINVAL_SHAPE;
+    e = mxfp6::launch_gemm_mid(g, s);
   } else if (mxfp6::gemm_skinny_supports(g)) {
     e = mxfp6::launch_gemm_skinny(g, s);
+  } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
+    e = mxfp6::launch_gemm_mid(g, s);
   } else if (mxfp6::gemm_tiled_supports(g)) {
     e = mxfp6::launch_gemm_tiled(g, s);
   } else {
@@ -107,7 +112,7 @@ int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, voi
 }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 3) return g_force.load();
+  if (which < 0 || which > 4) return g_force.load();
   return g_force.exchange(which);
 }
 

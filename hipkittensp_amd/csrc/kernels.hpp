@@ -17,6 +17,9 @@ struct GemmArgs {
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
+bool gemm_mid_supports(const GemmArgs& g);
+bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the 256x256 tiling
+hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);

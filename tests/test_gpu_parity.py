@@ -168,6 +168,30 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
+# ------------------------------------------------------------------ mid-M kernel
+@pytest.mark.parametrize("M,N,K", [(33, 32, 1024), (64, 64, 1024), (48, 100, 2048), (64, 520, 3072), (65, 40, 1024), (128, 96, 4096), (100, 33, 2048),
+                                   (200, 72, 1024), (256, 160, 5120), (129, 31, 3072)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3)])
+def test_mid_kernel_vs_oracle(hk, M, N, K, fa, fb):
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + 2 * N + K, kind_a="laplace", kind_b="weights_outliers")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=4)
+    check(got, ref, fa, fb, ap, asc, bp, bsc)
+    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=4)
+    assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+
+
+def test_mid_kernel_is_chosen_and_rejects_other_shapes(hk):
+    # few 256x256 tiles, K in whole B slots: the automatic choice is the mid kernel and agrees with the forced one bit for bit
+    ap, asc, bp, bsc = operands(96, 288, 2048, 2, 2, seed=9, kind_b="weights")
+    assert np.array_equal(gemm(hk, ap, bp, asc, bsc, kernel=0), gemm(hk, ap, bp, asc, bsc, kernel=4))
+    check(gemm(hk, ap, bp, asc, bsc, kernel=4), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)
+    for M, N, K in ((32, 64, 1024), (300, 64, 1024), (64, 64, 1536)):   # M <= 32, M > 256, K % 1024
+        ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=5)
+        with pytest.raises(RuntimeError, match="bad shape"):
+            gemm(hk, ap, bp, asc, bsc, kernel=4)
+
+
 # ------------------------------------------------------------------ tile-major operand layout
 @pytest.mark.parametrize("rows,K", [(32, 128), (64, 512), (256, 1152), (96, 8192), (64, 640)])
 def test_tile_operand_matches_format_definition(hk, rows, K):
@@ -187,11 +211,11 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
 
 
 @pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
-                                          (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (0, 32, 32, 128)])
+                                          (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
-    if kernel == 3 and la == 1:
-        pytest.skip("the skinny kernel takes a row-major A (M need not be a multiple of 32)")
+    if kernel in (3, 4) and la == 1:
+        pytest.skip("the skinny and mid-M kernels take a row-major A (M need not be a multiple of 32)")
     fa, fb = 3, 2
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + N + K + la, kind_a="laplace", kind_b="weights")
     if la == 1 and M % 32:
