@@ -41,6 +41,8 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_quantize_ex.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.mxfp6_tile_operand.restype = ci
         L.mxfp6_tile_operand.argtypes = [vp, vp, ci, ci, ci, vp]
+        L.mxfp6_set_relayout.restype = ci
+        L.mxfp6_set_relayout.argtypes = [ci]
         L.mxfp6_tile_scales.restype = ci
         L.mxfp6_tile_scales.argtypes = [vp, vp, ci, ci, ci, vp]
         L.mxfp6_set_kernel.restype = ci

@@ -1,5 +1,6 @@
 // C ABI of the MXFP6 GEMM library (declared in include/mxfp6_gemm.h): argument validation and
-// kernel selection.  Nothing here allocates or synchronises.
+// kernel selection.  Nothing here synchronises; the only allocation is the stream-ordered workspace of the
+// re-layout pre-pass (relayout_then_tiled), which mxfp6_set_relayout(0) switches off.
 #include "../../include/mxfp6_gemm.h"
 
 #include <atomic>
@@ -9,6 +10,7 @@
 namespace {
 
 std::atomic<int> g_force{0};
+std::atomic<int> g_relayout{1};
 
 int check_device() {
   // cached per process: the library only carries gfx950 code objects
@@ -20,6 +22,42 @@ int check_device() {
     return __builtin_strncmp(p.gcnArchName, "gfx950", 6) == 0 ? MXFP6_OK : MXFP6_ENODEVICE;
   }();
   return cached;
+}
+
+// Large row-major problems on the tiled kernel are bound by L2 request throughput: a 96-byte row piece straddles
+// 128-byte lines and every row's scales are a request of their own (896 requests per K-tile and workgroup against
+// 648 with one operand tile-major).  Re-laying ONE operand (the one with fewer rows) out tile-major first costs
+// two passes over it at HBM speed and saves more than that from about 8192^3 on (measured there: 21 us of
+// pre-pass, 50 us less GEMM).  The workspace comes from the stream-ordered allocator and is returned to it on the
+// same stream right after the GEMM has been enqueued.  Returns false when the pre-pass does not pay or cannot
+// run (then the caller launches the row-major path).
+bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
+  if (!g_relayout.load(std::memory_order_relaxed) || g.layout_a || g.layout_b || g.K % 128) return false;
+  const bool a_ok = g.M % 32 == 0, b_ok = g.N % 32 == 0;
+  if (!a_ok && !b_ok) return false;
+  const bool pick_a = a_ok && (!b_ok || g.M <= g.N);
+  const int rows = pick_a ? g.M : g.N;
+  const double tiles = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
+  const double t_gemm_us = (tiles > 256 ? tiles / 256 : 1.0) * (g.K / 128) * 1.5;      // row-major tiled kernel
+  const double t_pre_us = (double)rows * g.K * 0.78125 * 2 / 4.9e6;                   // read + write at 4.9 TB/s
+  if (0.12 * t_gemm_us < 1.5 * t_pre_us) return false;
+  const size_t pbytes = (size_t)rows * (g.K / 4 * 3), sbytes = (size_t)rows * ((g.K + 511) / 512) * 16;
+  const size_t poff = (pbytes + 255) & ~(size_t)255;
+  uint8_t* ws = nullptr;
+  if (hipMallocAsync((void**)&ws, poff + sbytes, s) != hipSuccess || !ws) {
+    (void)hipGetLastError();
+    return false;
+  }
+  e = mxfp6::launch_tile_operand(pick_a ? g.A : g.B, ws, rows, g.K, 1, s);
+  if (e == hipSuccess) e = mxfp6::launch_tile_scales(pick_a ? g.As : g.Bs, ws + poff, rows, g.K, 1, s);
+  if (e == hipSuccess) {
+    mxfp6::GemmArgs t = g;
+    if (pick_a) { t.A = ws; t.As = ws + poff; t.layout_a = 1; } else { t.B = ws; t.Bs = ws + poff; t.layout_b = 1; }
+    e = mxfp6::launch_gemm_tiled(t, s);
+  }
+  const hipError_t fe = hipFreeAsync(ws, s);
+  if (e == hipSuccess) e = fe;
+  return true;
 }
 
 int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
@@ -62,7 +100,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
     e = mxfp6::launch_gemm_mid(g, s);
   } else if (mxfp6::gemm_tiled_supports(g)) {
-    e = mxfp6::launch_gemm_tiled(g, s);
+    if (!relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
   } else {
     e = mxfp6::launch_gemm_generic(g, s);
   }
@@ -111,6 +149,8 @@ int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, voi
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
+int mxfp6_set_relayout(int on) { return g_relayout.exchange(on ? 1 : 0); }
+
 int mxfp6_set_kernel(int which) {
   if (which < 0 || which > 4) return g_force.load();
   return g_force.exchange(which);
@@ -149,7 +189,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 102; }
+int mxfp6_abi_version(void) { return 103; }
 
 #pragma GCC visibility pop
 }  // extern "C"

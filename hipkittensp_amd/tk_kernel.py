@@ -178,6 +178,11 @@ def tile_scales(scales, K: int, untile: bool = False):
     return out
 
 
+def set_relayout(on: bool) -> bool:
+    """Switch the re-layout pre-pass of large row-major GEMMs on / off; returns the previous setting."""
+    return bool(_lib.lib().mxfp6_set_relayout(1 if on else 0))
+
+
 def set_kernel(which: int) -> int:
     """Force a kernel (KERNEL_*) for measurement / tests; returns the previous setting."""
     return _lib.lib().mxfp6_set_kernel(int(which))

@@ -73,6 +73,16 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
 int mxfp6_set_kernel(int which);
 
 /*
+ * Re-layout pre-pass of the automatic path (on by default; returns the previous setting).  For large row-major
+ * problems the gemm calls first copy the operand with fewer rows (and its scales) into tile-major order in a
+ * workspace taken from, and returned to, the stream-ordered allocator (hipMallocAsync / hipFreeAsync on the
+ * caller's stream), because the tiled kernel is bound by L2 requests on row-major operands; results are
+ * bit-identical.  Switch it off to measure the row-major kernel itself or where the caller cannot tolerate an
+ * allocation (e.g. stream capture).  No counterpart in the reference.
+ */
+int mxfp6_set_relayout(int on);
+
+/*
  * Quantise + pack on the GPU: X [rows, K] fp32 row-major -> packed [rows, 3K/4] u8 + scales
  * [rows, K/32] u8, scale = 2^(floor(log2(blockmax)) - emax(fmt)) (emax 2 for e2m3, 4 for e3m2),
  * round-to-nearest-even, saturating; an all-zero block gets scale byte 0.  K % 32 == 0.

@@ -254,6 +254,14 @@ def test_cfg1_and_cfg3_tile_major_full_size(hk):
     hk.dispatch_micro(dA, dB, dAs, dBs, C)
     hk.dispatch_micro(hk.tile_operand(dA), hk.tile_operand(dB), hk.tile_scales(dAs, K), hk.tile_scales(dBs, K), Ct, layout_a=1, layout_b=1)
     assert torch.equal(C, Ct)
+    prev = hk.tk_kernel.set_relayout(False)     # the row-major kernel itself, without the re-layout pre-pass of this size
+    try:
+        assert prev is True
+        Ct.zero_()
+        hk.dispatch_micro(dA, dB, dAs, dBs, Ct)
+        assert torch.equal(C, Ct)
+    finally:
+        hk.tk_kernel.set_relayout(prev)
     del dA, dB, C, Ct
     M, N, K = 16, 8192, 28672
     ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=3, kind_b="weights")
