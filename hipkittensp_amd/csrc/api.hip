@@ -26,35 +26,46 @@ int check_device() {
 
 // Large row-major problems on the tiled kernel are bound by L2 request throughput: a 96-byte row piece straddles
 // 128-byte lines and every row's scales are a request of their own (896 requests per K-tile and workgroup against
-// 648 with one operand tile-major).  Re-laying ONE operand (the one with fewer rows) out tile-major first costs
-// two passes over it at HBM speed and saves more than that from about 8192^3 on (measured there: 21 us of
-// pre-pass, 50 us less GEMM).  The workspace comes from the stream-ordered allocator and is returned to it on the
-// same stream right after the GEMM has been enqueued.  Returns false when the pre-pass does not pay or cannot
-// run (then the caller launches the row-major path).
+// 648 with one operand tile-major and 400 with both).  Re-laying an operand out tile-major first costs two passes
+// over it at HBM speed (measured 23 us for 8192 x 8192) and shortens the GEMM by about 15 % (first operand) and
+// 11 % (second): from about 8192^3 on that pays for both, for a tall or wide problem only for the operand with
+// fewer rows.  The workspace comes from the stream-ordered allocator and is returned to it on the same stream
+// right after the GEMM has been enqueued.  Returns false when no pre-pass pays or it cannot run (then the caller
+// launches the row-major path).
 bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
   if (!g_relayout.load(std::memory_order_relaxed) || g.layout_a || g.layout_b || g.K % 128) return false;
-  const bool a_ok = g.M % 32 == 0, b_ok = g.N % 32 == 0;
-  if (!a_ok && !b_ok) return false;
-  const bool pick_a = a_ok && (!b_ok || g.M <= g.N);
-  const int rows = pick_a ? g.M : g.N;
   const double tiles = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  const double t_gemm_us = (tiles > 256 ? tiles / 256 : 1.0) * (g.K / 128) * 1.5;      // row-major tiled kernel
-  const double t_pre_us = (double)rows * g.K * 0.78125 * 2 / 4.9e6;                   // read + write at 4.9 TB/s
-  if (0.12 * t_gemm_us < 1.5 * t_pre_us) return false;
-  const size_t pbytes = (size_t)rows * (g.K / 4 * 3), sbytes = (size_t)rows * ((g.K + 511) / 512) * 16;
-  const size_t poff = (pbytes + 255) & ~(size_t)255;
+  const double t_gemm_us = (tiles > 256 ? tiles / 256 : 1.0) * (g.K / 128) * 1.5;            // row-major tiled kernel
+  auto cost_us = [&](int rows) { return (double)rows * g.K * 0.78125 * 2 / 4.9e6; };         // read + write at 4.9 TB/s
+  // the operand with fewer rows first (it is the cheaper one to convert; the gain is the same)
+  const bool a_first = g.M <= g.N;
+  const int rows1 = a_first ? g.M : g.N, rows2 = a_first ? g.N : g.M;
+  bool conv1 = rows1 % 32 == 0 && 0.15 * t_gemm_us > 1.5 * cost_us(rows1);
+  bool conv2 = rows2 % 32 == 0 && (conv1 ? 0.11 : 0.15) * t_gemm_us > 1.5 * cost_us(rows2);
+  if (!conv1 && !conv2) return false;
+  const bool conv_a = a_first ? conv1 : conv2, conv_b = a_first ? conv2 : conv1;
+  auto bytes_of = [&](int rows) { return (((size_t)rows * (g.K / 4 * 3) + 255) & ~(size_t)255) + (((size_t)rows * ((g.K + 511) / 512) * 16 + 255) & ~(size_t)255); };
+  const size_t bytes_a = conv_a ? bytes_of(g.M) : 0, bytes_b = conv_b ? bytes_of(g.N) : 0;
   uint8_t* ws = nullptr;
-  if (hipMallocAsync((void**)&ws, poff + sbytes, s) != hipSuccess || !ws) {
+  if (hipMallocAsync((void**)&ws, bytes_a + bytes_b, s) != hipSuccess || !ws) {
     (void)hipGetLastError();
     return false;
   }
-  e = mxfp6::launch_tile_operand(pick_a ? g.A : g.B, ws, rows, g.K, 1, s);
-  if (e == hipSuccess) e = mxfp6::launch_tile_scales(pick_a ? g.As : g.Bs, ws + poff, rows, g.K, 1, s);
-  if (e == hipSuccess) {
-    mxfp6::GemmArgs t = g;
-    if (pick_a) { t.A = ws; t.As = ws + poff; t.layout_a = 1; } else { t.B = ws; t.Bs = ws + poff; t.layout_b = 1; }
-    e = mxfp6::launch_gemm_tiled(t, s);
+  mxfp6::GemmArgs t = g;
+  e = hipSuccess;
+  if (conv_a) {
+    uint8_t* p = ws;
+    uint8_t* sc = p + (((size_t)g.M * (g.K / 4 * 3) + 255) & ~(size_t)255);
+    e = mxfp6::launch_tile_both(g.A, p, g.As, sc, g.M, g.K, s);
+    t.A = p; t.As = sc; t.layout_a = 1;
   }
+  if (conv_b && e == hipSuccess) {
+    uint8_t* p = ws + bytes_a;
+    uint8_t* sc = p + (((size_t)g.N * (g.K / 4 * 3) + 255) & ~(size_t)255);
+    e = mxfp6::launch_tile_both(g.B, p, g.Bs, sc, g.N, g.K, s);
+    t.B = p; t.Bs = sc; t.layout_b = 1;
+  }
+  if (e == hipSuccess) e = mxfp6::launch_gemm_tiled(t, s);
   const hipError_t fe = hipFreeAsync(ws, s);
   if (e == hipSuccess) e = fe;
   return true;

@@ -151,6 +151,38 @@ hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K,
   return hipGetLastError();
 }
 
+// both of the above in one launch (row-major -> tile-major only): blocks [0, pblocks) move operand pieces, the rest scale
+// chunks.  Used by the re-layout pre-pass of the gemm entry points, where a second launch would cost as much as the copy.
+__global__ __launch_bounds__(256) void tile_both_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                       const uint8_t* __restrict__ ssrc, uint8_t* __restrict__ sdst, long npieces,
+                                                       long nchunks, int nkt, int nkb, int nk4, unsigned pblocks) {
+  if (blockIdx.x < pblocks) {
+    const long s = (long)blockIdx.x * 256 + threadIdx.x;
+    if (s >= npieces) return;
+    const int per_row = 6 * nkt;
+    const int row = (int)(s / per_row), p = (int)(s - (long)row * per_row);
+    *reinterpret_cast<v4i*>(dst + tile_major_offset(row, p * 16, nkt)) = *reinterpret_cast<const v4i*>(src + (size_t)s * 16);
+  } else {
+    const long s = (long)(blockIdx.x - pblocks) * 256 + threadIdx.x;
+    if (s >= nchunks) return;
+    const int row = (int)(s / nk4), g = (int)(s - (long)row * nk4);
+    const int nvalid = min(16, nkb - g * 16);
+    const size_t rm = (size_t)row * nkb + (size_t)g * 16, tm = tile_major_scale_offset(row, g * 16, nk4);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      *reinterpret_cast<uint32_t*>(sdst + tm + 4 * i) = 4 * i < nvalid ? *reinterpret_cast<const uint32_t*>(ssrc + rm + 4 * i) : 0u;
+  }
+}
+
+hipError_t launch_tile_both(const uint8_t* src, uint8_t* dst, const uint8_t* ssrc, uint8_t* sdst, int rows, int K, hipStream_t s) {
+  const int nkt = K / 128, nkb = K / 32, nk4 = (nkb + 15) / 16;
+  const long npieces = (long)rows * nkt * 6, nchunks = (long)rows * nk4;
+  if (npieces == 0) return hipSuccess;
+  const unsigned pblocks = (unsigned)((npieces + 255) / 256), sblocks = (unsigned)((nchunks + 255) / 256);
+  tile_both_kernel<<<pblocks + sblocks, 256, 0, s>>>(src, dst, ssrc, sdst, npieces, nchunks, nkt, nkb, nk4, pblocks);
+  return hipGetLastError();
+}
+
 __global__ void fill_zero_kernel(uint8_t* p, size_t n) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, st = (size_t)gridDim.x * 256;
   for (; i < n; i += st) p[i] = 0;

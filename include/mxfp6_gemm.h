@@ -74,7 +74,7 @@ int mxfp6_set_kernel(int which);
 
 /*
  * Re-layout pre-pass of the automatic path (on by default; returns the previous setting).  For large row-major
- * problems the gemm calls first copy the operand with fewer rows (and its scales) into tile-major order in a
+ * problems the gemm calls first copy one operand or both (with their scales) into tile-major order in a
  * workspace taken from, and returned to, the stream-ordered allocator (hipMallocAsync / hipFreeAsync on the
  * caller's stream), because the tiled kernel is bound by L2 requests on row-major operands; results are
  * bit-identical.  Switch it off to measure the row-major kernel itself or where the caller cannot tolerate an
