@@ -1,20 +1,22 @@
 // Mid-M MXFP6 GEMM for gfx950: 32 < M <= 256 or so, where a 256x256 tiling leaves most CUs idle and the
 // problem is bound by streaming B (weights) once from HBM and A many times from L2.
 //
-// One workgroup (8 waves) owns BM rows of A (64 or 128) x 32 rows of B over all of K.  All waves work on the
-// same K-tile; operands are staged through LDS by direct loads with the lane->address map and LDS image of
+// One workgroup (8 waves) owns BM rows of A (64 or 128) x BN rows of B (32 or 64) over all of K.  All waves work
+// on the same K-tile; operands are staged through LDS by direct loads with the lane->address map and LDS image of
 // the tiled kernel (gemm_tiled.hip), in two rings:
 //   A ring: three slots of BM rows x 2 K-tiles (192 contiguous bytes per row and slot), from L2;
-//   B ring: KB slots of 32 rows x 8 K-tiles = 24 KB (768 contiguous bytes per row; one contiguous run when B is
-//           tile-major), KB - 1 of them in flight: HBM latency is hidden by bytes in flight, and LDS is what
-//           limits them (BM = 64: KB = 4, 72 KB in flight; BM = 128: KB = 3, 48 KB).
+//   B ring: KB slots of BN rows x GB K-tiles = 24 KB (GB = 256 / BN: 768 or 384 contiguous bytes per row; whole
+//           3 KB tiles when B is tile-major), KB - 1 of them in flight: HBM latency is hidden by bytes in flight,
+//           and LDS is what limits them (BM = 64: KB = 4, 72 KB in flight; BM = 128: KB = 3, 48 KB).
+// Every workgroup re-reads its rows of A from L2, which is what bounds the kernel (about 10.5 TB/s of L2 -> LDS
+// traffic in aggregate): BN = 64 halves that traffic per output and is used when N still gives enough workgroups.
 // The VMEM counter is in-order, so a wave that waits for a young A slot would also wait for every older B
 // slot.  The two streams therefore belong to different waves: waves 0-3 issue all loads of A and of the scales,
 // waves 4-7 all loads of B, and each wave waits only for its own stream before the barrier that publishes a slot.
 // The E8M0 bytes of eight K-tiles (32 bytes per row) are direct-loaded into one of two small LDS buffers at
-// every B-slot boundary, one boundary ahead.  The BM/32 row tiles x 32 columns are too few for 8 waves, so
-// KP = 8 / (BM/32) waves share one 32x32 accumulator tile and split the 64-element MFMA steps of K between
-// them; the partial tiles are summed through LDS at the end (no scratch, no atomics).
+// every eighth K-tile, eight K-tiles ahead.  The (BM/32) x (BN/32) accumulator tiles are at most 8, so
+// KP = 8 / tiles waves share one 32x32 tile and split the 64-element MFMA steps of K between them; the partial
+// tiles are summed through LDS at the end (no scratch, no atomics).
 //
 // The reference has no kernel for these shapes (its GEMMs need M, N multiples of the 256 tile,
 // analysis/bf16_gemm/mi325x/kernel_8192.cpp:24-32).
@@ -25,7 +27,7 @@ namespace mxfp6 {
 
 namespace {
 
-constexpr int kBSlot = 24576;  // bytes of one B slot: 32 rows x 8 K-tiles
+constexpr int kBSlot = 24576;  // bytes of one B slot: BN rows x GB K-tiles
 constexpr int kASlots = 3;
 
 __device__ __forceinline__ void dma16_md(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
@@ -52,22 +54,24 @@ __device__ __forceinline__ void barrier_md() {
 
 }  // namespace
 
-template <int FA, int FB, typename Out, int BM>
+template <int FA, int FB, typename Out, int BM, int BN>
 __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                        const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                        typename Out::type* __restrict__ C, int M, int N, int K, int mblocks,
                                                        int layout_b) {
-  static_assert(BM == 64 || BM == 128, "BM");
+  static_assert((BM == 64 || BM == 128) && (BN == 32 || BN == 64), "tile");
   constexpr int GA = 2;                       // K-tiles per A slot
-  constexpr int TMW = BM / 32;                // 32-row tiles of A per workgroup
-  constexpr int KP = 8 / TMW;                 // waves per accumulator tile
+  constexpr int GB = 256 / BN;                // K-tiles per B slot: 8 or 4
+  constexpr int TMW = BM / 32, TNW = BN / 32; // 32-row tiles of A and of B per workgroup
+  constexpr int TILES = TMW * TNW;            // accumulator tiles: 2, 4 or 8
+  constexpr int KP = 8 / TILES;               // waves per accumulator tile
   constexpr int kASlot = BM * GA * 96;        // 12 or 24 KB
   constexpr int NA = kASlot / 1024 / 4;       // direct loads per A slot and A-wave: 3 or 6
   constexpr int NB = kBSlot / 1024 / 4;       // direct loads per B slot and B-wave: 6
   constexpr int KB = BM == 64 ? 4 : 3;        // B slots
   constexpr int kBRing = kASlots * kASlot;    // B ring starts after the A ring
   constexpr int kScBase = kBRing + KB * kBSlot;
-  constexpr int kScBuf = BM * 32 + 1024;      // scales of eight K-tiles: A rows x 32 bytes, then B's 32 rows x 32 bytes
+  constexpr int kScBuf = (BM + BN) * 32;      // scales of eight K-tiles: A rows x 32 bytes, then B rows x 32 bytes
   constexpr int kLds = kScBase + 2 * kScBuf;
   static_assert(kLds <= 163840 && kASlots * kASlot >= 8 * 16 * 64 * 4, "LDS budget (the A ring doubles as the reduction buffer)");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[kLds];
@@ -76,20 +80,21 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, r32 = lane & 31;
-  const int ti = wave % TMW, part = wave / TMW;  // accumulator tile and which MFMA steps of it this wave takes
+  const int tile = wave % TILES, ti = tile % TMW, tj = tile / TMW;  // accumulator tile of this wave ...
+  const int part = wave / TILES;                                     // ... and which MFMA steps of it the wave takes
   const bool a_wave = wave < 4;                  // waves 0-3 load A and the scales, waves 4-7 load B
   const int lw = wave & 3;
   const int nkt = K / 128, sbytes = K / 32, rowbytes = K / 4 * 3, nk4 = nkt / 4;
   // consecutive workgroups share their rows of B (they hit in L2 / the last-level cache together)
   const int nb = blockIdx.x / mblocks, mb = blockIdx.x - nb * mblocks;
-  const int n0 = nb * 32, m0 = mb * BM;
-  const int nrows = min(32, N - n0), mrows = min(BM, M - m0);
+  const int n0 = nb * BN, m0 = mb * BM;
+  const int nrows = min(BN, N - n0), mrows = min(BM, M - m0);
 
   // rows that do not exist lie past the end of the resource and read as zeros
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A + (size_t)m0 * rowbytes, (uint32_t)mrows * rowbytes);
   const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
   const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As + (size_t)m0 * sbytes, (uint32_t)mrows * sbytes);
-  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)nb * nk4 * 512, (uint32_t)nk4 * 512)
+  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)nb * TNW * nk4 * 512, (uint32_t)TNW * nk4 * 512)
                                               : make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
 
   // direct-load address maps.  Load q of a slot fills its LDS bytes [q*1024, q*1024 + 1024); a slot is a sequence of
@@ -104,22 +109,24 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
       voff_ld[i] = r * rowbytes + kin * 96 + c * 16;
     } else {
       const int o = (lw * NB + i) * 64 + lane;
-      const int kin = o / 192, rem = o - kin * 192, r = rem / 6, c = (rem - r * 6) ^ ((r >> 3) & 1);
-      voff_ld[i] = layout_b ? o * 16 : r * rowbytes + kin * 96 + c * 16;
+      const int kin = o / (BN * 6), rem = o - kin * (BN * 6), r = rem / 6, c = (rem - r * 6) ^ ((r >> 3) & 1);
+      // tile-major B: K-tile image kin of the slot = the 3 KB tiles (row-tile q, K-tile) of the workgroup's TNW row-tiles
+      voff_ld[i] = layout_b ? ((rem / 192) * nkt + kin) * 3072 + (rem % 192) * 16 : r * rowbytes + kin * 96 + c * 16;
     }
   }
-  const int bstep = layout_b ? 8 * 3072 : 8 * 96;  // bytes between B slots
+  const int bstep = layout_b ? GB * 3072 : GB * 96;  // bytes between B slots
 
-  // scale loads (A-waves): wave w < TMW fetches rows 32w .. 32w+31 of A, wave kScBWave the 32 rows of B: two lanes per row,
-  // 16 bytes (four K-tiles) each.  LDS image [row][32 bytes]; tile-major scales (two consecutive 512-byte chunks): [half][row][16].
-  constexpr int kScBWave = TMW < 4 ? TMW : 0;
-  const bool sc_a = wave < TMW, sc_b = wave == kScBWave;
-  const int n_sc = (sc_a ? 1 : 0) + (sc_b ? 1 : 0);  // scale loads of this wave per B-slot boundary
-  const int voff_sa = (wave * 32 + (lane >> 1)) * sbytes + (lane & 1) * 16;
-  const int voff_sb = layout_b ? lane * 16 : (lane >> 1) * sbytes + (lane & 1) * 16;
+  // scale loads (A-waves): job i < TMW fetches rows 32i .. 32i+31 of A, job TMW + q the rows of B's row-tile q: two lanes
+  // per row, 16 bytes (four K-tiles) each; job i belongs to wave i % 4.  LDS image per job: [row][32 bytes]; tile-major
+  // scales (two consecutive 512-byte chunks): [half][row][16].
+  constexpr int kScJobs = TMW + TNW;
+  int n_sc = 0;  // scale loads of this wave per group of eight K-tiles
+#pragma unroll
+  for (int i = 0; i < kScJobs; i++) n_sc += (a_wave && (i & 3) == wave) ? 1 : 0;
+  const int voff_srow = (lane >> 1) * sbytes + (lane & 1) * 16;
   const int sstep_b = layout_b ? 1024 : 32;  // bytes between groups of eight K-tiles
   const int sa_rd = kScBase + (ti * 32 + r32) * 32 + 2 * h;
-  const int sb_rd = kScBase + BM * 32 + (layout_b ? r32 * 16 : r32 * 32) + 2 * h;
+  const int sb_rd = kScBase + BM * 32 + tj * 1024 + (layout_b ? r32 * 16 : r32 * 32) + 2 * h;
   const int sb_half = layout_b ? 512 : 16;  // offset of K-tiles 4..7 of a group inside B's scale image
 
   const int sw = (r32 >> 3) & 1;
@@ -127,13 +134,23 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
 #pragma unroll
   for (int c = 0; c < 3; c++) {
     a_rd[c] = (ti * 32 + r32) * 96 + ((3 * h + c) ^ sw) * 16;
-    b_rd[c] = kBRing + r32 * 96 + ((3 * h + c) ^ sw) * 16;
+    b_rd[c] = kBRing + (tj * 32 + r32) * 96 + ((3 * h + c) ^ sw) * 16;
   }
 
   auto issue_scales = [&](int sg) __attribute__((always_inline)) {  // K-tiles 8 sg .. 8 sg + 7 into buffer sg & 1
     const uint32_t dst = lds0 + kScBase + (sg & 1) * kScBuf;
-    if (sc_a) dma16_md(rAs, dst + wave * 1024, voff_sa, __builtin_amdgcn_readfirstlane(sg * 32));
-    if (sc_b) dma16_md(rBs, dst + BM * 32, voff_sb, __builtin_amdgcn_readfirstlane(sg * sstep_b));
+#pragma unroll
+    for (int i = 0; i < kScJobs; i++) {
+      if (a_wave && (i & 3) == wave) {
+        if (i < TMW) {
+          dma16_md(rAs, dst + i * 1024, i * 32 * sbytes + voff_srow, __builtin_amdgcn_readfirstlane(sg * 32));
+        } else {
+          const int q = i - TMW;
+          dma16_md(rBs, dst + BM * 32 + q * 1024, layout_b ? q * nk4 * 512 + lane * 16 : q * 32 * sbytes + voff_srow,
+                   __builtin_amdgcn_readfirstlane(sg * sstep_b));
+        }
+      }
+    }
   };
   auto issue_a = [&](int j) __attribute__((always_inline)) {  // A slot j: K-tiles j*GA .. j*GA + GA-1 (A-waves)
     const uint32_t dst = lds0 + (j % kASlots) * kASlot + lw * (NA * 1024);
@@ -141,7 +158,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
 #pragma unroll
     for (int i = 0; i < NA; i++) dma16_md(rA, dst + i * 1024, voff_ld[i], so);
   };
-  auto issue_b = [&](int b) __attribute__((always_inline)) {  // B slot b: K-tiles 8b .. 8b+7 (B-waves)
+  auto issue_b = [&](int b) __attribute__((always_inline)) {  // B slot b: K-tiles GB b .. GB b + GB-1 (B-waves)
     const uint32_t dst = lds0 + kBRing + (b % KB) * kBSlot + lw * (NB * 1024);
     const int so = __builtin_amdgcn_readfirstlane(b * bstep);
 #pragma unroll
@@ -152,8 +169,8 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
 #pragma unroll
   for (int e = 0; e < 16; e++) acc[e] = 0.f;
 
-  const int nslots_a = nkt / GA, nslots_b = nkt / 8;
-  // prologue.  A-waves: scales of B slot 0, A slots 0 and 1.  B-waves: B slots 0 .. KB-2.
+  const int nslots_a = nkt / GA, nslots_b = nkt / GB, ngroups = nkt / 8;
+  // prologue.  A-waves: scales of the first eight K-tiles, A slots 0 and 1.  B-waves: B slots 0 .. KB-2.
   if (a_wave) {
     issue_scales(0);
     issue_a(0);
@@ -163,47 +180,46 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
     for (int b = 0; b < KB - 1; b++)
       if (b < nslots_b) issue_b(b);
   }
-  // A-wave loads issued at the boundary in front of K-tile kt, in this order: when kt % 8 == 0 the scales of B slot
-  // kt/8 + 1; always A slot kt/GA + 2
+  // A-wave loads issued at the boundary in front of K-tile kt, in this order: when kt % 8 == 0 the scales of K-tiles
+  // kt + 8 .. kt + 15; always A slot kt/GA + 2
   auto a_issued_at = [&](int kt) __attribute__((always_inline)) -> int {
     int n = 0;
-    if ((kt & 7) == 0 && (kt >> 3) + 1 < nslots_b) n += n_sc;
+    if ((kt & 7) == 0 && (kt >> 3) + 1 < ngroups) n += n_sc;
     if (kt / GA + 2 < nslots_a) n += NA;
     return n;
   };
 
   for (int kt0 = 0; kt0 < nkt; kt0 += 8) {
-    const int b = kt0 >> 3;
-    const int bslot = (b % KB) * kBSlot;
+    const int grp = kt0 >> 3;
 #pragma unroll
     for (int u = 0; u < 8; u += GA) {
-      const int kt = kt0 + u, j = kt / GA;
+      const int kt = kt0 + u, j = kt / GA, b = kt / GB;
+      const bool b_boundary = u % GB == 0;
       // boundary in front of K-tile kt.  A-waves: everything they issued before the previous boundary has landed (A slot j
-      // and, at a B-slot boundary, the scales of B slot b among it); the previous boundary's loads may stay in flight.
+      // and, at kt % 8 == 0, the scales of this group among it); the previous boundary's loads may stay in flight.
       // B-waves (B-slot boundaries only): B slot b has landed; the slots after it that exist may stay in flight.
       if (a_wave) {
         wait_loads_md(kt == 0 ? (nslots_a > 1 ? NA : 0) : a_issued_at(kt - GA));
-      } else if (u == 0) {
+      } else if (b_boundary) {
         wait_loads_md(NB * min(KB - 2, nslots_b - 1 - b));
       }
       barrier_md();
       if (a_wave) {
-        if (u == 0 && b + 1 < nslots_b) issue_scales(b + 1);
+        if (u == 0 && grp + 1 < ngroups) issue_scales(grp + 1);
         if (j + 2 < nslots_a) issue_a(j + 2);
-      } else if (u == 0 && b + KB - 1 < nslots_b) {
+      } else if (b_boundary && b + KB - 1 < nslots_b) {
         issue_b(b + KB - 1);
       }
 #pragma unroll
       for (int v = 0; v < GA; v++) {
         const int uu = u + v;  // K-tile kt0 + uu
-        // which MFMA step (64 elements of K) of this K-tile is this wave's: KP = 2: step `part`; KP = 4: waves with
-        // part < 2 take the even K-tiles, the others the odd ones
-        const bool active = KP == 2 || ((uu & 1) == (part >> 1));
+        // which MFMA steps (64 elements of K) of this K-tile are this wave's: KP = 1: both; KP = 2: step `part`; KP = 4:
+        // waves with part < 2 take the even K-tiles, the others the odd ones, step part & 1
+        const bool active = KP <= 2 || ((uu & 1) == (part >> 1));
         if (active) {
-          const int step = KP == 2 ? part : (part & 1);
           const uint8_t* sta = smem + (j % kASlots) * kASlot + v * (BM * 96);
-          const uint8_t* stb = smem + bslot + uu * 3072;
-          const uint8_t* scp = smem + (b & 1) * kScBuf;
+          const uint8_t* stb = smem + (b % KB) * kBSlot + (uu % GB) * (BN * 96);
+          const uint8_t* scp = smem + (grp & 1) * kScBuf;
           v4i fa[3], fb[3];
 #pragma unroll
           for (int c = 0; c < 3; c++) {
@@ -212,11 +228,13 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
           }
           const int sa = *reinterpret_cast<const uint16_t*>(scp + sa_rd + (uu >> 2) * 16 + (uu & 3) * 4);
           const int sb = *reinterpret_cast<const uint16_t*>(scp + sb_rd + (uu >> 2) * sb_half + (uu & 3) * 4);
-          if (step == 0) {
+          const int step = KP == 2 ? part : (part & 1);
+          if (KP == 1 || step == 0) {
             const v8i b0 = __builtin_shufflevector(fb[0], fb[1], 0, 1, 2, 3, 4, 5, -1, -1);
             const v8i a0 = __builtin_shufflevector(fa[0], fa[1], 0, 1, 2, 3, 4, 5, -1, -1);
             acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, sb, sa);
-          } else {
+          }
+          if (KP == 1 || step == 1) {
             const v8i b1 = __builtin_shufflevector(fb[1], fb[2], 2, 3, 4, 5, 6, 7, -1, -1);
             const v8i a1 = __builtin_shufflevector(fa[1], fa[2], 2, 3, 4, 5, 6, 7, -1, -1);
             acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, sb, sa);
@@ -226,20 +244,20 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
     }
   }
 
-  // sum the KP partial tiles: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4] of tile ti.
+  // sum the KP partial tiles: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4] of tile (ti, tj).
   // The A ring doubles as the reduction buffer once every wave is past its last LDS read.
   __syncthreads();
   float* partial = reinterpret_cast<float*>(smem);
 #pragma unroll
   for (int e = 0; e < 16; e++) partial[(wave * 16 + e) * 64 + lane] = acc[e];
   __syncthreads();
-  for (int idx = tid; idx < TMW * 1024; idx += 512) {
+  for (int idx = tid; idx < TILES * 1024; idx += 512) {
     const int t = idx >> 10, e = (idx >> 6) & 15, l = idx & 63;
     float s = 0.f;
 #pragma unroll
-    for (int p = 0; p < KP; p++) s += partial[((p * TMW + t) * 16 + e) * 64 + l];
-    const int m = m0 + t * 32 + (l & 31);
-    const long nn = (long)n0 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
+    for (int p = 0; p < KP; p++) s += partial[((p * TILES + t) * 16 + e) * 64 + l];
+    const int m = m0 + (t % TMW) * 32 + (l & 31);
+    const long nn = (long)n0 + (t / TMW) * 32 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
     if (m < M && nn < N) store1(C + (long)m * N + nn, s);
   }
 }
@@ -251,26 +269,38 @@ bool gemm_mid_supports(const GemmArgs& g) {
   return true;
 }
 
+// 64 rows of B per workgroup when 32 would need more than one round of workgroups (tile-major B: whole row-tiles only):
+// the time per K-tile and round is about the same for both widths, so halving the rounds is what counts
+static bool mid_wide(const GemmArgs& g) {
+  const long narrow = (long)((g.N + 31) / 32) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
+  return narrow > 256 && (!g.layout_b || g.N % 64 == 0) && (long)64 * (g.K / 4 * 3) < (1L << 31);
+}
+
 // Automatic choice against the 256x256 tiling: rounds of workgroups x time per K-tile and round of the two candidates
-// (the constants are measured, in microseconds: this kernel 0.36 / 0.47 for BM = 64 / 128, the tiled kernel 1.2).
+// (the constants are measured, in microseconds: this kernel 0.36 / 0.50 for BM = 64 / 128, the tiled kernel 1.2).
 bool gemm_mid_preferred(const GemmArgs& g) {
   if (!gemm_mid_supports(g)) return false;
   const double tiles256 = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  const double wgs = (double)((g.N + 31) / 32) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
+  const int bn = mid_wide(g) ? 64 : 32;
+  const double wgs = (double)((g.N + bn - 1) / bn) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
   const double rounds_mid = wgs > 256 ? wgs / 256 : 1, rounds_tiled = tiles256 > 256 ? tiles256 / 256 : 1;
-  return rounds_mid * (g.M <= 64 ? 0.36 : 0.47) < rounds_tiled * 1.2;
+  return rounds_mid * (g.M <= 64 ? 0.36 : 0.50) < rounds_tiled * 1.2;
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  const int nblocks = (g.N + 31) / 32;
+  typedef typename Out::type T;
+  const bool wide = mid_wide(g);
+  const int nblocks = wide ? (g.N + 63) / 64 : (g.N + 31) / 32;
+  const int mblocks = g.M <= 64 ? 1 : (g.M + 127) / 128;
+#define MXFP6_MID_LAUNCH(BM, BN) \
+  gemm_mid_kernel<FA, FB, Out, BM, BN><<<nblocks * mblocks, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, mblocks, g.layout_b)
   if (g.M <= 64) {
-    gemm_mid_kernel<FA, FB, Out, 64><<<nblocks, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, 1, g.layout_b);
+    if (wide) MXFP6_MID_LAUNCH(64, 64); else MXFP6_MID_LAUNCH(64, 32);
   } else {
-    const int mblocks = (g.M + 127) / 128;
-    gemm_mid_kernel<FA, FB, Out, 128><<<nblocks * mblocks, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, mblocks,
-                                                                        g.layout_b);
+    if (wide) MXFP6_MID_LAUNCH(128, 64); else MXFP6_MID_LAUNCH(128, 32);
   }
+#undef MXFP6_MID_LAUNCH
   return hipGetLastError();
 }
 

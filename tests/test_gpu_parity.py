@@ -170,7 +170,8 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
 
 # ------------------------------------------------------------------ mid-M kernel
 @pytest.mark.parametrize("M,N,K", [(33, 32, 1024), (64, 64, 1024), (48, 100, 2048), (64, 520, 3072), (65, 40, 1024), (128, 96, 4096), (100, 33, 2048),
-                                   (200, 72, 1024), (256, 160, 5120), (129, 31, 3072)])
+                                   (200, 72, 1024), (256, 160, 5120), (129, 31, 3072),
+                                   (64, 8320, 1024), (40, 8250, 2048), (160, 4200, 1024), (256, 4160, 2048)])   # 64 rows of B per workgroup
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3)])
 def test_mid_kernel_vs_oracle(hk, M, N, K, fa, fb):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + 2 * N + K, kind_a="laplace", kind_b="weights_outliers")
@@ -211,7 +212,7 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
 
 
 @pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
-                                          (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (0, 32, 32, 128)])
+                                          (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
     if kernel in (3, 4) and la == 1:
