@@ -40,8 +40,10 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
   // the operand with fewer rows first (it is the cheaper one to convert; the gain is the same)
   const bool a_first = g.M <= g.N;
   const int rows1 = a_first ? g.M : g.N, rows2 = a_first ? g.N : g.M;
-  bool conv1 = rows1 % 32 == 0 && 0.15 * t_gemm_us > 1.5 * cost_us(rows1);
-  bool conv2 = rows2 % 32 == 0 && (conv1 ? 0.11 : 0.15) * t_gemm_us > 1.5 * cost_us(rows2);
+  // fixed costs: the allocation and the dependent launch in front of the GEMM (about 10 us measured on a 33 us GEMM), a
+  // second launch about 3 us
+  bool conv1 = rows1 % 32 == 0 && 0.15 * t_gemm_us > 10 + 1.5 * cost_us(rows1);
+  bool conv2 = rows2 % 32 == 0 && (conv1 ? 0.11 * t_gemm_us > 3 + 1.5 * cost_us(rows2) : 0.15 * t_gemm_us > 10 + 1.5 * cost_us(rows2));
   if (!conv1 && !conv2) return false;
   const bool conv_a = a_first ? conv1 : conv2, conv_b = a_first ? conv2 : conv1;
   auto bytes_of = [&](int rows) { return (((size_t)rows * (g.K / 4 * 3) + 255) & ~(size_t)255) + (((size_t)rows * ((g.K + 511) / 512) * 16 + 255) & ~(size_t)255); };

@@ -1,4 +1,4 @@
-// Mid-M MXFP6 GEMM for gfx950: 32 < M <= 256 or so, where a 256x256 tiling leaves most CUs idle and the
+// Mid-M MXFP6 GEMM for gfx950: 32 < M <= 512, where a 256x256 tiling leaves most CUs idle and the
 // problem is bound by streaming B (weights) once from HBM and A many times from L2.
 //
 // One workgroup (8 waves) owns BM rows of A (64 or 128) x BN rows of B (32 or 64) over all of K.  All waves work
@@ -264,7 +264,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
 
 bool gemm_mid_supports(const GemmArgs& g) {
   // B slots are 8 K-tiles; A row-major (M need not be a multiple of 32)
-  if (g.layout_a != 0 || g.M <= 32 || g.M > 256 || g.N <= 0 || g.K < 1024 || g.K % 1024 != 0) return false;
+  if (g.layout_a != 0 || g.M <= 32 || g.M > 512 || g.N <= 0 || g.K < 1024 || g.K % 1024 != 0) return false;
   if ((long)g.M * (g.K / 4 * 3) >= (1L << 31) || (long)32 * (g.K / 4 * 3) >= (1L << 31)) return false;
   return true;
 }

@@ -64,7 +64,7 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
 /*
  * Kernel selection override for measurement and tests: 0 = automatic (default), 1 = generic
  * one-wave-per-tile kernel, 2 = LDS-tiled MFMA kernel (needs N % 8 == 0, K % 128 == 0),
- * 3 = skinny-M streaming kernel (needs M <= 32, K % 512 == 0), 4 = mid-M kernel (needs 32 < M <= 256,
+ * 3 = skinny-M streaming kernel (needs M <= 32, K % 512 == 0), 4 = mid-M kernel (needs 32 < M <= 512,
  * K % 1024 == 0, row-major A).  A forced kernel that cannot run the given
  * shape makes the gemm calls return MXFP6_EINVAL_SHAPE.  Returns the previous value.
  * No counterpart in the reference, whose shapes are compile-time constants per binary

@@ -171,7 +171,7 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
 # ------------------------------------------------------------------ mid-M kernel
 @pytest.mark.parametrize("M,N,K", [(33, 32, 1024), (64, 64, 1024), (48, 100, 2048), (64, 520, 3072), (65, 40, 1024), (128, 96, 4096), (100, 33, 2048),
                                    (200, 72, 1024), (256, 160, 5120), (129, 31, 3072),
-                                   (64, 8320, 1024), (40, 8250, 2048), (160, 4200, 1024), (256, 4160, 2048)])   # 64 rows of B per workgroup
+                                   (64, 8320, 1024), (40, 8250, 2048), (160, 4200, 1024), (256, 4160, 2048), (500, 2100, 1024)])   # 64 rows of B per workgroup
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3)])
 def test_mid_kernel_vs_oracle(hk, M, N, K, fa, fb):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + 2 * N + K, kind_a="laplace", kind_b="weights_outliers")
@@ -187,7 +187,7 @@ def test_mid_kernel_is_chosen_and_rejects_other_shapes(hk):
     ap, asc, bp, bsc = operands(96, 288, 2048, 2, 2, seed=9, kind_b="weights")
     assert np.array_equal(gemm(hk, ap, bp, asc, bsc, kernel=0), gemm(hk, ap, bp, asc, bsc, kernel=4))
     check(gemm(hk, ap, bp, asc, bsc, kernel=4), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)
-    for M, N, K in ((32, 64, 1024), (300, 64, 1024), (64, 64, 1536)):   # M <= 32, M > 256, K % 1024
+    for M, N, K in ((32, 64, 1024), (520, 64, 1024), (64, 64, 1536)):   # M <= 32, M > 512, K % 1024
         ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=5)
         with pytest.raises(RuntimeError, match="bad shape"):
             gemm(hk, ap, bp, asc, bsc, kernel=4)
