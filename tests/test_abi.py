@@ -141,3 +141,21 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.Mxfp6LibraryMissing, match="no CPU or PyTorch fallback"):
         _lib.lib()
+
+
+def test_torch_op_fake_shapes():
+    """The registered operator gives shapes and dtypes on meta tensors (no GPU, no library call)."""
+    import torch
+    from hipkittensp_amd import torch_op  # noqa: F401  (registers torch.ops.hipkittensp.mxfp6_gemm)
+
+    K, N = 1024, 96
+    A = torch.empty(3, 5, K // 4 * 3, dtype=torch.uint8, device="meta")
+    B = torch.empty(N, K // 4 * 3, dtype=torch.uint8, device="meta")
+    As = torch.empty(3, 5, K // 32, dtype=torch.uint8, device="meta")
+    Bs = torch.empty(N, 2 * 16, dtype=torch.uint8, device="meta")          # tile-major scales: ceil(K/512) * 16 bytes per row
+    C = torch.ops.hipkittensp.mxfp6_gemm(A, B, As, Bs, 2, 2, 0, 1, False)
+    assert C.shape == (3, 5, N) and C.dtype == torch.bfloat16
+    assert torch.ops.hipkittensp.mxfp6_gemm(A, B, As, Bs, 2, 3, 0, 1, True).dtype == torch.float32
+    import pytest
+    with pytest.raises(RuntimeError):
+        torch.ops.hipkittensp.mxfp6_gemm(A, B, As, Bs[:, :7], 2, 2, 0, 0, False)

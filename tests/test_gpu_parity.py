@@ -275,6 +275,25 @@ def test_cfg1_and_cfg3_tile_major_full_size(hk):
     assert torch.equal(C, Ct)
 
 
+# ------------------------------------------------------------------ torch.library operator
+def test_torch_op_and_linear_module(hk):
+    from hipkittensp_amd import torch_op
+
+    rng = np.random.default_rng(21)
+    w = o.make_source("weights", (160, 1024), rng)
+    x = o.make_source("normal", (2, 24, 1024), rng)
+    lin = torch_op.MXFP6Linear(dev(w))
+    assert lin.layout_w == hk.LAYOUT_TILE
+    y = lin(dev(x))
+    assert y.shape == (2, 24, 160) and y.dtype == torch.bfloat16
+    wp, ws = co.quantise(w, 2)
+    xp, xs = co.quantise(x.reshape(48, 1024), 2)
+    ref = o.gemm_ref(xp, wp, xs, ws, acc=np.float32)
+    got = y.view(torch.int16).cpu().numpy().view(np.uint16).reshape(48, 160)
+    assert np.array_equal(got, o.f32_to_bf16_bits(torch.ops.hipkittensp.mxfp6_gemm(dev(xp), dev(wp), dev(xs), dev(ws), 2, 2, 0, 0, True).cpu().numpy()))
+    assert o.rel_err(o.bf16_bits_to_f32(got), ref) <= 2 ** -7      # bf16 rounding of an in-tolerance result
+
+
 # ------------------------------------------------------------------ edge cases
 def test_empty_and_degenerate(hk):
     z = lambda *s: torch.zeros(*s, dtype=torch.uint8, device="cuda")
