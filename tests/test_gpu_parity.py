@@ -275,6 +275,33 @@ def test_cfg1_and_cfg3_tile_major_full_size(hk):
     assert torch.equal(C, Ct)
 
 
+# ------------------------------------------------------------------ automatic dispatch over ragged shapes
+def test_automatic_dispatch_agrees_with_generic_kernel_on_ragged_shapes(hk):
+    """Whatever kernel the library picks (skinny, mid-M, tiled, generic; row- or tile-major operands), the result agrees with
+    the independent one-wave-per-tile kernel on the row-major operands.  Seeded; shapes straddle every dispatch boundary."""
+    rng = np.random.default_rng(2024)
+    ks = [32, 96, 128, 384, 512, 640, 1024, 1536, 2048, 3072]
+    ms = [1, 7, 16, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 257, 300, 512, 513, 600]
+    ns = [8, 24, 32, 33, 64, 100, 256, 264, 520, 1000, 2048, 4160]
+    for it in range(40):
+        M, N, K = int(rng.choice(ms)), int(rng.choice(ns)), int(rng.choice(ks))
+        fa, fb = (2, 2) if it % 3 else (3, 2)
+        la = int(rng.integers(0, 2)) if (M % 32 == 0 and K % 128 == 0) else 0
+        lb = int(rng.integers(0, 2)) if (N % 32 == 0 and K % 128 == 0) else 0
+        ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=1000 + it, kind_b="weights")
+        ref = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=1)
+        A = hk.tile_operand(dev(ap)) if la else dev(ap)
+        B = hk.tile_operand(dev(bp)) if lb else dev(bp)
+        As = hk.tile_scales(dev(asc), K) if la else dev(asc)
+        Bs = hk.tile_scales(dev(bsc), K) if lb else dev(bsc)
+        C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        hk.dispatch_micro(A, B, As, Bs, C, fa, fb, layout_a=la, layout_b=lb)
+        torch.cuda.synchronize()
+        got = C.cpu().numpy()
+        assert np.isfinite(got).all(), (M, N, K, la, lb)
+        assert o.rel_err(got, ref) <= TOL_TIGHT, (M, N, K, la, lb, o.rel_err(got, ref))
+
+
 # ------------------------------------------------------------------ torch.library operator
 def test_torch_op_and_linear_module(hk):
     from hipkittensp_amd import torch_op
