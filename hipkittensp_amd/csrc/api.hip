@@ -48,25 +48,31 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
   const bool conv_a = a_first ? conv1 : conv2, conv_b = a_first ? conv2 : conv1;
   auto bytes_of = [&](int rows) { return (((size_t)rows * (g.K / 4 * 3) + 255) & ~(size_t)255) + (((size_t)rows * ((g.K + 511) / 512) * 16 + 255) & ~(size_t)255); };
   const size_t bytes_a = conv_a ? bytes_of(g.M) : 0, bytes_b = conv_b ? bytes_of(g.N) : 0;
+  // never allocate into a stream that is being captured: the caller replays the graph with its own memory plan
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return false;
+  }
   uint8_t* ws = nullptr;
   if (hipMallocAsync((void**)&ws, bytes_a + bytes_b, s) != hipSuccess || !ws) {
     (void)hipGetLastError();
     return false;
   }
   mxfp6::GemmArgs t = g;
-  e = hipSuccess;
-  if (conv_a) {
-    uint8_t* p = ws;
-    uint8_t* sc = p + (((size_t)g.M * (g.K / 4 * 3) + 255) & ~(size_t)255);
-    e = mxfp6::launch_tile_both(g.A, p, g.As, sc, g.M, g.K, s);
-    t.A = p; t.As = sc; t.layout_a = 1;
+  uint8_t* pa = ws;
+  uint8_t* sa = pa + (((size_t)g.M * (g.K / 4 * 3) + 255) & ~(size_t)255);
+  uint8_t* pb = ws + bytes_a;
+  uint8_t* sb = pb + (((size_t)g.N * (g.K / 4 * 3) + 255) & ~(size_t)255);
+  if (conv_a && conv_b) {
+    e = mxfp6::launch_tile_both(g.A, pa, g.As, sa, g.M, g.B, pb, g.Bs, sb, g.N, g.K, s);
+  } else if (conv_a) {
+    e = mxfp6::launch_tile_both(g.A, pa, g.As, sa, g.M, nullptr, nullptr, nullptr, nullptr, 0, g.K, s);
+  } else {
+    e = mxfp6::launch_tile_both(g.B, pb, g.Bs, sb, g.N, nullptr, nullptr, nullptr, nullptr, 0, g.K, s);
   }
-  if (conv_b && e == hipSuccess) {
-    uint8_t* p = ws + bytes_a;
-    uint8_t* sc = p + (((size_t)g.N * (g.K / 4 * 3) + 255) & ~(size_t)255);
-    e = mxfp6::launch_tile_both(g.B, p, g.Bs, sc, g.N, g.K, s);
-    t.B = p; t.Bs = sc; t.layout_b = 1;
-  }
+  if (conv_a) { t.A = pa; t.As = sa; t.layout_a = 1; }
+  if (conv_b) { t.B = pb; t.Bs = sb; t.layout_b = 1; }
   if (e == hipSuccess) e = mxfp6::launch_gemm_tiled(t, s);
   const hipError_t fe = hipFreeAsync(ws, s);
   if (e == hipSuccess) e = fe;

@@ -25,7 +25,8 @@ hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);
 hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);
 hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);
-hipError_t launch_tile_both(const uint8_t* src, uint8_t* dst, const uint8_t* ssrc, uint8_t* sdst, int rows, int K, hipStream_t s);
+hipError_t launch_tile_both(const uint8_t* src0, uint8_t* dst0, const uint8_t* ssrc0, uint8_t* sdst0, int rows0, const uint8_t* src1,
+                            uint8_t* dst1, const uint8_t* ssrc1, uint8_t* sdst1, int rows1, int K, hipStream_t s);
 hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 
 }  // namespace mxfp6

@@ -151,35 +151,60 @@ hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K,
   return hipGetLastError();
 }
 
-// both of the above in one launch (row-major -> tile-major only): blocks [0, pblocks) move operand pieces, the rest scale
-// chunks.  Used by the re-layout pre-pass of the gemm entry points, where a second launch would cost as much as the copy.
-__global__ __launch_bounds__(256) void tile_both_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
-                                                       const uint8_t* __restrict__ ssrc, uint8_t* __restrict__ sdst, long npieces,
-                                                       long nchunks, int nkt, int nkb, int nk4, unsigned pblocks) {
-  if (blockIdx.x < pblocks) {
-    const long s = (long)blockIdx.x * 256 + threadIdx.x;
-    if (s >= npieces) return;
-    const int per_row = 6 * nkt;
-    const int row = (int)(s / per_row), p = (int)(s - (long)row * per_row);
-    *reinterpret_cast<v4i*>(dst + tile_major_offset(row, p * 16, nkt)) = *reinterpret_cast<const v4i*>(src + (size_t)s * 16);
+// Row-major -> tile-major for up to two operands (packed bytes and scales) in one launch: the re-layout pre-pass of
+// the gemm entry points, where every extra launch would cost as much as part of the copy.  One lane writes one
+// 16-byte piece of the destination (consecutive lanes: consecutive bytes of a tile-major operand, i.e. whole 3 KB
+// tiles) or the 16 scale bytes one row has for four K-tiles.
+struct TileJob {
+  const uint8_t* src;
+  uint8_t* dst;
+  const uint8_t* ssrc;
+  uint8_t* sdst;
+  long npieces, nchunks;
+  unsigned pblocks, sblocks;
+};
+
+__global__ __launch_bounds__(256) void tile_both_kernel(TileJob j0, TileJob j1, int nkt, int nkb, int nk4) {
+  unsigned bid = blockIdx.x;
+  const bool second = bid >= j0.pblocks + j0.sblocks;
+  if (second) bid -= j0.pblocks + j0.sblocks;
+  const TileJob& j = second ? j1 : j0;
+  if (bid < j.pblocks) {
+    const long d = (long)bid * 256 + threadIdx.x;  // destination piece
+    if (d >= j.npieces) return;
+    // destination piece d lives in tile d / 192 = rt * nkt + kt, slot d % 192 = r * 6 + (c ^ ((r >> 3) & 1))
+    const long tile = d / 192;
+    const int in = (int)(d - tile * 192), r = in / 6, c = (in - r * 6) ^ ((r >> 3) & 1);
+    const long rt = tile / nkt;
+    const int kt = (int)(tile - rt * nkt);
+    const size_t so = ((size_t)(rt * 32 + r) * nkt + kt) * 96 + (size_t)c * 16;
+    *reinterpret_cast<v4i*>(j.dst + (size_t)d * 16) = *reinterpret_cast<const v4i*>(j.src + so);
   } else {
-    const long s = (long)(blockIdx.x - pblocks) * 256 + threadIdx.x;
-    if (s >= nchunks) return;
+    const long s = (long)(bid - j.pblocks) * 256 + threadIdx.x;
+    if (s >= j.nchunks) return;
     const int row = (int)(s / nk4), g = (int)(s - (long)row * nk4);
     const int nvalid = min(16, nkb - g * 16);
     const size_t rm = (size_t)row * nkb + (size_t)g * 16, tm = tile_major_scale_offset(row, g * 16, nk4);
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      *reinterpret_cast<uint32_t*>(sdst + tm + 4 * i) = 4 * i < nvalid ? *reinterpret_cast<const uint32_t*>(ssrc + rm + 4 * i) : 0u;
+      *reinterpret_cast<uint32_t*>(j.sdst + tm + 4 * i) = 4 * i < nvalid ? *reinterpret_cast<const uint32_t*>(j.ssrc + rm + 4 * i) : 0u;
   }
 }
 
-hipError_t launch_tile_both(const uint8_t* src, uint8_t* dst, const uint8_t* ssrc, uint8_t* sdst, int rows, int K, hipStream_t s) {
+// rows1 == 0: only the first operand
+hipError_t launch_tile_both(const uint8_t* src0, uint8_t* dst0, const uint8_t* ssrc0, uint8_t* sdst0, int rows0, const uint8_t* src1,
+                            uint8_t* dst1, const uint8_t* ssrc1, uint8_t* sdst1, int rows1, int K, hipStream_t s) {
   const int nkt = K / 128, nkb = K / 32, nk4 = (nkb + 15) / 16;
-  const long npieces = (long)rows * nkt * 6, nchunks = (long)rows * nk4;
-  if (npieces == 0) return hipSuccess;
-  const unsigned pblocks = (unsigned)((npieces + 255) / 256), sblocks = (unsigned)((nchunks + 255) / 256);
-  tile_both_kernel<<<pblocks + sblocks, 256, 0, s>>>(src, dst, ssrc, sdst, npieces, nchunks, nkt, nkb, nk4, pblocks);
+  auto job = [&](const uint8_t* src, uint8_t* dst, const uint8_t* ssrc, uint8_t* sdst, int rows) {
+    TileJob j{src, dst, ssrc, sdst, (long)rows * nkt * 6, (long)rows * nk4, 0, 0};
+    j.pblocks = (unsigned)((j.npieces + 255) / 256);
+    j.sblocks = (unsigned)((j.nchunks + 255) / 256);
+    return j;
+  };
+  const TileJob j0 = job(src0, dst0, ssrc0, sdst0, rows0), j1 = job(src1, dst1, ssrc1, sdst1, rows1);
+  const unsigned blocks = j0.pblocks + j0.sblocks + j1.pblocks + j1.sblocks;
+  if (blocks == 0) return hipSuccess;
+  tile_both_kernel<<<blocks, 256, 0, s>>>(j0, j1, nkt, nkb, nk4);
   return hipGetLastError();
 }
 

@@ -77,8 +77,9 @@ int mxfp6_set_kernel(int which);
  * problems the gemm calls first copy one operand or both (with their scales) into tile-major order in a
  * workspace taken from, and returned to, the stream-ordered allocator (hipMallocAsync / hipFreeAsync on the
  * caller's stream), because the tiled kernel is bound by L2 requests on row-major operands; results are
- * bit-identical.  Switch it off to measure the row-major kernel itself or where the caller cannot tolerate an
- * allocation (e.g. stream capture).  No counterpart in the reference.
+ * bit-identical.  It is skipped by itself on a stream that is being captured.  Switch it off to measure the
+ * row-major kernel itself or where the caller cannot tolerate a stream-ordered allocation.  No counterpart in
+ * the reference.
  */
 int mxfp6_set_relayout(int on);
 

@@ -302,6 +302,40 @@ def test_automatic_dispatch_agrees_with_generic_kernel_on_ragged_shapes(hk):
         assert o.rel_err(got, ref) <= TOL_TIGHT, (M, N, K, la, lb, o.rel_err(got, ref))
 
 
+# ------------------------------------------------------------------ stream capture
+def test_graph_capture_replays_match_eager(hk):
+    """A size at which the eager path takes the re-layout pre-pass (workspace from the stream-ordered allocator): under
+    capture the library must not allocate, and every replay must reproduce the eager result bit for bit."""
+    M = N = K = 8192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(77)
+    sets = []
+    for _ in range(2):
+        a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+        b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g), 2)
+        sets.append((a, b, asc, bsc))
+    eager = []
+    for a, b, asc, bsc in sets:
+        C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        hk.dispatch_micro(a, b, asc, bsc, C)
+        eager.append(C)
+    torch.cuda.synchronize()
+    sa, sb, sas, sbs = (t.clone() for t in sets[0])
+    Cg = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hk.dispatch_micro(sa, sb, sas, sbs, Cg)
+    for rep in range(4):
+        a, b, asc, bsc = sets[rep % 2]
+        sa.copy_(a); sb.copy_(b); sas.copy_(asc); sbs.copy_(bsc)
+        Cg.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Cg, eager[rep % 2]), f"replay {rep}"
+        hk.dispatch_micro(a, b, asc, bsc, torch.empty_like(Cg))   # eager work between replays
+        torch.cuda.synchronize()
+
+
 # ------------------------------------------------------------------ torch.library operator
 def test_torch_op_and_linear_module(hk):
     from hipkittensp_amd import torch_op
