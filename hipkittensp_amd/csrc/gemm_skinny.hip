@@ -1,18 +1,26 @@
 // Skinny-M (decode-shaped) MXFP6 GEMM for gfx950: M <= 32, bound by HBM.
 //
-// Every byte of B (weights) is read from HBM once.  One workgroup owns 32 consecutive rows of B
-// (32 output columns) and splits K over its waves in chunks of four K-tiles (4 x 128 elements =
-// 384 bytes per row = three whole 128-byte lines), dealt round-robin: wave w takes chunks w, w+NW, ...
-// so the workgroup streams one contiguous K range of its 32 rows and no cache line is shared
-// between chunks.  With a tile-major B the 32 rows x K of a workgroup are one contiguous run of HBM.  Each wave owns a private 4-stage LDS ring (one stage per K-tile of a chunk):
-//   global --buffer_load_dwordx4 ... lds--> LDS --ds_read_b128--> MFMA sources
-// with the same lane->address map as the tiled kernel (consecutive lanes fetch consecutive 16-byte
-// pieces of a row; row-major 96-byte LDS rows with a pair swap that makes the reads conflict-free).
-// Staging through LDS is what lets the loads be coalesced: the MFMA wants lane = row, the memory
-// system wants lane = consecutive bytes.  A's rows (M <= 32) are staged the same way from L2.  The
-// E8M0 bytes of a chunk are 16 bytes per row: one 16-byte load per lane per chunk, kept in VGPRs.
-// All loads are issued from inline assembly and waited for with hand-counted vmcnt, four K-tiles
-// ahead.  The partial 32x32 tiles of the waves are summed through LDS: no scratch, no atomics.
+// Every byte of B (weights) is read from HBM once.  One workgroup owns 32 consecutive rows of B (32 output
+// columns) and splits K over its waves in chunks of four K-tiles (4 x 128 elements = 384 bytes per row = three
+// whole 128-byte lines), dealt round-robin: wave w takes chunks w, w+NW, ... so the workgroup streams one
+// contiguous K range of its 32 rows.  Each wave owns a private LDS buffer for one chunk (B: 12 KB, A: 6 or 12 KB)
+// and runs
+//   issue the chunk's direct loads -> wait for all of them -> LDS -> registers (all four K-tiles) ->
+//   issue the next chunk's loads -> 8 MFMAs
+// so that a wave's whole buffer is in flight except while it is being read out (a few hundred clocks against
+// microseconds of HBM latency), and the 6-8 waves of a workgroup are out of phase with each other.
+// A direct load fetches, per row, the chunk's 384 contiguous bytes (24 lanes x 16 bytes), i.e. whole cache lines:
+// a row-major B costs the same L2 requests and HBM bursts as a tile-major one.  The LDS image of a row-major
+// chunk is [row][384 bytes] with the 16-byte pieces of a row permuted inside groups of eight,
+//     piece p of row r lives at  r * 384 + (p ^ ((r >> 1) & 7)) * 16,
+// which spreads the 16 rows of a ds_read_b128 phase over all 64 banks (rows r and r+16 share banks and are never
+// in the same phase, analysis/paper_experiments/phases/ds_read_b128/phase_results.txt:4-7); the permutation is
+// applied by choosing which global bytes each lane fetches, as in the tiled kernel.  A tile-major B arrives as
+// four 3 KB tiles in the tiled kernel's image.  A's rows (M <= 32) are staged like a row-major B, from L2.  The
+// E8M0 bytes of a chunk are 16 bytes per row: one more direct load each for B and A (no load of this kernel has a
+// register destination, so nothing can read a register before its load has landed).  All loads are issued from
+// inline assembly and waited for with vmcnt by hand.  The partial 32x32 tiles of the waves are summed
+// through LDS: no scratch, no atomics.
 //
 // The reference has no kernel for this shape (its GEMMs need M, N multiples of the 256 tile,
 // analysis/bf16_gemm/mi325x/kernel_8192.cpp:24-32).  Algorithmic bytes per launch:
@@ -24,38 +32,26 @@ namespace mxfp6 {
 
 namespace {
 
-constexpr int kStagesSk = 4;  // = K-tiles per chunk
-
 __device__ __forceinline__ void dma16_sk(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory");
 }
-__device__ __forceinline__ v4i load128_sk(const __amdgpu_buffer_rsrc_t& r, int voff, int soff) {
-  v4i d;
-  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(d) : "v"(voff), "s"(r), "s"(soff) : "memory");
-  return d;
-}
-// wait until at most N of this wave's loads are outstanding; the scale registers ride along as
-// read-write operands so that no use of them can be scheduled above the wait
-template <int N>
-__device__ __forceinline__ void wait_loads(v4i& s0, v4i& s1) {
-  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(s0), "+v"(s1) : "n"(N) : "memory");
-}
+__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 }  // namespace
 
-// AR = rows of A staged per K-tile (16 or 32); NW = waves per workgroup
+// AR = rows of A staged (16 or 32); NW = waves per workgroup
 template <int FA, int FB, typename Out, int AR, int NW>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                               typename Out::type* __restrict__ C, int M, int N, int K, int layout_b) {
-  constexpr int kBTile = 32 * 96, kATile = AR * 96, kStage = kBTile + kATile, kRing = kStagesSk * kStage;
-  constexpr int kADma = (kATile + 1023) / 1024;  // direct loads per A tile (the last one half full when AR = 16)
-  constexpr int kDmaPerTile = 3 + kADma;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kRing];
-  static_assert(NW * kRing <= 163840 && NW * kRing >= NW * 16 * 64 * 4, "LDS budget (ring doubles as the reduction buffer)");
+  constexpr int kBBuf = 32 * 384, kABuf = AR * 384, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then 2 x 1 KB of scales
+  constexpr int kBuf = kScOff + 2048;
+  constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024;                    // direct loads per chunk: 12 and 6 or 12
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kBuf];
+  static_assert(NW * kBuf <= 163840 && NW * kBuf >= NW * 16 * 64 * 4, "LDS budget (the buffers double as the reduction buffer)");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -68,126 +64,96 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, (uint32_t)M * rowbytes);
   // tile-major B: this workgroup's 32 rows are one row-tile, whose scales are nk4 chunks of 512 bytes (row r at r * 16)
-  const int nk4 = (nkt + 3) / 4;
+  const int nk4 = nkt / 4;
   const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)blockIdx.x * nk4 * 512, (uint32_t)nk4 * 512)
                                               : make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
   const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * sbytes);
 
-  // direct-load address map: LDS slot o (16 bytes) of a tile holds chunk (o%6) ^ ((row>>3)&1) of row o/6
-  int voff[3];
+  // direct-load address maps: load i fills LDS bytes [i*1024, i*1024 + 1024) of the buffer; slot o = i*64 + lane holds
+  // piece (o % 24) ^ ((row >> 1) & 7) of row o / 24.  Tile-major B: four consecutive 3 KB tiles, copied as they are.
+  int voff_b[NBL], voff_a[NAL];
 #pragma unroll
-  for (int i = 0; i < 3; i++) {
-    const int o = i * 64 + lane, r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
-    voff[i] = r * rowbytes + c * 16;
+  for (int i = 0; i < NBL; i++) {
+    const int o = i * 64 + lane, r = o / 24, p = (o - r * 24) ^ ((r >> 1) & 7);
+    voff_b[i] = layout_b ? o * 16 : r * rowbytes + p * 16;
   }
-  // tile-major B: the 32-row tile is stored in LDS image order, a load is one contiguous KiB
-  int voff_bt[3];
 #pragma unroll
-  for (int i = 0; i < 3; i++) voff_bt[i] = layout_b ? (i * 64 + lane) * 16 : voff[i];
-  const int voff_bs = layout_b ? r32 * 16 : r32 * sbytes, voff_as = (AR == 16 ? (r32 & 15) : r32) * sbytes;
+  for (int i = 0; i < NAL; i++) {
+    const int o = i * 64 + lane, r = o / 24, p = (o - r * 24) ^ ((r >> 1) & 7);
+    voff_a[i] = r * rowbytes + p * 16;
+  }
+  // scale loads: lane l fetches the 16 bytes of row l % 32 (both halves of the wave fetch the same rows)
+  const int voff_bs = layout_b ? r32 * 16 : r32 * sbytes;
+  const int voff_as = r32 * sbytes;
+  const int ra = AR == 16 ? (r32 & 15) : r32;  // AR = 16: lanes 16-31 mirror rows 0-15 (their outputs are never stored)
 
-  const uint32_t ring = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kRing;
-  const uint8_t* ringp = smem + wave * kRing;
-  const int sw = (r32 >> 3) & 1;
-  int b_rd[3], a_rd[3];
+  const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kBuf;
+  const uint8_t* bufp = smem + wave * kBuf;
+  // LDS read offsets of this lane: K-tile u, piece c of its half (pieces 3h .. 3h+2 of the K-tile)
+  int b_rd[4][3], a_rd[4][3];
 #pragma unroll
-  for (int c = 0; c < 3; c++) {
-    b_rd[c] = r32 * 96 + ((3 * h + c) ^ sw) * 16;
-    const int ra = AR == 16 ? (r32 & 15) : r32;  // AR = 16: lanes 16-31 mirror rows 0-15 (their outputs are never stored)
-    a_rd[c] = kBTile + ra * 96 + ((3 * h + c) ^ ((ra >> 3) & 1)) * 16;
-  }
+  for (int u = 0; u < 4; u++)
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      const int p = u * 6 + 3 * h + c;
+      b_rd[u][c] = layout_b ? u * 3072 + r32 * 96 + ((3 * h + c) ^ ((r32 >> 3) & 1)) * 16 : r32 * 384 + (p ^ ((r32 >> 1) & 7)) * 16;
+      a_rd[u][c] = kBBuf + ra * 384 + (p ^ ((ra >> 1) & 7)) * 16;
+    }
 
   // chunks of this wave: wave, wave + NW, ...
-  const int nchunks = (nkt + 3) / 4;
+  const int nchunks = nkt / 4;
   const int mine = wave < nchunks ? (nchunks - wave + NW - 1) / NW : 0;
 
-  v4i sc_b_next, sc_a_next, sc_b, sc_a;
-  sc_b_next = sc_a_next = sc_b = sc_a = v4i{0, 0, 0, 0};
-
-  auto issue_scales = [&](int chunk) {  // 16 scale bytes per row: the chunk's four K-tiles
-    const int so = __builtin_amdgcn_readfirstlane(chunk * 16);
-    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * 512 : chunk * 16);
-    sc_b_next = load128_sk(rBs, voff_bs, sob);
-    sc_a_next = load128_sk(rAs, voff_as, so);
-  };
-  auto issue_tile = [&](int chunk, int u) {  // K-tile u of a chunk into stage u
-    const int t = min(chunk * 4 + u, nkt - 1);  // past-the-end tiles re-read the last one and are never multiplied
-    const int so = __builtin_amdgcn_readfirstlane(t * 96);
-    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? t * 3072 : t * 96);
-    const uint32_t dst = ring + u * kStage;
+  auto issue_chunk = [&](int chunk) __attribute__((always_inline)) {
+    const int sos = __builtin_amdgcn_readfirstlane(chunk * 16);
+    const int sosb = __builtin_amdgcn_readfirstlane(layout_b ? chunk * 512 : chunk * 16);
+    dma16_sk(rBs, buf + kScOff, voff_bs, sosb);
+    dma16_sk(rAs, buf + kScOff + 1024, voff_as, sos);
+    const int so = __builtin_amdgcn_readfirstlane(chunk * 384);
+    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * (4 * 3072) : chunk * 384);
 #pragma unroll
-    for (int i = 0; i < 3; i++) dma16_sk(rB, dst + i * 1024, voff_bt[i], sob);
-    dma16_sk(rA, dst + kBTile, voff[0], so);
-    if constexpr (kADma == 2) {
-      if (lane < 32) dma16_sk(rA, dst + kBTile + 1024, voff[1], so);
-    } else {
-      dma16_sk(rA, dst + kBTile + 1024, voff[1], so);
-      dma16_sk(rA, dst + kBTile + 2048, voff[2], so);
-    }
+    for (int i = 0; i < NBL; i++) dma16_sk(rB, buf + i * 1024, voff_b[i], sob);
+#pragma unroll
+    for (int i = 0; i < NAL; i++) dma16_sk(rA, buf + kBBuf + i * 1024, voff_a[i], so);
   };
 
   v16f acc;
 #pragma unroll
   for (int e = 0; e < 16; e++) acc[e] = 0.f;
 
-  auto consume = [&](int chunk, int u) {
-    if (chunk * 4 + u >= nkt) return;
-    const uint8_t* st = ringp + u * kStage;
-    v4i fb[3], fa[3];
-#pragma unroll
-    for (int c = 0; c < 3; c++) {
-      fb[c] = *reinterpret_cast<const v4i*>(st + b_rd[c]);
-      fa[c] = *reinterpret_cast<const v4i*>(st + a_rd[c]);
-    }
-    const int sb = (uint32_t)sc_b[u] >> (16 * h), sa = (uint32_t)sc_a[u] >> (16 * h);
-    const v8i b0 = __builtin_shufflevector(fb[0], fb[1], 0, 1, 2, 3, 4, 5, -1, -1);
-    const v8i b1 = __builtin_shufflevector(fb[1], fb[2], 2, 3, 4, 5, 6, 7, -1, -1);
-    const v8i a0 = __builtin_shufflevector(fa[0], fa[1], 0, 1, 2, 3, 4, 5, -1, -1);
-    const v8i a1 = __builtin_shufflevector(fa[1], fa[2], 2, 3, 4, 5, 6, 7, -1, -1);
-    acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, sb, sa);
-    acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, sb, sa);
-    // the stage is about to be refilled: its reads must have left LDS
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  };
-
   if (mine > 0) {
-    issue_scales(wave);
+    issue_chunk(wave);
+    for (int j = 0; j < mine; j++) {
+      wait_all_loads();
+      const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + r32 * 16);
+      const v4i sc_a = *reinterpret_cast<const v4i*>(bufp + kScOff + 1024 + ra * 16);
+      v4i fb[4][3], fa[4][3];
 #pragma unroll
-    for (int u = 0; u < 4; u++) issue_tile(wave, u);
-    int j = 0;
-    // steady state: waiting for tile (j,u) leaves the direct loads of the next three tiles in flight,
-    // plus the two scale loads of chunk j+1 once they have been issued (u >= 1)
-    for (; j + 1 < mine; j++) {
-      const int chunk = wave + j * NW, next = chunk + NW;
-      wait_loads<3 * kDmaPerTile>(sc_b_next, sc_a_next);
-      sc_b = sc_b_next;
-      sc_a = sc_a_next;
-      consume(chunk, 0);
-      issue_scales(next);
-      issue_tile(next, 0);
+      for (int u = 0; u < 4; u++)
 #pragma unroll
-      for (int u = 1; u < 4; u++) {
-        wait_loads<3 * kDmaPerTile + 2>(sc_b_next, sc_a_next);
-        consume(chunk, u);
-        issue_tile(next, u);
+        for (int c = 0; c < 3; c++) {
+          fb[u][c] = *reinterpret_cast<const v4i*>(bufp + b_rd[u][c]);
+          fa[u][c] = *reinterpret_cast<const v4i*>(bufp + a_rd[u][c]);
+        }
+      // the buffer is about to be refilled: its reads must have left LDS
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      if (j + 1 < mine) issue_chunk(wave + (j + 1) * NW);
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int sb = (uint32_t)sc_b[u] >> (16 * h), sa = (uint32_t)sc_a[u] >> (16 * h);
+        const v8i b0 = __builtin_shufflevector(fb[u][0], fb[u][1], 0, 1, 2, 3, 4, 5, -1, -1);
+        const v8i b1 = __builtin_shufflevector(fb[u][1], fb[u][2], 2, 3, 4, 5, 6, 7, -1, -1);
+        const v8i a0 = __builtin_shufflevector(fa[u][0], fa[u][1], 0, 1, 2, 3, 4, 5, -1, -1);
+        const v8i a1 = __builtin_shufflevector(fa[u][1], fa[u][2], 2, 3, 4, 5, 6, 7, -1, -1);
+        acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, sb, sa);
+        acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, sb, sa);
       }
     }
-    // last chunk: nothing more to issue
-    const int chunk = wave + j * NW;
-    wait_loads<3 * kDmaPerTile>(sc_b_next, sc_a_next);
-    sc_b = sc_b_next;
-    sc_a = sc_a_next;
-    consume(chunk, 0);
-    wait_loads<2 * kDmaPerTile>(sc_b_next, sc_a_next);
-    consume(chunk, 1);
-    wait_loads<1 * kDmaPerTile>(sc_b_next, sc_a_next);
-    consume(chunk, 2);
-    wait_loads<0>(sc_b_next, sc_a_next);
-    consume(chunk, 3);
   }
 
   // sum the K-slices: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4].
-  // The ring doubles as the reduction buffer once every wave has drained its loads.
+  // The buffers double as the reduction buffer once every wave has drained its loads.
   __syncthreads();
   float* part = reinterpret_cast<float*>(smem);
 #pragma unroll
