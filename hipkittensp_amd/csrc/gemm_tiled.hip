@@ -3,7 +3,12 @@
 // Data path (no operand byte ever passes through a VGPR on its way to LDS):
 //   global --buffer_load_dwordx4 ... lds--> LDS (3-stage ring) --ds_read_b128--> MFMA source VGPRs
 //   v_mfma_scale_f32_32x32x64_f8f6f4 (fp32 accumulate, E8M0 block scales applied by the instruction)
-//   accumulators --v_cvt_pk_bf16_f32--> LDS --> whole rows to global
+//   accumulators --v_cvt_pk_bf16_f32, v_permlane32_swap--> 16 bytes per lane to global
+// When there are more output tiles than compute units, one workgroup per CU walks through several tiles:
+// the K-tiles of all its output tiles form one stream through the ring, so the loads of the next tile
+// run under the last K-tiles of the current one and the stores of a finished tile under the first
+// K-tiles of the next (measured: +1-2 % at K = 8192, +10 % at K = 1024; what remains per output tile,
+// ~10 000 clocks at 8192^3, is the time all CUs together need to push 32 MB of C to HBM at once).
 //
 // LDS image of one operand tile (256 rows x 96 bytes = 6 pieces of 16 B per row): row-major, 96 bytes
 // per row, with pieces 2p and 2p+1 exchanged in every row whose bit 3 is set:
@@ -44,6 +49,8 @@
 
 namespace mxfp6 {
 
+int g_tiled_walk = 1;  // 0: always one workgroup per output tile (development switch)
+
 constexpr int kBM = 256, kBN = 256, kBK = 128;
 constexpr int kOpStage = 256 * 96;  // bytes of one operand tile
 constexpr int kScStage = 256 * 16;  // bytes of one operand's scales for four K-tiles
@@ -80,50 +87,77 @@ __device__ __forceinline__ void barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// The kernel's arguments, passed as one struct: a workgroup that walks through several output tiles reads
+// them again from the kernel-argument segment whenever it moves on, instead of keeping all of them in
+// scalar registers through the K loop.
+struct TiledArgs {
+  const uint8_t *A, *B, *As, *Bs;
+  void* C;
+  int M, N, K, tiles_m, tiles_n, layout_a, layout_b;
+};
+
 template <int FA, int FB, typename Out>
-__global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
-                                                             const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
-                                                             typename Out::type* __restrict__ C, int M, int N, int K,
-                                                             int tiles_m, int tiles_n, int layout_a, int layout_b) {
+__global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
   // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
   __shared__ __attribute__((aligned(1024))) uint8_t smem[kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
+  const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
+  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK;
+  const int nk4 = (nkt + 3) / 4;  // groups of four K-tiles; tile-major scales hold one 512-byte chunk per 32 rows and group
+  const bool sc_a = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) < 4;  // this wave loads A's scales (else B's)
 
-  // ---- workgroup -> output tile: undo the round-robin XCD placement, then a grouped raster.
-  // Hardware places workgroup b on XCD b % 8; remapping gives each XCD a contiguous run of logical
-  // tiles so that the 32 tiles an XCD works on at once share operand rows in its L2
-  // (the idea of chiplet_transform_chunked, include/common/util.cuh:78-101, as an exact bijection).
-  const int nb = tiles_m * tiles_n;
-  int L;
-  {
-    const int bid = blockIdx.x, xcd = bid & 7, idx = bid >> 3;
+  // the arguments, read afresh (the empty asm hides from the compiler that the pointer is always the same)
+  auto fresh_args = [&]() __attribute__((always_inline)) {
+    auto p = (const __attribute__((address_space(4))) TiledArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return p;
+  };
+
+  // ---- workgroup -> output tiles.  Workgroup b works on tiles b, b + gridDim.x, ... of a logical order in
+  // which the round-robin XCD placement is undone and the raster is grouped.  Hardware places workgroup b on
+  // XCD b % 8; the remapping gives each XCD a contiguous run of logical tiles so that the 32 tiles an XCD
+  // works on at once share operand rows in its L2 (the idea of chiplet_transform_chunked,
+  // include/common/util.cuh:78-101, as an exact bijection).  Returns pm | pn << 16, or -1 past the last tile.
+  auto tile_of = [&](int bid) __attribute__((always_inline)) {
+    const auto g = fresh_args();
+    const int tiles_m = g->tiles_m, tiles_n = g->tiles_n, nb = tiles_m * tiles_n;
+    if (bid >= nb) return -1;
+    const int xcd = bid & 7, idx = bid >> 3;
     const int per = nb >> 3, rem = nb & 7;
-    L = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
-  }
-  int pm, pn;
-  {
+    const int L = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
     const int width = kGroupM * tiles_n, group = L / width, first = group * kGroupM;
     const int gsz = min(tiles_m - first, kGroupM), in = L - group * width;
-    pm = first + in % gsz;
-    pn = in / gsz;
-  }
+    return (first + in % gsz) | (in / gsz) << 16;
+  };
+  // Buffer resources of one output tile's operand rows (A and B) and of the scale rows this wave loads.  Edge
+  // tiles: rows past M (or N) lie beyond the end of the resource and read as zeros.  tile < 0: resources of
+  // length zero, loads through them fetch nothing.
+  __amdgpu_buffer_rsrc_t rA, rB, rS;
+  auto operand_rsrc = [&](int tile) __attribute__((always_inline)) {
+    const auto g = fresh_args();
+    const int pm = tile < 0 ? 0 : tile & 0xffff, pn = tile < 0 ? 0 : tile >> 16;
+    const int rows_a = tile < 0 ? 0 : min(kBM, g->M - pm * kBM), rows_b = tile < 0 ? 0 : min(kBN, g->N - pn * kBN);
+    rA = make_rsrc(g->A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
+    rB = make_rsrc(g->B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+  };
+  auto scale_rsrc = [&](int tile) __attribute__((always_inline)) {
+    const auto g = fresh_args();
+    const int pm = tile < 0 ? 0 : tile & 0xffff, pn = tile < 0 ? 0 : tile >> 16;
+    const int rows_a = tile < 0 ? 0 : min(kBM, g->M - pm * kBM), rows_b = tile < 0 ? 0 : min(kBN, g->N - pn * kBN);
+    const uint8_t* sp = sc_a ? g->As : g->Bs;
+    const int slay = sc_a ? layout_a : layout_b, srows = sc_a ? rows_a : rows_b, stile = sc_a ? pm : pn;
+    rS = slay ? make_rsrc(sp + (size_t)stile * (256 / 32) * nk4 * 512, (uint32_t)((srows + 31) / 32) * nk4 * 512)
+              : make_rsrc(sp + (size_t)stile * 256 * sbytes, (uint32_t)srows * sbytes);
+  };
+  int bid_next = blockIdx.x + gridDim.x;
+  int tile_cur = tile_of(blockIdx.x), tile_next = tile_of(bid_next);
+  operand_rsrc(tile_cur);
+  scale_rsrc(tile_cur);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int h = lane >> 5, r32 = lane & 31;
-
-  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK;
-  // edge tiles: rows past M (or N) lie beyond the end of the buffer resource and read as zeros
-  const int rows_a = min(kBM, M - pm * kBM), rows_b = min(kBN, N - pn * kBN);
-  const __amdgpu_buffer_rsrc_t rA = make_rsrc(A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
-  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
-  // tile-major scales: the 16 bytes a row has for four K-tiles, 32 rows adjacent (512-byte chunks, nk4 per row-tile)
-  const int nk4 = (nkt + 3) / 4;
-  const __amdgpu_buffer_rsrc_t rSA = layout_a ? make_rsrc(As + (size_t)pm * (kBM / 32) * nk4 * 512, (uint32_t)((rows_a + 31) / 32) * nk4 * 512)
-                                              : make_rsrc(As + (size_t)pm * kBM * sbytes, (uint32_t)rows_a * sbytes);
-  const __amdgpu_buffer_rsrc_t rSB = layout_b ? make_rsrc(Bs + (size_t)pn * (kBN / 32) * nk4 * 512, (uint32_t)((rows_b + 31) / 32) * nk4 * 512)
-                                              : make_rsrc(Bs + (size_t)pn * kBN * sbytes, (uint32_t)rows_b * sbytes);
 
   // per-lane global byte offsets of the OPS direct loads.  Load q = wave*OPS + i fills LDS bytes
   // [q*1024, q*1024 + 1024) of the operand tile.  Row-major operand: slot o holds piece
@@ -157,30 +191,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   const int sa_rd = kScaleBase + (wm * (TM * 32) + r32) * 16 + 2 * h;
   const int sb_rd = kScaleBase + kScStage + (wn * (TN * 32) + r32) * 16 + 2 * h;
 
-  v16f acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++)
-#pragma unroll
-      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+  v16f acc[TM][TN];  // never zeroed: the first K-tile of an output tile multiplies into a zero C operand
+
+  int p0 = 0;  // scale buffer that holds group 0 of the current output tile
 
   // ---- loads.  A wave's batch for K-tile t is its 2*OPS operand loads (n = 0..OPS-1: A, then B) and,
   // when t % 4 == 2, the scale load for the four K-tiles starting at t + 2 (at the end of the batch, so
   // that a wait that leaves a whole batch in flight also covers the scales of the batch before).
-  auto issue_scales = [&](int grp) __attribute__((always_inline)) {
-    const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + (wave & 3) * 1024;
-    const int soff = grp * sstep;
-    if (wave < 4) dma16(rSA, dst, voff_s, soff); else dma16(rSB, dst + kScStage, voff_s, soff);
+  // K-tile (or group of four K-tiles) number kk counts on from the current output tile into the next one.
+  // The resources rA, rB (and rS) are those of the output tile the loads have reached: they move on to the
+  // next output tile just before the first load that belongs to it, and past the workgroup's last output
+  // tile to empty resources.  INSIDE says that the caller knows kk to lie in the current tile.
+  auto issue_scales = [&]<bool INSIDE>(int grp) __attribute__((always_inline)) {
+    const int buf = (p0 + grp) & 1;
+    const uint32_t dst = lds0 + kScaleBase + buf * kScaleBuf + (wave & 3) * 1024;
+    dma16(rS, sc_a ? dst : dst + kScStage, voff_s, (INSIDE || grp < nk4 ? grp : grp - nk4) * sstep);
   };
-  auto issue_one = [&](int t, int slot, int n) __attribute__((always_inline)) {
+  auto issue_one = [&]<bool INSIDE>(int kk, int slot, int n) __attribute__((always_inline)) {
+    const int t = INSIDE || kk < nkt ? kk : kk - nkt;
     const uint32_t dst = lds0 + slot * kStage + wave * (OPS * 1024);
     if (n < OPS) dma16(rA, dst + n * 1024, voff_a[n], t * kstep_a);
     else dma16(rB, dst + kOpStage + (n - OPS) * 1024, voff_b[n - OPS], t * kstep_b);
-  };
-  auto issue_ops = [&](int t, int slot) __attribute__((always_inline)) {
-#pragma unroll
-    for (int n = 0; n < 2 * OPS; n++) issue_one(t, slot, n);
   };
 
   // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
@@ -213,16 +244,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
     }
   };
   // first K-block of every lane for all tiles, then the second: two MFMAs into the same accumulator
-  // are TM*TN instructions apart.  First source = B rows (index n), second = A rows (index m): a
-  // lane ends up owning 4 consecutive n of one m.  between(i) runs after the i-th MFMA.
-  auto mma_tile = [&](auto&& between) __attribute__((always_inline)) {
+  // are TM*TN instructions apart.  First source = B rows (index n), second = A rows (index m): a lane
+  // ends up owning 4 consecutive n of row m = lane % 32, four times.  FIRST: the K-tile opens an output tile,
+  // so the first MFMA into every accumulator takes zero as its C operand.  between(i) runs after the i-th MFMA.
+  auto mma_tile = [&]<bool FIRST>(auto&& between) __attribute__((always_inline)) {
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const v8i a0 = __builtin_shufflevector(fa[i], fa[i], 0, 1, 2, 3, 4, 5, -1, -1);
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const v8i b0 = __builtin_shufflevector(fb[j], fb[j], 0, 1, 2, 3, 4, 5, -1, -1);
-        acc[i][j] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[i][j], scb[j], sca[i]);
+        acc[i][j] = mfma_fp6<FB, FA, 0, 0>(b0, a0, FIRST ? zero : acc[i][j], scb[j], sca[i]);
         between(i * TN + j);
       }
     }
@@ -249,22 +282,32 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
   // one of tile k: group 1's compute cluster starts at barrier 2k+2, by which both groups have read
   // tile k.  In program order every tile's batch is contiguous for both groups, so one wait count
   // serves both: everything older than the newest batch has landed.
-  // The body is instantiated per group (GRP) and per k mod 4 (KM), so the steady state carries no
-  // branch: STEADY means tiles k+2, k+3 and (for the scales) k+4 exist.
+  // The K-tiles of all output tiles of a workgroup form ONE stream: K-tile k+2 or k+3 past the end of
+  // an output tile is K-tile 0, 1 or 2 of the workgroup's next output tile, so the ring never drains
+  // between output tiles, and the finished tile's stores run while the other group still multiplies.
+  // Past the last output tile the stream continues with loads through an empty buffer resource: they
+  // fetch nothing and fill ring slots nobody reads, which keeps every step's load and wait pattern the same.
+  // The body is instantiated per group (GRP) and per k mod 4 (KM); STEADY means that tiles k+2, k+3 and
+  // (for the scales) k+4 lie in the current output tile, so its loads need no choice of descriptor.
   int stage = 0, stage2 = 2;  // ring slots of tile k and tile k+2
-  auto step = [&]<int GRP, int KM, bool STEADY>(int kt) __attribute__((always_inline)) {
+  auto step = [&]<int GRP, int KM, bool STEADY, bool FIRST>(int kt) __attribute__((always_inline)) {
     constexpr int AHEAD = GRP == 0 ? 2 : 3;
-    const bool has2 = STEADY || kt + 2 < nkt;             // tile kt+2 exists
-    const bool hasx = STEADY || kt + AHEAD < nkt;         // the tile the compute-cluster loads belong to exists
-    const bool has_sc = STEADY || kt + 4 < nkt;           // the scales this step's batch would carry exist
+    // outside the steady state every step derives its offsets and choices from kt on the spot: related to each
+    // other across the steps of a trip they become a few dozen induction variables in scalar registers
+    if (!STEADY) asm volatile("" : "+s"(kt));
     const int slotx = GRP == 0 ? stage2 : stage;
-    read_tile(stage, ((kt >> 2) & 1) * kScaleBuf + KM * 4);
+    read_tile(stage, ((p0 + (kt >> 2)) & 1) * kScaleBuf + KM * 4);
     __builtin_amdgcn_sched_barrier(0);
-    if (has2) {
+    // the loads reach the next output tile: group 0's with K-tile kt+2 at the start of a step, group 1's
+    // with K-tile kt+3 in its compute cluster; the scales with group nk4
+    if (!STEADY && GRP == 0 && kt + 2 == nkt) operand_rsrc(tile_next);
 #pragma unroll
-      for (int n = kLoadsInCompute; n < 2 * OPS; n++) issue_one(kt + 2, stage2, n);
-      if (KM == 0 && has_sc) issue_scales((kt + 4) >> 2);
+    for (int n = kLoadsInCompute; n < 2 * OPS; n++) issue_one.template operator()<STEADY>(kt + 2, stage2, n);
+    if (KM == 0) {
+      if (!STEADY && (kt + 4) >> 2 == nk4) scale_rsrc(tile_next);
+      issue_scales.template operator()<STEADY>((kt + 4) >> 2);
     }
+    if (!STEADY && GRP == 1 && kt + 3 == nkt) operand_rsrc(tile_next);
     wait_lds_reads();  // this tile's LDS reads are done before anyone may refill its slot
     // the middle 16-byte piece straddles the two operands; naming each fragment as one 384-bit value here
     // makes the register allocator keep it in one tuple, and the MFMAs read sub-tuples of it instead of
@@ -273,122 +316,193 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const uint8_t* __re
     for (int i = 0; i < TM; i++) asm volatile("" : "+v"(fa[i]));
 #pragma unroll
     for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
-    auto wait_next = [&]() __attribute__((always_inline)) {  // own share of tile kt+1 has landed; tile kt+2's batch may be in flight
-      if (has2) {
-        if (KM == 0 && has_sc) wait_vmcnt<2 * OPS + SCL>(); else wait_vmcnt<2 * OPS>();
-      } else {
-        wait_vmcnt<0>();
-      }
-    };
-    if (GRP == 1) wait_next();
+    // own share of the next K-tile has landed; the batch after it may be in flight
+    if (GRP == 1) wait_vmcnt<2 * OPS + (KM == 0 ? SCL : 0)>();
     barrier();
     __builtin_amdgcn_s_setprio(1);
-    mma_tile([&](int i) __attribute__((always_inline)) {
-      if (hasx && (i & 1) && i / 2 < kLoadsInCompute) {
+    mma_tile.template operator()<FIRST>([&](int i) __attribute__((always_inline)) {
+      if ((i & 1) && i / 2 < kLoadsInCompute) {
         __builtin_amdgcn_sched_barrier(0);
-        issue_one(kt + AHEAD, slotx, i / 2);
+        issue_one.template operator()<STEADY>(kt + AHEAD, slotx, i / 2);
         __builtin_amdgcn_sched_barrier(0);
       }
     });
     __builtin_amdgcn_s_setprio(0);
-    if (GRP == 0) wait_next();
+    if (GRP == 0) wait_vmcnt<2 * OPS + (KM == 0 ? SCL : 0)>();
     barrier();
     stage = stage == kStages - 1 ? 0 : stage + 1;
     stage2 = stage2 == kStages - 1 ? 0 : stage2 + 1;
   };
   auto k_loop = [&]<int GRP>() __attribute__((always_inline)) {
-    int kt = 0;
+    // first four K-tiles of the output tile (the first of them starts the accumulators)
+    if (nkt >= 8) {
+      step.template operator()<GRP, 0, true, true>(0);
+      step.template operator()<GRP, 1, true, false>(1);
+      step.template operator()<GRP, 2, true, false>(2);
+      step.template operator()<GRP, 3, true, false>(3);
+    } else {
+      step.template operator()<GRP, 0, false, true>(0);
+      if (1 < nkt) step.template operator()<GRP, 1, false, false>(1);
+      if (2 < nkt) step.template operator()<GRP, 2, false, false>(2);
+      if (3 < nkt) step.template operator()<GRP, 3, false, false>(3);
+    }
+    int kt = 4;
     for (; kt + 8 <= nkt; kt += 4) {  // four tiles per trip, all of them with tiles kt+2 .. kt+7 in range
-      step.template operator()<GRP, 0, true>(kt);
-      step.template operator()<GRP, 1, true>(kt + 1);
-      step.template operator()<GRP, 2, true>(kt + 2);
-      step.template operator()<GRP, 3, true>(kt + 3);
+      step.template operator()<GRP, 0, true, false>(kt);
+      step.template operator()<GRP, 1, true, false>(kt + 1);
+      step.template operator()<GRP, 2, true, false>(kt + 2);
+      step.template operator()<GRP, 3, true, false>(kt + 3);
     }
     for (; kt < nkt; kt += 4) {  // last (up to seven) tiles: same body with the range checks
-      step.template operator()<GRP, 0, false>(kt);
-      if (kt + 1 < nkt) step.template operator()<GRP, 1, false>(kt + 1);
-      if (kt + 2 < nkt) step.template operator()<GRP, 2, false>(kt + 2);
-      if (kt + 3 < nkt) step.template operator()<GRP, 3, false>(kt + 3);
+      step.template operator()<GRP, 0, false, false>(kt);
+      if (kt + 1 < nkt) step.template operator()<GRP, 1, false, false>(kt + 1);
+      if (kt + 2 < nkt) step.template operator()<GRP, 2, false, false>(kt + 2);
+      if (kt + 3 < nkt) step.template operator()<GRP, 3, false, false>(kt + 3);
+    }
+  };
+
+  // ---- epilogue of one output tile, straight from the accumulators.  Register v of lane l is C[m][n] with
+  // m = l % 32 and n = 8 (v / 4) + 4 (l / 32) + v % 4 inside every 32x32 tile: lanes l and l + 32 hold the two
+  // halves of each run of 8 consecutive n of one row.  bf16: after the conversion the two lanes trade halves
+  // (v_permlane32_swap: the upper lanes' first run for the lower lanes' second), so that every lane owns 8
+  // consecutive outputs and stores them as 16 bytes; two stores complete a row's 64-byte sector and four its
+  // 128-byte line, back to back.  (8 bytes per lane and row, the accumulators as they are, measured 1.4x the
+  // output in HBM write traffic; 4 bytes per lane with rows down the lanes, 64 stores per wave, measured
+  // ~47 clocks per store instruction.)  Nothing here touches LDS, so the ring keeps streaming the next output
+  // tile meanwhile.  The stores count in vmcnt like the loads and retire in order with them, so the waits of
+  // the K loop ("all but the newest batch") stay valid.
+  // EDGE: the tile has fewer than 256 valid rows or columns; those stores are predicated per lane.
+  typedef typename Out::type OutT;
+  auto epilogue = [&]<bool EDGE>(int rows_a, int rows_b) __attribute__((always_inline)) {
+    const auto g = fresh_args();
+    const int N = g->N, N2 = N * (int)sizeof(OutT);  // N2: bytes per row of C
+    // the resource ends with the tile's last valid element
+    const __amdgpu_buffer_rsrc_t rC = make_rsrc((OutT*)g->C + (size_t)(tile_cur & 0xffff) * kBM * N + (size_t)(tile_cur >> 16) * kBN,
+                                                (uint32_t)((rows_a - 1) * N + rows_b) * (uint32_t)sizeof(OutT));
+    const int row_l = wm * (TM * 32) + r32;
+    if constexpr (sizeof(OutT) == 2) {
+      const int col_l = wn * (TN * 32) + 8 * h;
+      const int voff = row_l * N2 + col_l * 2;
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        // each phase for the whole 32-row band before the next one, so that no dword waits for its predecessor
+        uint32_t pk[TN][8];
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) pk[j][e] = pack_bf16x2(acc[i][j][2 * e], acc[i][j][2 * e + 1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+              // runs 2t and 2t+1 (dwords 4t+c and 4t+2+c): lower lanes keep run 2t and get the partner's, upper lanes run 2t+1
+              const auto sw = __builtin_amdgcn_permlane32_swap(pk[j][4 * t + c], pk[j][4 * t + 2 + c], false, false);
+              pk[j][4 * t + c] = sw[0], pk[j][4 * t + 2 + c] = sw[1];
+            }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int t = 0; t < 2; t++) {
+            const v4i v = {(int)pk[j][4 * t], (int)pk[j][4 * t + 1], (int)pk[j][4 * t + 2], (int)pk[j][4 * t + 3]};
+            if (!EDGE || (row_l + i * 32 < rows_a && col_l + j * 32 + t * 16 < rows_b))
+              __builtin_amdgcn_raw_buffer_store_b128(v, rC, voff + j * 64 + t * 32, i * 32 * N2, 0);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      const int col_l = wn * (TN * 32) + 4 * h;
+      const int voff = row_l * N2 + col_l * 4;
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int gq = 0; gq < 4; gq++) {
+            const v4f f = {acc[i][j][4 * gq], acc[i][j][4 * gq + 1], acc[i][j][4 * gq + 2], acc[i][j][4 * gq + 3]};
+            if (!EDGE || (row_l + i * 32 < rows_a && col_l + j * 32 + gq * 8 < rows_b))
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, f), rC, voff + j * 128 + gq * 32, i * 32 * N2, 0);
+          }
+    }
+  };
+
+  // ---- all output tiles of this workgroup
+  auto run = [&]<int GRP>() __attribute__((always_inline)) {
+    for (;;) {
+      k_loop.template operator()<GRP>();
+      {
+        const auto g = fresh_args();
+        const int rows_a = min(kBM, g->M - (tile_cur & 0xffff) * kBM), rows_b = min(kBN, g->N - (tile_cur >> 16) * kBN);
+        if (rows_a == kBM && rows_b == kBN) epilogue.template operator()<false>(rows_a, rows_b);
+        else epilogue.template operator()<true>(rows_a, rows_b);
+      }
+      if (tile_next < 0) break;
+      p0 = (p0 + nk4) & 1;
+      tile_cur = tile_next;
+      bid_next += gridDim.x;
+      tile_next = tile_of(bid_next);
     }
   };
 
   // prologue: scales of the first four K-tiles, K-tiles 0 and 1 and, for group 1, the loads of tile 2
   // that its compute cluster of "step -1" would have issued; tile 0 must have landed everywhere
-  issue_scales(0);
-  issue_ops(0, 0);
-  if (nkt > 1) issue_ops(1, 1);
-  if (wm == 1 && nkt > 2 && kLoadsInCompute > 0) {
+  issue_scales.template operator()<true>(0);
 #pragma unroll
-    for (int n = 0; n < kLoadsInCompute; n++) issue_one(2, 2, n);
+  for (int n = 0; n < 2 * OPS; n++) issue_one.template operator()<true>(0, 0, n);
+#pragma unroll
+  for (int n = 0; n < 2 * OPS; n++) issue_one.template operator()<false>(1, 1, n);
+  if (wm == 1) {
+#pragma unroll
+    for (int n = 0; n < kLoadsInCompute; n++) issue_one.template operator()<false>(2, 2, n);
     wait_vmcnt<2 * OPS + kLoadsInCompute>();
-  } else if (nkt > 1) {
-    wait_vmcnt<2 * OPS>();
   } else {
-    wait_vmcnt<0>();
+    wait_vmcnt<2 * OPS>();
   }
   barrier();
   if (wm == 0) {
-    k_loop.template operator()<0>();
+    run.template operator()<0>();
     barrier();  // every wave executes the same number of barriers
   } else {
     barrier();  // phase offset of group 1
-    k_loop.template operator()<1>();
+    run.template operator()<1>();
   }
-
-  // ---- epilogue.  A lane owns C[m][n .. n+3] for four values of n per 32x32 tile, i.e. 8 bytes of
-  // bf16 per store: written straight to global memory those are partial-line writes (measured 1.4x
-  // the output in HBM write traffic and a visible tail after every tile).  The bf16 tile (128 KB)
-  // is therefore staged through LDS, which is free once the K loop is over, and written out in
-  // whole rows: one wave store = two rows x 512 contiguous bytes.
-  if constexpr (sizeof(typename Out::type) == 2) {
-    constexpr int kRowPitch = 512 + 16;  // bytes; the pad spreads the 32 rows of a store over the banks
-    static_assert(256 * kRowPitch <= kLdsBytes, "C tile fits the ring");
-    __syncthreads();  // every wave is done reading the ring
-    uint8_t* cs = smem + (wm * (TM * 32) + r32) * kRowPitch + (wn * (TN * 32) + 4 * h) * 2;
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const u32x2 v = {pack_bf16x2(acc[i][j][4 * g], acc[i][j][4 * g + 1]), pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
-          *reinterpret_cast<u32x2*>(cs + i * 32 * kRowPitch + (j * 32 + 8 * g) * 2) = v;
-        }
-    __syncthreads();
-    const int chunk = tid & 31, row0 = tid >> 5;  // 32 lanes cover one 512-byte row
-    uint8_t* cg = reinterpret_cast<uint8_t*>(C) + ((size_t)pm * kBM + row0) * (size_t)N * 2 + (size_t)pn * kBN * 2 + chunk * 16;
-    constexpr int kRowsPerPass = NW * 2;
-    const bool col_ok = chunk * 8 < rows_b;  // N % 8 == 0: a 16-byte piece is inside or outside as a whole
-#pragma unroll 4
-    for (int r = 0; r < 256; r += kRowsPerPass) {
-      const v4i v = *reinterpret_cast<const v4i*>(smem + (row0 + r) * kRowPitch + chunk * 16);
-      if (col_ok && row0 + r < rows_a) *reinterpret_cast<v4i*>(cg + (size_t)r * N * 2) = v;
-    }
-  } else {
-    typename Out::type* cbase = C + ((size_t)pm * kBM + wm * (TM * 32) + r32) * (size_t)N + (size_t)pn * kBN + wn * (TN * 32) + 4 * h;
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int g = 0; g < 4; g++)
-          if (wm * (TM * 32) + i * 32 + r32 < rows_a && wn * (TN * 32) + j * 32 + 8 * g + 4 * h < rows_b)
-            store4(cbase + (size_t)i * 32 * N + j * 32 + 8 * g, acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                   acc[i][j][4 * g + 3]);
-  }
+  wait_vmcnt<0>();  // no direct load may still be on its way into LDS when the workgroup gives the memory back
 }
 
 bool gemm_tiled_supports(const GemmArgs& g) {
-  // any M; N % 8 keeps every 16-byte output piece whole and aligned; K in whole K-tiles
+  // any M; N % 8 keeps every pair of bf16 outputs whole and aligned; K in whole K-tiles; 32-bit byte
+  // offsets inside one tile's operand rows and inside one tile's rows of C
   return g.M > 0 && g.N > 0 && g.K > 0 && g.N % 8 == 0 && g.K % kBK == 0 && (long)kBM * (g.K / 4 * 3) < (1L << 31) &&
-         ((uintptr_t)g.C % 16) == 0;
+         (long)kBM * g.N * 4 < (1L << 31) && g.M <= 65535 * kBM && ((uintptr_t)g.C % 16) == 0;
+}
+
+// Workgroups to launch: one per output tile, or, when the tiles outnumber the compute units (one
+// workgroup of this kernel fills a CU's LDS), one per CU, each walking through several tiles.  The
+// scales of the next output tile are fetched with the last group of four K-tiles of the current one
+// and must have two steps to land: K-tile counts of 4n+1 (and fewer than four K-tiles) keep one
+// workgroup per tile.
+static int grid_size(const GemmArgs& g, int tiles) {
+  static int cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return tiles;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return tiles;
+    cus[dev] = n & ~7;  // whole multiples of the 8 XCDs keep the tile -> XCD mapping of the walk
+  }
+  const int nkt = g.K / kBK;
+  if (g_tiled_walk == 0 || nkt < 4 || nkt % 4 == 1 || cus[dev] < 8) return tiles;
+  return tiles < cus[dev] ? tiles : cus[dev];
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int tm = (g.M + kBM - 1) / kBM, tn = (g.N + kBN - 1) / kBN;
-  gemm_tiled_kernel<FA, FB, Out><<<tm * tn, NW * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, tm, tn,
-                                                            g.layout_a, g.layout_b);
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b};
+  gemm_tiled_kernel<FA, FB, Out><<<grid_size(g, tm * tn), NW * 64, 0, s>>>(ta);
   return hipGetLastError();
 }
 

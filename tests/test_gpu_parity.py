@@ -302,6 +302,38 @@ def test_automatic_dispatch_agrees_with_generic_kernel_on_ragged_shapes(hk):
         assert o.rel_err(got, ref) <= TOL_TIGHT, (M, N, K, la, lb, o.rel_err(got, ref))
 
 
+# ------------------------------------------------------------------ workgroups that walk through several output tiles
+@pytest.mark.parametrize("M,N,K,la,lb", [(8192, 8192, 512, 0, 0), (8192, 8192, 768, 0, 0), (8192, 8192, 896, 1, 1), (8192, 8192, 640, 0, 0),
+                                         (5000, 5000, 1024, 0, 0), (4352, 4352, 1280, 0, 1), (4128, 8200, 2048, 0, 0), (8192, 16384, 1152, 1, 0)])
+@pytest.mark.parametrize("out", [torch.float32, torch.bfloat16])
+def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, lb, out):
+    """More output tiles than compute units: every workgroup of the tiled kernel takes several tiles in turn, the loads of
+    the next tile running under the last K-tiles of the current one (K-tile counts 4n, 4n+2, 4n+3; 4n+1 keeps one workgroup
+    per tile), with ragged edge tiles and tile-major operands.  The result must equal the one-wave-per-tile kernel's in every
+    bit (both round the same fp32 sums once), and nothing may be written outside C (guard rows before and after it)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(M + N + K)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2, layout=la)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.05, 2, layout=lb)
+    prev_r = hk.tk_kernel.set_relayout(0)
+    res = []
+    try:
+        for kern in (1, 2):
+            full = torch.full((M + 2, N), 12345.0, dtype=out, device="cuda")
+            prev = hk.tk_kernel.set_kernel(kern)
+            try:
+                hk.dispatch_micro(a, b, asc, bsc, full[1:M + 1], 2, 2, layout_a=la, layout_b=lb)
+                torch.cuda.synchronize()
+            finally:
+                hk.tk_kernel.set_kernel(prev)
+            res.append(full)
+    finally:
+        hk.tk_kernel.set_relayout(prev_r)
+    ref, got = res
+    assert bool((got[0] == 12345.0).all()) and bool((got[-1] == 12345.0).all())
+    assert torch.equal(ref[1:-1], got[1:-1])
+
+
 # ------------------------------------------------------------------ stream capture
 def test_graph_capture_replays_match_eager(hk):
     """A size at which the eager path takes the re-layout pre-pass (workspace from the stream-ordered allocator): under
