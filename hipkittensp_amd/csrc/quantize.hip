@@ -152,15 +152,17 @@ hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K,
 }
 
 // Row-major -> tile-major for up to two operands (packed bytes and scales) in one launch: the re-layout pre-pass of
-// the gemm entry points, where every extra launch would cost as much as part of the copy.  One lane writes one
-// 16-byte piece of the destination (consecutive lanes: consecutive bytes of a tile-major operand, i.e. whole 3 KB
-// tiles) or the 16 scale bytes one row has for four K-tiles.
+// the gemm entry points, where every extra launch would cost as much as part of the copy.  A workgroup copies 32
+// rows x four K-tiles (384 source bytes per row = three whole cache lines; a single K-tile's 96 bytes straddle
+// lines, and lines shared between workgroups on different XCDs were fetched twice: 1.64x read traffic) in source
+// order: consecutive lanes read consecutive 16-byte pieces of a row and write runs of 96 bytes into the four 3 KB
+// tiles.  Other workgroups move the 16 scale bytes one row has for four K-tiles, one row per lane.
 struct TileJob {
   const uint8_t* src;
   uint8_t* dst;
   const uint8_t* ssrc;
   uint8_t* sdst;
-  long npieces, nchunks;
+  long ngroups, nchunks;  // groups of 32 rows x four K-tiles; (row, four K-tiles) scale chunks
   unsigned pblocks, sblocks;
 };
 
@@ -170,15 +172,18 @@ __global__ __launch_bounds__(256) void tile_both_kernel(TileJob j0, TileJob j1, 
   if (second) bid -= j0.pblocks + j0.sblocks;
   const TileJob& j = second ? j1 : j0;
   if (bid < j.pblocks) {
-    const long d = (long)bid * 256 + threadIdx.x;  // destination piece
-    if (d >= j.npieces) return;
-    // destination piece d lives in tile d / 192 = rt * nkt + kt, slot d % 192 = r * 6 + (c ^ ((r >> 3) & 1))
-    const long tile = d / 192;
-    const int in = (int)(d - tile * 192), r = in / 6, c = (in - r * 6) ^ ((r >> 3) & 1);
-    const long rt = tile / nkt;
-    const int kt = (int)(tile - rt * nkt);
-    const size_t so = ((size_t)(rt * 32 + r) * nkt + kt) * 96 + (size_t)c * 16;
-    *reinterpret_cast<v4i*>(j.dst + (size_t)d * 16) = *reinterpret_cast<const v4i*>(j.src + so);
+    const int rt = bid / nk4, g = bid - rt * nk4;  // row-tile, group of four K-tiles
+    const int ntile = min(4, nkt - 4 * g);
+    const uint8_t* src = j.src + ((size_t)rt * 32 * nkt + 4 * g) * 96;
+    uint8_t* dst = j.dst + ((size_t)rt * nkt + 4 * g) * 3072;
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      const int p = threadIdx.x + 256 * i, r = p / 24, q = p - r * 24;  // piece q of the row's 384 bytes
+      const int tg = q / 6, c = q - tg * 6;
+      if (tg < ntile)
+        *reinterpret_cast<v4i*>(dst + tg * 3072 + (r * 6 + (c ^ ((r >> 3) & 1))) * 16) =
+            *reinterpret_cast<const v4i*>(src + (size_t)r * nkt * 96 + q * 16);
+    }
   } else {
     const long s = (long)(bid - j.pblocks) * 256 + threadIdx.x;
     if (s >= j.nchunks) return;
@@ -196,8 +201,8 @@ hipError_t launch_tile_both(const uint8_t* src0, uint8_t* dst0, const uint8_t* s
                             uint8_t* dst1, const uint8_t* ssrc1, uint8_t* sdst1, int rows1, int K, hipStream_t s) {
   const int nkt = K / 128, nkb = K / 32, nk4 = (nkb + 15) / 16;
   auto job = [&](const uint8_t* src, uint8_t* dst, const uint8_t* ssrc, uint8_t* sdst, int rows) {
-    TileJob j{src, dst, ssrc, sdst, (long)rows * nkt * 6, (long)rows * nk4, 0, 0};
-    j.pblocks = (unsigned)((j.npieces + 255) / 256);
+    TileJob j{src, dst, ssrc, sdst, (long)(rows / 32) * nk4, (long)rows * nk4, 0, 0};
+    j.pblocks = (unsigned)j.ngroups;
     j.sblocks = (unsigned)((j.nchunks + 255) / 256);
     return j;
   };
