@@ -105,8 +105,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   hipError_t e;
   if (force == 1) {
     e = mxfp6::launch_gemm_generic(g, s);
-  } else if (force == 2) {
+  } else if (force == 2 || force == 5 || force == 6) {
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
+    g.tile_rows = force == 5 ? 128 : force == 6 ? 256 : 0;
     e = mxfp6::launch_gemm_tiled(g, s);
   } else if (force == 3) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
@@ -171,7 +172,7 @@ int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, voi
 int mxfp6_set_relayout(int on) { return g_relayout.exchange(on ? 1 : 0); }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 4) return g_force.load();
+  if (which < 0 || which > 6) return g_force.load();
   return g_force.exchange(which);
 }
 
@@ -208,7 +209,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 103; }
+int mxfp6_abi_version(void) { return 104; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -276,15 +276,24 @@ static bool mid_wide(const GemmArgs& g) {
   return narrow > 256 && (!g.layout_b || g.N % 64 == 0) && (long)64 * (g.K / 4 * 3) < (1L << 31);
 }
 
-// Automatic choice against the 256x256 tiling: rounds of workgroups x time per K-tile and round of the two candidates
-// (the constants are measured, in microseconds: this kernel 0.36 / 0.50 for BM = 64 / 128, the tiled kernel 1.2).
+// Estimated time of this kernel in microseconds: rounds of workgroups x K-tiles x time per K-tile and round.
+// Constants measured on MI355X (N = 8192 and 28672, K = 8192): 0.33 / 0.48 us for 64 rows of A with 32 / 64
+// rows of B per workgroup, 0.45 / 0.55 us for 128 rows of A; row-major B costs about 6 % more; 5 us fixed.
+double mid_estimate_us(const GemmArgs& g) {
+  const bool wide = mid_wide(g);
+  const int bn = wide ? 64 : 32;
+  const double wgs = (double)((g.N + bn - 1) / bn) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
+  const double rounds = wgs > 256 ? wgs / 256 : 1;
+  const double c = g.M <= 64 ? (wide ? 0.48 : 0.33) : (wide ? 0.55 : 0.45);
+  return 5.0 + rounds * (g.K / 128) * c * (g.layout_b ? 1.0 : 1.06);
+}
+
+// Automatic choice against the LDS-tiled kernel with either tile height.
 bool gemm_mid_preferred(const GemmArgs& g) {
   if (!gemm_mid_supports(g)) return false;
-  const double tiles256 = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  const int bn = mid_wide(g) ? 64 : 32;
-  const double wgs = (double)((g.N + bn - 1) / bn) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
-  const double rounds_mid = wgs > 256 ? wgs / 256 : 1, rounds_tiled = tiles256 > 256 ? tiles256 / 256 : 1;
-  return rounds_mid * (g.M <= 64 ? 0.36 : 0.50) < rounds_tiled * 1.2;
+  if (!gemm_tiled_supports(g)) return true;
+  const double t = mid_estimate_us(g);
+  return t < tiled_estimate_us(g, 128) && t < tiled_estimate_us(g, 256);
 }
 
 template <int FA, int FB, typename Out>

@@ -51,20 +51,28 @@ namespace mxfp6 {
 
 int g_tiled_walk = 1;  // 0: always one workgroup per output tile (development switch)
 
-constexpr int kBM = 256, kBN = 256, kBK = 128;
-constexpr int kOpStage = 256 * 96;  // bytes of one operand tile
-constexpr int kScStage = 256 * 16;  // bytes of one operand's scales for four K-tiles
+constexpr int kBN = 256, kBK = 128;  // the tile has 256 (TM = 4) or 128 (TM = 2) rows of A
+constexpr int kScStage = 256 * 16;   // bytes of one operand's scales for four K-tiles
 constexpr int kGroupM = 4;          // tile rows per raster group
 constexpr int kStages = 3;          // operand ring depth
-constexpr int kStage = 2 * kOpStage, kScaleBase = kStages * kStage, kScaleBuf = 2 * kScStage;
-constexpr int kLdsBytes = kScaleBase + 2 * kScaleBuf;
-constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile 128 x 64
-constexpr int TM = 8 / WM, TN = 8 / WN;      // 32x32 MFMA tiles per wave in M and N
-constexpr int OPS = 24 / NW;                 // operand direct loads per wave per operand per K-tile
+constexpr int kScaleBuf = 2 * kScStage;
+constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile (TM * 32) x 64
+constexpr int TN = 8 / WN;                   // 32x32 MFMA tiles per wave in N; in M: TM, a template parameter (4 or 2)
+constexpr int OPB = 24 / NW;                 // direct loads per wave and K-tile for B's 256 rows
 constexpr int SCL = 1;                       // scale direct loads per wave per slot that carries scales
-constexpr int kLoadsInCompute = 4;           // of the 2*OPS operand loads per wave and K-tile: issued between MFMAs
-static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= 2 * OPS && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
-static_assert(kLdsBytes <= 163840, "LDS budget");
+constexpr int kLoadsInCompute = 4;           // of the operand loads per wave and K-tile: issued between MFMAs
+// Per tile height.  A's 128 rows are 12 loads of 1 KB for 8 waves: every wave issues two, and the last four of
+// the sixteen lie past the end of A's buffer resource (they fetch nothing and fill padding behind the A tile).
+template <int TM>
+struct Shape {
+  static constexpr int BM = WM * TM * 32;
+  static constexpr int OPA = (BM * 96 / 1024 + NW - 1) / NW;  // direct loads per wave and K-tile for A
+  static constexpr int NL = OPA + OPB;                        // operand loads per wave and K-tile
+  static constexpr int kAStage = OPA * NW * 1024, kStage = kAStage + kBN * 96;  // LDS bytes of A's tile (padded), of a ring slot
+  static constexpr int kScaleBase = kStages * kStage, kLdsBytes = kScaleBase + 2 * kScaleBuf;
+  static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= NL && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
+  static_assert(kLdsBytes <= 163840, "LDS budget");
+};
 
 // One direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff and the hardware
 // writes them at LDS address lds_base + 16 * lane.  Issued from inline assembly so that the VMEM
@@ -96,10 +104,12 @@ struct TiledArgs {
   int M, N, K, tiles_m, tiles_n, layout_a, layout_b;
 };
 
-template <int FA, int FB, typename Out>
+template <int FA, int FB, typename Out, int TM>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
+  typedef Shape<TM> S;
+  constexpr int kBM = S::BM, OPA = S::OPA, NL = S::NL, kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase;
   // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[kLdsBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[S::kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
   const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
   const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK;
@@ -146,8 +156,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const int rows_a = tile < 0 ? 0 : min(kBM, g->M - pm * kBM), rows_b = tile < 0 ? 0 : min(kBN, g->N - pn * kBN);
     const uint8_t* sp = sc_a ? g->As : g->Bs;
     const int slay = sc_a ? layout_a : layout_b, srows = sc_a ? rows_a : rows_b, stile = sc_a ? pm : pn;
-    rS = slay ? make_rsrc(sp + (size_t)stile * (256 / 32) * nk4 * 512, (uint32_t)((srows + 31) / 32) * nk4 * 512)
-              : make_rsrc(sp + (size_t)stile * 256 * sbytes, (uint32_t)srows * sbytes);
+    const int sheight = sc_a ? kBM : kBN;  // rows per tile of the operand whose scales these are
+    rS = slay ? make_rsrc(sp + (size_t)stile * (sheight / 32) * nk4 * 512, (uint32_t)((srows + 31) / 32) * nk4 * 512)
+              : make_rsrc(sp + (size_t)stile * sheight * sbytes, (uint32_t)srows * sbytes);
   };
   int bid_next = blockIdx.x + gridDim.x;
   int tile_cur = tile_of(blockIdx.x), tile_next = tile_of(bid_next);
@@ -159,21 +170,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   const int wm = wave / WN, wn = wave % WN;
   const int h = lane >> 5, r32 = lane & 31;
 
-  // per-lane global byte offsets of the OPS direct loads.  Load q = wave*OPS + i fills LDS bytes
-  // [q*1024, q*1024 + 1024) of the operand tile.  Row-major operand: slot o holds piece
+  // per-lane global byte offsets of the direct loads.  Load q = wave*OPA + i (A) or wave*OPB + i (B) fills
+  // LDS bytes [q*1024, q*1024 + 1024) of the operand tile.  Row-major operand: slot o holds piece
   // (o%6) ^ ((row>>3)&1) of row o/6, K-tile t starts at byte 96 t of a row.  Tile-major operand:
   // the 3072-byte tile of 32 rows is stored in exactly this order, so the load is one contiguous
   // KiB, row-tiles are (K/128)*3072 bytes apart and K-tile t starts at byte 3072 t.
-  int voff_a[OPS], voff_b[OPS];
-#pragma unroll
-  for (int i = 0; i < OPS; i++) {
-    const int q = wave * OPS + i, o = q * 64 + lane;  // linear 16-byte slot inside the LDS image
+  int voff_a[OPA], voff_b[OPB];
+  auto load_offset = [&](int q, int layout) __attribute__((always_inline)) {
+    const int o = q * 64 + lane;  // linear 16-byte slot inside the LDS image
     const int r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
     const int vrow = r * rowbytes + c * 16;
     const int vtile = (q / 3) * (nkt * 3072) + (q % 3) * 1024 + lane * 16;
-    voff_a[i] = layout_a ? vtile : vrow;
-    voff_b[i] = layout_b ? vtile : vrow;
-  }
+    return layout ? vtile : vrow;
+  };
+#pragma unroll
+  for (int i = 0; i < OPA; i++) voff_a[i] = load_offset(wave * OPA + i, layout_a);
+#pragma unroll
+  for (int i = 0; i < OPB; i++) voff_b[i] = load_offset(wave * OPB + i, layout_b);
   const int kstep_a = layout_a ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
   // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; waves 0-3 load A's, 4-7 B's
   const int srow = (wave & 3) * 64 + lane, slay = wave < 4 ? layout_a : layout_b;
@@ -186,7 +199,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
   for (int c = 0; c < 3; c++) {
     a_rd[c] = (wm * (TM * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
-    b_rd[c] = kOpStage + (wn * (TN * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
+    b_rd[c] = kAStage + (wn * (TN * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
   }
   const int sa_rd = kScaleBase + (wm * (TM * 32) + r32) * 16 + 2 * h;
   const int sb_rd = kScaleBase + kScStage + (wn * (TN * 32) + r32) * 16 + 2 * h;
@@ -195,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 
   int p0 = 0;  // scale buffer that holds group 0 of the current output tile
 
-  // ---- loads.  A wave's batch for K-tile t is its 2*OPS operand loads (n = 0..OPS-1: A, then B) and,
+  // ---- loads.  A wave's batch for K-tile t is its NL operand loads (n = 0..OPA-1: A, then B) and,
   // when t % 4 == 2, the scale load for the four K-tiles starting at t + 2 (at the end of the batch, so
   // that a wait that leaves a whole batch in flight also covers the scales of the batch before).
   // K-tile (or group of four K-tiles) number kk counts on from the current output tile into the next one.
@@ -209,9 +222,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   };
   auto issue_one = [&]<bool INSIDE>(int kk, int slot, int n) __attribute__((always_inline)) {
     const int t = INSIDE || kk < nkt ? kk : kk - nkt;
-    const uint32_t dst = lds0 + slot * kStage + wave * (OPS * 1024);
-    if (n < OPS) dma16(rA, dst + n * 1024, voff_a[n], t * kstep_a);
-    else dma16(rB, dst + kOpStage + (n - OPS) * 1024, voff_b[n - OPS], t * kstep_b);
+    const uint32_t dst = lds0 + slot * kStage;
+    if (n < OPA) dma16(rA, dst + (wave * OPA + n) * 1024, voff_a[n], t * kstep_a);
+    else dma16(rB, dst + kAStage + (wave * OPB + n - OPA) * 1024, voff_b[n - OPA], t * kstep_b);
   };
 
   // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
@@ -302,7 +315,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     // with K-tile kt+3 in its compute cluster; the scales with group nk4
     if (!STEADY && GRP == 0 && kt + 2 == nkt) operand_rsrc(tile_next);
 #pragma unroll
-    for (int n = kLoadsInCompute; n < 2 * OPS; n++) issue_one.template operator()<STEADY>(kt + 2, stage2, n);
+    for (int n = kLoadsInCompute; n < NL; n++) issue_one.template operator()<STEADY>(kt + 2, stage2, n);
     if (KM == 0) {
       if (!STEADY && (kt + 4) >> 2 == nk4) scale_rsrc(tile_next);
       issue_scales.template operator()<STEADY>((kt + 4) >> 2);
@@ -317,7 +330,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
     for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
     // own share of the next K-tile has landed; the batch after it may be in flight
-    if (GRP == 1) wait_vmcnt<2 * OPS + (KM == 0 ? SCL : 0)>();
+    if (GRP == 1) wait_vmcnt<NL + (KM == 0 ? SCL : 0)>();
     barrier();
     __builtin_amdgcn_s_setprio(1);
     mma_tile.template operator()<FIRST>([&](int i) __attribute__((always_inline)) {
@@ -328,7 +341,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
       }
     });
     __builtin_amdgcn_s_setprio(0);
-    if (GRP == 0) wait_vmcnt<2 * OPS + (KM == 0 ? SCL : 0)>();
+    if (GRP == 0) wait_vmcnt<NL + (KM == 0 ? SCL : 0)>();
     barrier();
     stage = stage == kStages - 1 ? 0 : stage + 1;
     stage2 = stage2 == kStages - 1 ? 0 : stage2 + 1;
@@ -451,15 +464,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // that its compute cluster of "step -1" would have issued; tile 0 must have landed everywhere
   issue_scales.template operator()<true>(0);
 #pragma unroll
-  for (int n = 0; n < 2 * OPS; n++) issue_one.template operator()<true>(0, 0, n);
+  for (int n = 0; n < NL; n++) issue_one.template operator()<true>(0, 0, n);
 #pragma unroll
-  for (int n = 0; n < 2 * OPS; n++) issue_one.template operator()<false>(1, 1, n);
+  for (int n = 0; n < NL; n++) issue_one.template operator()<false>(1, 1, n);
   if (wm == 1) {
 #pragma unroll
     for (int n = 0; n < kLoadsInCompute; n++) issue_one.template operator()<false>(2, 2, n);
-    wait_vmcnt<2 * OPS + kLoadsInCompute>();
+    wait_vmcnt<NL + kLoadsInCompute>();
   } else {
-    wait_vmcnt<2 * OPS>();
+    wait_vmcnt<NL>();
   }
   barrier();
   if (wm == 0) {
@@ -473,10 +486,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 }
 
 bool gemm_tiled_supports(const GemmArgs& g) {
-  // any M; N % 8 keeps every pair of bf16 outputs whole and aligned; K in whole K-tiles; 32-bit byte
+  // any M; N % 8 keeps every run of 8 bf16 outputs whole and aligned; K in whole K-tiles; 32-bit byte
   // offsets inside one tile's operand rows and inside one tile's rows of C
-  return g.M > 0 && g.N > 0 && g.K > 0 && g.N % 8 == 0 && g.K % kBK == 0 && (long)kBM * (g.K / 4 * 3) < (1L << 31) &&
-         (long)kBM * g.N * 4 < (1L << 31) && g.M <= 65535 * kBM && ((uintptr_t)g.C % 16) == 0;
+  return g.M > 0 && g.N > 0 && g.K > 0 && g.N % 8 == 0 && g.K % kBK == 0 && (long)256 * (g.K / 4 * 3) < (1L << 31) &&
+         (long)256 * g.N * 4 < (1L << 31) && g.M <= 65535 * 128 && ((uintptr_t)g.C % 16) == 0;
+}
+
+static int cu_count() {
+  static int cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    cus[dev] = n;
+  }
+  return cus[dev];
 }
 
 // Workgroups to launch: one per output tile, or, when the tiles outnumber the compute units (one
@@ -485,24 +510,48 @@ bool gemm_tiled_supports(const GemmArgs& g) {
 // and must have two steps to land: K-tile counts of 4n+1 (and fewer than four K-tiles) keep one
 // workgroup per tile.
 static int grid_size(const GemmArgs& g, int tiles) {
-  static int cus[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return tiles;
-  if (cus[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return tiles;
-    cus[dev] = n & ~7;  // whole multiples of the 8 XCDs keep the tile -> XCD mapping of the walk
-  }
+  const int cus = cu_count() & ~7;  // whole multiples of the 8 XCDs keep the tile -> XCD mapping of the walk
   const int nkt = g.K / kBK;
-  if (g_tiled_walk == 0 || nkt < 4 || nkt % 4 == 1 || cus[dev] < 8) return tiles;
-  return tiles < cus[dev] ? tiles : cus[dev];
+  if (g_tiled_walk == 0 || nkt < 4 || nkt % 4 == 1 || cus < 8) return tiles;
+  return tiles < cus ? tiles : cus;
+}
+
+// Estimated time of this kernel with tiles of `rows` (128 or 256) rows of A, in microseconds: the tiles are
+// dealt to the CUs in rounds, and a K-tile of a round takes longer the fuller the round is (fewer active CUs run
+// at a higher clock and meet less L2 contention).  Constants measured on MI355X with tile-major B: 8192-wide
+// problems of 64 K-tiles took 57.7 / 62.7 / 70.1 / 86.9 us with 64 / 128 / 192 / 256 tiles of 256 rows and
+// 43.5 / 46.5 / 53.9 us with 128 / 192 / 256 tiles of 128 rows; row-major B costs about 28 % more, and no shape
+// runs faster than its bytes stream.
+double tiled_estimate_us(const GemmArgs& g, int rows) {
+  int cus = cu_count();
+  if (cus <= 0) cus = 256;
+  const long tiles = (long)((g.M + rows - 1) / rows) * ((g.N + kBN - 1) / kBN);
+  const long full = tiles / cus;
+  const double f = (double)(tiles % cus) / cus;
+  const double c0 = rows == 128 ? 0.62 : 0.85, c1 = rows == 128 ? 0.22 : 0.50;
+  const double per_ktile = full * (c0 + c1) + (f > 0 ? c0 + c1 * f * f : 0.0);
+  const double layout = 1.0 + (g.layout_b ? 0.0 : 0.28) - (g.layout_a ? 0.05 : 0.0);
+  // few rows of A against a large B is a streaming problem: measured 3.5 / 3.3 TB/s (tile-major B, 128- / 256-row
+  // tiles) and 2.35 / 2.1 TB/s (row-major B)
+  const double bytes = (0.75 + 1.0 / 32) * g.K * ((double)g.M + g.N) + 2.0 * g.M * g.N;
+  const double stream = bytes / (g.layout_b ? (rows == 128 ? 3.5e6 : 3.3e6) : (rows == 128 ? 2.35e6 : 2.1e6));
+  const double compute = 3.0 + (g.K / kBK) * per_ktile * layout;
+  return compute > stream ? compute : stream;
+}
+
+// Tile height: 256 rows of A per tile unless tiles of 128 rows fill the machine better.
+static int tile_rows(const GemmArgs& g) {
+  if (g.tile_rows == 128 || g.tile_rows == 256) return g.tile_rows;
+  return tiled_estimate_us(g, 128) < tiled_estimate_us(g, 256) ? 128 : 256;
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  const int tm = (g.M + kBM - 1) / kBM, tn = (g.N + kBN - 1) / kBN;
+  const int bm = tile_rows(g);
+  const int tm = (g.M + bm - 1) / bm, tn = (g.N + kBN - 1) / kBN;
   const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b};
-  gemm_tiled_kernel<FA, FB, Out><<<grid_size(g, tm * tn), NW * 64, 0, s>>>(ta);
+  if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2><<<grid_size(g, tm * tn), NW * 64, 0, s>>>(ta);
+  else gemm_tiled_kernel<FA, FB, Out, 4><<<grid_size(g, tm * tn), NW * 64, 0, s>>>(ta);
   return hipGetLastError();
 }
 

@@ -12,13 +12,16 @@ struct GemmArgs {
   int fmt_a, fmt_b;  // 2 = e2m3, 3 = e3m2
   bool f32out;
   int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (operand: 32 rows x 128 elements in LDS image order; scales: 32 rows x 16 bytes)
+  int tile_rows = 0;               // tiled kernel: rows of A per output tile, 128 or 256; 0 = chosen per shape
 };
 
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
-bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the 256x256 tiling
+bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
+double tiled_estimate_us(const GemmArgs& g, int rows);  // estimated time of the tiled kernel with 128- or 256-row tiles
+double mid_estimate_us(const GemmArgs& g);
 hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);

@@ -35,7 +35,7 @@ E3M2 = 3
 LAYOUT_ROW = 0
 LAYOUT_TILE = 1
 
-KERNEL_AUTO, KERNEL_GENERIC, KERNEL_TILED, KERNEL_SKINNY, KERNEL_MID = 0, 1, 2, 3, 4
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_TILED, KERNEL_SKINNY, KERNEL_MID, KERNEL_TILED_128, KERNEL_TILED_256 = 0, 1, 2, 3, 4, 5, 6
 
 
 def _as_tensor(obj, name: str):

@@ -304,12 +304,14 @@ def test_automatic_dispatch_agrees_with_generic_kernel_on_ragged_shapes(hk):
 
 # ------------------------------------------------------------------ workgroups that walk through several output tiles
 @pytest.mark.parametrize("M,N,K,la,lb", [(8192, 8192, 512, 0, 0), (8192, 8192, 768, 0, 0), (8192, 8192, 896, 1, 1), (8192, 8192, 640, 0, 0),
-                                         (5000, 5000, 1024, 0, 0), (4352, 4352, 1280, 0, 1), (4128, 8200, 2048, 0, 0), (8192, 16384, 1152, 1, 0)])
+                                         (5000, 5000, 1024, 0, 0), (4352, 4352, 1280, 0, 1), (4128, 8200, 2048, 0, 0), (8192, 16384, 1152, 1, 0),
+                                         (100, 264, 640, 0, 0), (1000, 4104, 1280, 0, 0), (2176, 8192, 896, 1, 1)])
 @pytest.mark.parametrize("out", [torch.float32, torch.bfloat16])
 def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, lb, out):
     """More output tiles than compute units: every workgroup of the tiled kernel takes several tiles in turn, the loads of
     the next tile running under the last K-tiles of the current one (K-tile counts 4n, 4n+2, 4n+3; 4n+1 keeps one workgroup
-    per tile), with ragged edge tiles and tile-major operands.  The result must equal the one-wave-per-tile kernel's in every
+    per tile), with ragged edge tiles and tile-major operands, for both tile heights (128 and 256 rows of A).  The result
+    must equal the one-wave-per-tile kernel's in every
     bit (both round the same fp32 sums once), and nothing may be written outside C (guard rows before and after it)."""
     g = torch.Generator(device="cuda")
     g.manual_seed(M + N + K)
@@ -318,7 +320,7 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
     prev_r = hk.tk_kernel.set_relayout(0)
     res = []
     try:
-        for kern in (1, 2):
+        for kern in (1, hk.tk_kernel.KERNEL_TILED_128, hk.tk_kernel.KERNEL_TILED_256):
             full = torch.full((M + 2, N), 12345.0, dtype=out, device="cuda")
             prev = hk.tk_kernel.set_kernel(kern)
             try:
@@ -329,9 +331,10 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
             res.append(full)
     finally:
         hk.tk_kernel.set_relayout(prev_r)
-    ref, got = res
-    assert bool((got[0] == 12345.0).all()) and bool((got[-1] == 12345.0).all())
-    assert torch.equal(ref[1:-1], got[1:-1])
+    ref = res[0]
+    for got in res[1:]:
+        assert bool((got[0] == 12345.0).all()) and bool((got[-1] == 12345.0).all())
+        assert torch.equal(ref[1:-1], got[1:-1])
 
 
 # ------------------------------------------------------------------ stream capture
