@@ -1,106 +1,124 @@
-// fp32 -> MXFP6 quantise + pack on the GPU, and the zero fill used for K == 0.
-// One lane handles one 32-element block: 128 bytes in (8 x 16-byte loads), 24 bytes + 1 scale byte out.
+// fp32 -> MXFP6 quantise + pack on the GPU, the tile-major re-layout copies, and the zero fill used for K == 0.
 // HBM-bound elementwise work: 4 B/element read, 0.78 B/element written.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace mxfp6 {
 
-// Round a non-negative, already scaled magnitude to the fp6 grid (ties to even, saturating) with
-// integer arithmetic on the fp32 bits.  MB = mantissa bits, BIAS = exponent bias, EB = exponent bits.
-template <int MB, int BIAS, int EB>
-__device__ __forceinline__ uint32_t quantise_mag(float a) {
-  const uint32_t u = __float_as_uint(a);
-  if (a != a) return 31u;
-  const int be = (int)(u >> 23);
-  if (be == 0) return 0u;  // fp32 subnormal: far below half of the smallest fp6 step
-  const int ex = be - 127;
-  constexpr int emin = 1 - BIAS;
-  const int e = ex < emin ? emin : ex;
-  const int shift = 23 - MB + (e - ex);
-  uint32_t q = 0;
-  if (shift < 32) {
-    const uint32_t man = (u & 0x7FFFFFu) | 0x800000u;
-    const uint32_t half = 1u << (shift - 1), frac = man & ((half << 1) - 1);
-    q = man >> shift;
-    q += (frac > half || (frac == half && (q & 1u))) ? 1u : 0u;
-  }
-  uint32_t code;
-  if (ex < emin) {
-    code = q;  // subnormal (q == 2^MB lands on the smallest normal)
-  } else {
-    int ee = e;
-    if (q == (2u << MB)) { q = 1u << MB; ee += 1; }
-    code = ((uint32_t)(ee + BIAS) << MB) | (q - (1u << MB));
-    if (ee + BIAS >= (1 << EB)) code = 31u;
-  }
-  return code > 31u ? 31u : code;
+// Quantiser.  One lane handles one 32-element block (128 bytes in, 24 bytes + 1 scale byte out), but the memory
+// system wants consecutive lanes on consecutive bytes: a wave fetches 64 blocks (8 KB, contiguous) with eight
+// direct-to-LDS loads of 16 bytes per lane into a private buffer and every lane reads its own block back.  The
+// buffer is an image of memory with the eight 16-byte pieces of block b rotated: piece c lives in slot
+// b * 8 + (c ^ (b & 7)), chosen by which global bytes each lane fetches (a direct load writes lane l at 16 l), so
+// that the 16 lanes of a ds_read_b128 phase spread over all banks.  The conversion itself is the hardware's:
+// v_cvt_scalef32_2xpk16_{fp6,bf6}_f32 divides 32 floats by a power of two and rounds them to e2m3 / e3m2 (nearest
+// even, saturating, NaN -> largest magnitude, fp32 subnormals -> 0); its result interleaves its two sources,
+// so they are the even and the odd elements of the block.  (With the rounding done by integer arithmetic, ~25
+// instructions per element, the kernel was ALU-bound at 4.4 TB/s.)
+// Row-major output: a wave's 64 blocks are consecutive (1536 contiguous output bytes).  Tile-major output: they are
+// 16 rows x one K-tile (512 input bytes per row, four whole lines), which is half of a 3 KB output tile and again
+// 1536 contiguous bytes; a block's 24 bytes are three 8-byte stores (an aligned 8-byte run never straddles the
+// 16-byte pieces the tile-major order permutes).
+constexpr int kQWaves = 4, kQChunk = 64 * 128;  // waves per workgroup; bytes a wave fetches at a time (64 blocks)
+
+__device__ __forceinline__ void dma16_q(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_base), "v"(voff), "s"(rsrc) : "memory");
 }
 
 template <int FMT>
-__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ X, uint8_t* __restrict__ packed,
-                                                       uint8_t* __restrict__ scales, long nblocks, int nkb, int layout) {
-  constexpr int MB = FMT == 2 ? 3 : 2, BIAS = FMT == 2 ? 1 : 3, EB = FMT == 2 ? 2 : 3, EMAX = FMT == 2 ? 2 : 4;
-  const long b = (long)blockIdx.x * 256 + threadIdx.x;
-  if (b >= nblocks) return;
-  const v4f* src = reinterpret_cast<const v4f*>(X + b * 32);
-  v4f x[8];
+__global__ __launch_bounds__(kQWaves * 64) void quantize_kernel(const float* __restrict__ X, uint8_t* __restrict__ packed,
+                                                              uint8_t* __restrict__ scales, long nblocks, int nkb, int layout) {
+  constexpr int EMAX = FMT == 2 ? 2 : 4;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[kQWaves * kQChunk];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kQChunk;
+  const long nchunks = (nblocks + 63) / 64;
+  const long stride = (long)gridDim.x * kQWaves;
+  long chunk = (long)blockIdx.x * kQWaves + wave;
+  const int nkt = nkb / 4;  // tile-major only: K-tiles per row
+
+  // slot s = q * 64 + lane of load q holds piece (s % 8) ^ (b & 7) of the chunk's block b = s / 8; tile-major:
+  // block b is K-block b % 4 of row b / 4 of the chunk
+  int voff[8];
 #pragma unroll
-  for (int i = 0; i < 8; i++) x[i] = src[i];
-  float amax = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) amax = fmaxf(amax, fabsf(x[i][j]));
-  int sb = 0;
-  if (amax > 0.f) {
-    const uint32_t u = __float_as_uint(amax);
-    const int be = (int)(u >> 23);
-    const int fl = be ? be - 127 : (31 - __clz((int)u)) - 149;  // floor(log2(amax)), fp32 subnormals included
-    sb = fl - EMAX + 127;
-    sb = sb < 0 ? 0 : (sb > 254 ? 254 : sb);
+  for (int q = 0; q < 8; q++) {
+    const int sl = q * 64 + lane, b = sl >> 3, c = (sl & 7) ^ (b & 7);
+    voff[q] = layout ? (b >> 2) * (nkb * 128) + (b & 3) * 128 + c * 16 : (b * 8 + c) * 16;
   }
-  // multiply by 2^(127 - sb) exactly: split the power of two so that each factor is a normal fp32
-  const int ex = 127 - sb;  // in [-127, 127]
-  const float f1 = __uint_as_float((uint32_t)((ex / 2) + 127) << 23);
-  const float f2 = __uint_as_float((uint32_t)((ex - ex / 2) + 127) << 23);
-  uint32_t w[6] = {0, 0, 0, 0, 0, 0};
+  auto fetch = [&](long ch) __attribute__((always_inline)) {
+    // the resource covers this chunk only (the whole input may exceed 4 GB); bytes past the end read as zero
+    if (layout) {
+      const long g16 = ch / nkt, kt = ch - g16 * nkt;
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + (g16 * 16 * nkb + kt * 4) * 128, (uint32_t)(15 * nkb * 128 + 512));
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    uint32_t g = 0;
+      for (int q = 0; q < 8; q++) dma16_q(r, buf + q * 1024, voff[q]);
+    } else {
+      const long left = nblocks * 128 - ch * kQChunk;
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + ch * kQChunk, (uint32_t)(left < kQChunk ? left : kQChunk));
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const float v = x[i][j];
-      const float y = fabsf(v) * f1 * f2;
-      const uint32_t code = quantise_mag<MB, BIAS, EB>(y) | ((__float_as_uint(v) >> 31) << 5);
-      g |= code << (6 * j);
+      for (int q = 0; q < 8; q++) dma16_q(r, buf + q * 1024, voff[q]);
     }
-    // group i is 24 bits at bit 24*i of the 192-bit block
-    const int bit = 24 * i, d = bit >> 5, sh = bit & 31;
-    w[d] |= g << sh;
-    if (sh > 8) w[d + 1] |= g >> (32 - sh);
-  }
-  if (layout == 0) {
-    uint32_t* dst = reinterpret_cast<uint32_t*>(packed + b * 24);
+  };
+  if (chunk < nchunks) fetch(chunk);
+  for (; chunk < nchunks; chunk += stride) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    v4f x[8];
 #pragma unroll
-    for (int i = 0; i < 6; i++) dst[i] = w[i];
-  } else {
-    const int row = (int)(b / nkb), kb = (int)(b - (long)row * nkb);
+    for (int c = 0; c < 8; c++) x[c] = *reinterpret_cast<const v4f*>(smem + wave * kQChunk + lane * 128 + ((c ^ (lane & 7)) * 16));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (chunk + stride < nchunks) fetch(chunk + stride);  // the buffer is free again: the next chunk streams in under the arithmetic
+
+    float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 6; i++) *reinterpret_cast<uint32_t*>(packed + tile_major_offset(row, kb * 24 + 4 * i, nkb / 4)) = w[i];
-    scales[tile_major_scale_offset(row, kb, (nkb + 15) / 16)] = (uint8_t)sb;
-    return;
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) amax = fmaxf(amax, fabsf(x[i][j]));
+    int sb = 0;
+    if (amax > 0.f) {
+      const uint32_t u = __float_as_uint(amax);
+      const int be = (int)(u >> 23);
+      const int fl = be ? be - 127 : (31 - __clz((int)u)) - 149;  // floor(log2(amax)), fp32 subnormals included
+      sb = fl - EMAX + 127;
+      sb = sb < 0 ? 0 : (sb > 254 ? 254 : sb);
+    }
+    v16f ev, od;
+#pragma unroll
+    for (int i = 0; i < 16; i++) ev[i] = x[i / 2][(2 * i) & 3], od[i] = x[i / 2][(2 * i + 1) & 3];
+    const float scale = __uint_as_float((uint32_t)sb << 23);  // 2^(sb - 127); the instruction uses the exponent field
+    typedef unsigned v6u __attribute__((ext_vector_type(6)));
+    v6u w;
+    if constexpr (FMT == 2) w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, scale);
+    else w = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(ev, od, scale);
+    if (layout == 0) {
+      const long b = chunk * 64 + lane;
+      if (b >= nblocks) continue;
+      u32x2* dst = reinterpret_cast<u32x2*>(packed + b * 24);
+#pragma unroll
+      for (int i = 0; i < 3; i++) dst[i] = u32x2{w[2 * i], w[2 * i + 1]};
+      scales[b] = (uint8_t)sb;
+    } else {
+      const long g16 = chunk / nkt;
+      const int kt = (int)(chunk - g16 * nkt);
+      const int row = (int)(g16 * 16) + (lane >> 2), kb = kt * 4 + (lane & 3);
+#pragma unroll
+      for (int i = 0; i < 3; i++)
+        *reinterpret_cast<u32x2*>(packed + tile_major_offset(row, kb * 24 + 8 * i, nkt)) = u32x2{w[2 * i], w[2 * i + 1]};
+      scales[tile_major_scale_offset(row, kb, (nkb + 15) / 16)] = (uint8_t)sb;
+    }
   }
-  scales[b] = (uint8_t)sb;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s) {
   const long nblocks = (long)rows * (K / 32);
-  const unsigned grid = (unsigned)((nblocks + 255) / 256);
+  if (nblocks == 0) return hipSuccess;
+  const long nchunks = (nblocks + 63) / 64, want = (nchunks + kQWaves - 1) / kQWaves;
+  const unsigned grid = (unsigned)(want < 256 * 5 ? want : 256 * 5);  // five workgroups of 32 KB LDS fit a CU
   if (fmt == 2)
-    quantize_kernel<2><<<grid, 256, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
+    quantize_kernel<2><<<grid, kQWaves * 64, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
   else
-    quantize_kernel<3><<<grid, 256, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
+    quantize_kernel<3><<<grid, kQWaves * 64, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
   return hipGetLastError();
 }
 
