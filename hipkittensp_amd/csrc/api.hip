@@ -80,7 +80,7 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
 }
 
 int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
-                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream) {
+                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream, const mxfp6::Epilogue& ep = mxfp6::Epilogue()) {
   if (M < 0 || N < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
   if ((fmt_a != MXFP6_FMT_E2M3 && fmt_a != MXFP6_FMT_E3M2) || (fmt_b != MXFP6_FMT_E2M3 && fmt_b != MXFP6_FMT_E3M2))
     return MXFP6_EINVAL_FMT;
@@ -92,6 +92,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   if (!C) return MXFP6_EINVAL_PTR;
   if (K > 0 && (!A || !B || !As || !Bs)) return MXFP6_EINVAL_PTR;
   if (((uintptr_t)A & 3) || ((uintptr_t)B & 3) || ((uintptr_t)C & (f32out ? 3 : 1))) return MXFP6_EINVAL_ALIGN;
+  // the tiled kernel reads four floats (or four bf16) of the per-column vectors at a time
+  if (((uintptr_t)ep.col_scale & 15) || ((uintptr_t)ep.row_scale & 3) || ((uintptr_t)ep.bias & (ep.bias_bf16 ? 7 : 15))) return MXFP6_EINVAL_ALIGN;
+  if (ep.act < 0 || ep.act > 3) return MXFP6_EINVAL_EPILOGUE;
   if ((long)M * N >= (1L << 40) || (long)K / 4 * 3 * 256 >= (1L << 31)) return MXFP6_EINVAL_SHAPE;
   int rc = check_device();
   if (rc) return rc;
@@ -101,6 +104,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     return e == hipSuccess ? MXFP6_OK : (int)e;
   }
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out, layout_a, layout_b};
+  g.ep = ep;
   const int force = g_force.load(std::memory_order_relaxed);
   hipError_t e;
   if (force == 1) {
@@ -145,6 +149,14 @@ int mxfp6_gemm_f32out(const void* A, const void* B, const void* As, const void* 
 int mxfp6_gemm_ex(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
                   int fmt_b, int layout_a, int layout_b, int out_f32, void* stream) {
   return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, out_f32 != 0, layout_a, layout_b, stream);
+}
+
+int mxfp6_gemm_fused(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
+                     int fmt_b, int layout_a, int layout_b, int out_f32, const void* bias, int bias_bf16, const float* row_scale,
+                     const float* col_scale, int activation, void* stream) {
+  mxfp6::Epilogue ep;
+  ep.bias = bias, ep.bias_bf16 = bias_bf16 != 0, ep.row_scale = row_scale, ep.col_scale = col_scale, ep.act = activation;
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, out_f32 != 0, layout_a, layout_b, stream, ep);
 }
 
 int mxfp6_tile_operand(const void* src, void* dst, int rows, int K, int tile, void* stream) {
@@ -203,13 +215,14 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_EINVAL_ALIGN: return "mxfp6: pointer alignment (packed operands 4 bytes, fp32 input 16 bytes)";
     case MXFP6_ENODEVICE: return "mxfp6: the current device is not gfx950 (MI355X)";
     case MXFP6_EINVAL_LAYOUT: return "mxfp6: layout must be 0 (row-major) or 1 (tile-major)";
+    case MXFP6_EINVAL_EPILOGUE: return "mxfp6: activation must be 0 (none), 1 (relu), 2 (gelu) or 3 (silu)";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 104; }
+int mxfp6_abi_version(void) { return 105; }
 
 #pragma GCC visibility pop
 }  // extern "C"

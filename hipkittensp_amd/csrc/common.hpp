@@ -42,6 +42,44 @@ __device__ __forceinline__ void store4(float* p, float a, float b, float c, floa
 __device__ __forceinline__ void store1(uint16_t* p, float a) { *p = (uint16_t)(pack_bf16x2(a, 0.f) & 0xffffu); }
 __device__ __forceinline__ void store1(float* p, float a) { *p = a; }
 
+// Optional work fused into every kernel's epilogue, in fp32 before the output rounding:
+//   y = act(acc * row_scale[m] * col_scale[n] + bias[n])        (each factor / term only if its pointer is set)
+// act: 0 none, 1 relu, 2 gelu (erf form), 3 silu.  bias is float or bf16 (bias_bf16).
+struct Epilogue {
+  const void* bias = nullptr;
+  const float* row_scale = nullptr;
+  const float* col_scale = nullptr;
+  int bias_bf16 = 0;
+  int act = 0;
+};
+__host__ __device__ __forceinline__ bool epilogue_any(const Epilogue& e) { return e.bias || e.row_scale || e.col_scale || e.act; }
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+// The activations in a handful of instructions each (they are unrolled over every accumulator of a tile):
+// silu with the hardware exp2 / reciprocal (~1e-6 relative); gelu's erf by Abramowitz & Stegun 7.1.26
+// (|error| <= 1.5e-7 absolute).
+__device__ __forceinline__ float act_relu(float y) { return y > 0.f ? y : 0.f; }
+__device__ __forceinline__ float act_silu(float y) { return y * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * y)); }
+__device__ __forceinline__ float act_gelu(float y) {
+  const float z = fabsf(y) * 0.70710678118654752440f;
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.f));
+  const float poly = t * fmaf(t, fmaf(t, fmaf(t, fmaf(t, 1.061405429f, -1.453152027f), 1.421413741f), -0.284496736f), 0.254829592f);
+  const float erf_abs = 1.f - poly * __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
+  return 0.5f * y * (1.f + copysignf(erf_abs, y));
+}
+__device__ __forceinline__ float epilogue_act(float y, int act) {
+  if (act == 1) return act_relu(y);
+  if (act == 2) return act_gelu(y);
+  if (act == 3) return act_silu(y);
+  return y;
+}
+// one element; m < M and n < N are the caller's business
+__device__ __forceinline__ float epilogue_apply(const Epilogue& e, float v, long m, long n) {
+  if (e.row_scale) v *= e.row_scale[m];
+  if (e.col_scale) v *= e.col_scale[n];
+  if (e.bias) v += e.bias_bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(e.bias)[n]) : reinterpret_cast<const float*>(e.bias)[n];
+  return epilogue_act(v, e.act);
+}
+
 // Raw buffer resource over [base, base + bytes): out-of-range lanes of a buffer load read 0.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);

@@ -12,7 +12,7 @@ template <int FA, int FB, typename Out>
 __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                           const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                           typename Out::type* __restrict__ C, int M, int N, int K, int layout_a,
-                                                          int layout_b) {
+                                                          int layout_b, const Epilogue ep) {
   const int lane = threadIdx.x, h = lane >> 5, r = lane & 31;
   const long m = (long)blockIdx.y * 32 + r, n = (long)blockIdx.x * 32 + r;
   const int nkb = K / 32;
@@ -45,17 +45,18 @@ __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restr
   if (!mv) return;
   typename Out::type* crow = C + m * (long)N;
   const long n0 = (long)blockIdx.x * 32 + 4 * h;
+  const bool has_ep = epilogue_any(ep);
   for (int g = 0; g < 4; g++)
     for (int e = 0; e < 4; e++) {
       long nn = n0 + 8 * g + e;
-      if (nn < N) store1(crow + nn, acc[4 * g + e]);
+      if (nn < N) store1(crow + nn, has_ep ? epilogue_apply(ep, acc[4 * g + e], m, nn) : acc[4 * g + e]);
     }
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   dim3 grid((g.N + 31) / 32, (g.M + 31) / 32);
-  gemm_generic_kernel<FA, FB, Out><<<grid, 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_a, g.layout_b);
+  gemm_generic_kernel<FA, FB, Out><<<grid, 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_a, g.layout_b, g.ep);
   return hipGetLastError();
 }
 

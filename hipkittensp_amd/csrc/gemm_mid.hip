@@ -58,7 +58,7 @@ template <int FA, int FB, typename Out, int BM, int BN>
 __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                        const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                        typename Out::type* __restrict__ C, int M, int N, int K, int mblocks,
-                                                       int layout_b) {
+                                                       int layout_b, const Epilogue ep) {
   static_assert((BM == 64 || BM == 128) && (BN == 32 || BN == 64), "tile");
   constexpr int GA = 2;                       // K-tiles per A slot
   constexpr int GB = 256 / BN;                // K-tiles per B slot: 8 or 4
@@ -251,6 +251,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
 #pragma unroll
   for (int e = 0; e < 16; e++) partial[(wave * 16 + e) * 64 + lane] = acc[e];
   __syncthreads();
+  const bool has_ep = epilogue_any(ep);
   for (int idx = tid; idx < TILES * 1024; idx += 512) {
     const int t = idx >> 10, e = (idx >> 6) & 15, l = idx & 63;
     float s = 0.f;
@@ -258,7 +259,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
     for (int p = 0; p < KP; p++) s += partial[((p * TILES + t) * 16 + e) * 64 + l];
     const int m = m0 + (t % TMW) * 32 + (l & 31);
     const long nn = (long)n0 + (t / TMW) * 32 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
-    if (m < M && nn < N) store1(C + (long)m * N + nn, s);
+    if (m < M && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, s, m, nn) : s);
   }
 }
 
@@ -303,7 +304,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int nblocks = wide ? (g.N + 63) / 64 : (g.N + 31) / 32;
   const int mblocks = g.M <= 64 ? 1 : (g.M + 127) / 128;
 #define MXFP6_MID_LAUNCH(BM, BN) \
-  gemm_mid_kernel<FA, FB, Out, BM, BN><<<nblocks * mblocks, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, mblocks, g.layout_b)
+  gemm_mid_kernel<FA, FB, Out, BM, BN><<<nblocks * mblocks, 512, 0, s>>>(g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, mblocks, g.layout_b, g.ep)
   if (g.M <= 64) {
     if (wide) MXFP6_MID_LAUNCH(64, 64); else MXFP6_MID_LAUNCH(64, 32);
   } else {

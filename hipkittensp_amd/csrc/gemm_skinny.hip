@@ -46,7 +46,8 @@ __device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt
 template <int FA, int FB, typename Out, int AR, int NW>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
-                                                              typename Out::type* __restrict__ C, int M, int N, int K, int layout_b) {
+                                                              typename Out::type* __restrict__ C, int M, int N, int K, int layout_b,
+                                                              const Epilogue ep) {
   constexpr int kBBuf = 32 * 384, kABuf = AR * 384, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then 2 x 1 KB of scales
   constexpr int kBuf = kScOff + 2048;
   constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024;                    // direct loads per chunk: 12 and 6 or 12
@@ -159,6 +160,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 #pragma unroll
   for (int e = 0; e < 16; e++) part[(wave * 16 + e) * 64 + lane] = acc[e];
   __syncthreads();
+  const bool has_ep = epilogue_any(ep);
   for (int idx = tid; idx < 1024; idx += NW * 64) {
     const int e = idx >> 6, l = idx & 63;
     float s = 0.f;
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     for (int w = 0; w < NW; w++) s += part[(w * 16 + e) * 64 + l];
     const int m = l & 31;
     const long nn = (long)n0 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
-    if (m < M && nn < N) store1(C + (long)m * N + nn, s);
+    if (m < M && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, s, m, nn) : s);
   }
 }
 
@@ -179,9 +181,9 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const unsigned grid = (g.N + 31) / 32;
   if (g.M <= 16)
-    gemm_skinny_kernel<FA, FB, Out, 16, 8><<<grid, 8 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b);
+    gemm_skinny_kernel<FA, FB, Out, 16, 8><<<grid, 8 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b, g.ep);
   else
-    gemm_skinny_kernel<FA, FB, Out, 32, 6><<<grid, 6 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b);
+    gemm_skinny_kernel<FA, FB, Out, 32, 6><<<grid, 6 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b, g.ep);
   return hipGetLastError();
 }
 

@@ -102,9 +102,13 @@ struct TiledArgs {
   const uint8_t *A, *B, *As, *Bs;
   void* C;
   int M, N, K, tiles_m, tiles_n, layout_a, layout_b;
+  Epilogue ep;
 };
 
-template <int FA, int FB, typename Out, int TM>
+// FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
+// around updates of all accumulators make the compiler copy them at every output tile, taken or not (3-4 % of an
+// unfused 8192^3 GEMM).
+template <int FA, int FB, typename Out, int TM, bool FUSED>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
   typedef Shape<TM> S;
   constexpr int kBM = S::BM, OPA = S::OPA, NL = S::NL, kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase;
@@ -386,6 +390,60 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // the K loop ("all but the newest batch") stay valid.
   // EDGE: the tile has fewer than 256 valid rows or columns; those stores are predicated per lane.
   typedef typename Out::type OutT;
+  // Fused scales / bias / activation, on the accumulators themselves, before the epilogue proper.  Per 32x32 tile a
+  // lane owns row wm * TM * 32 + 32 i + lane % 32 and columns 8 q + 4 h .. + 3 for q = 0..3; N % 8 == 0, so a run of
+  // four is inside or outside N as a whole.  The loads here are the compiler's: its waits also wait for the direct
+  // loads in flight, which costs a fused call a fraction of a K-tile per output tile and an unfused one nothing.
+  auto fuse = [&]() __attribute__((always_inline)) {
+    const auto g = fresh_args();
+    const void* bias = g->ep.bias;
+    const float *row_scale = g->ep.row_scale, *col_scale = g->ep.col_scale;
+    const int act = g->ep.act, bias_bf16 = g->ep.bias_bf16;
+    const bool affine = bias || row_scale || col_scale;
+    const int M = g->M, N = g->N;
+    const long m0 = (long)(tile_cur & 0xffff) * kBM + wm * (TM * 32) + r32, n0 = (long)(tile_cur >> 16) * kBN + wn * (TN * 32) + 4 * h;
+    // one 32x32 tile at a time, each with its own branches: a branch around all 128 accumulators at once makes the
+    // compiler keep a second copy of them
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        if (affine) {
+          const float rs = row_scale && m0 + i * 32 < M ? row_scale[m0 + i * 32] : 1.f;
+          v4f cs[4], bi[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const long n = n0 + j * 32 + q * 8;
+            cs[q] = v4f{1.f, 1.f, 1.f, 1.f}, bi[q] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (n < N) {
+              if (col_scale) cs[q] = *reinterpret_cast<const v4f*>(col_scale + n);
+              if (bias && bias_bf16) {
+                const u32x2 b2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(bias) + n);
+                bi[q] = v4f{__uint_as_float(b2[0] << 16), __uint_as_float(b2[0] & 0xffff0000u), __uint_as_float(b2[1] << 16),
+                            __uint_as_float(b2[1] & 0xffff0000u)};
+              } else if (bias) {
+                bi[q] = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(bias) + n);
+              }
+            }
+          }
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[i][j][4 * q + e] = fmaf(acc[i][j][4 * q + e] * rs, cs[q][e], bi[q][e]);
+        }
+        if (act == 1) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) acc[i][j][e] = act_relu(acc[i][j][e]);
+        } else if (act == 2) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) acc[i][j][e] = act_gelu(acc[i][j][e]);
+        } else if (act == 3) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) acc[i][j][e] = act_silu(acc[i][j][e]);
+        }
+        asm volatile("" : "+v"(acc[i][j]));
+      }
+  };
   auto epilogue = [&]<bool EDGE>(int rows_a, int rows_b) __attribute__((always_inline)) {
     const auto g = fresh_args();
     const int N = g->N, N2 = N * (int)sizeof(OutT);  // N2: bytes per row of C
@@ -446,6 +504,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   auto run = [&]<int GRP>() __attribute__((always_inline)) {
     for (;;) {
       k_loop.template operator()<GRP>();
+      if constexpr (FUSED) fuse();
       {
         const auto g = fresh_args();
         const int rows_a = min(kBM, g->M - (tile_cur & 0xffff) * kBM), rows_b = min(kBN, g->N - (tile_cur >> 16) * kBN);
@@ -549,9 +608,15 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int bm = tile_rows(g);
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + kBN - 1) / kBN;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b};
-  if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2><<<grid_size(g, tm * tn), NW * 64, 0, s>>>(ta);
-  else gemm_tiled_kernel<FA, FB, Out, 4><<<grid_size(g, tm * tn), NW * 64, 0, s>>>(ta);
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep};
+  const int grid = grid_size(g, tm * tn);
+  if (epilogue_any(g.ep)) {
+    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, true><<<grid, NW * 64, 0, s>>>(ta);
+    else gemm_tiled_kernel<FA, FB, Out, 4, true><<<grid, NW * 64, 0, s>>>(ta);
+  } else {
+    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, false><<<grid, NW * 64, 0, s>>>(ta);
+    else gemm_tiled_kernel<FA, FB, Out, 4, false><<<grid, NW * 64, 0, s>>>(ta);
+  }
   return hipGetLastError();
 }
 

@@ -1,5 +1,6 @@
 // Internal launcher interface between the C ABI (api.hip) and the kernel translation units.
 #pragma once
+#include "common.hpp"
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -13,6 +14,7 @@ struct GemmArgs {
   bool f32out;
   int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (operand: 32 rows x 128 elements in LDS image order; scales: 32 rows x 16 bytes)
   int tile_rows = 0;               // tiled kernel: rows of A per output tile, 128 or 256; 0 = chosen per shape
+  Epilogue ep;                     // fused bias / scales / activation (all optional)
 };
 
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);

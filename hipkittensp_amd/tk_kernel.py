@@ -73,8 +73,15 @@ def scale_width(K: int, layout: int = LAYOUT_ROW) -> int:
     return K // 32 if layout == LAYOUT_ROW else (K + 511) // 512 * 16
 
 
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU = 0, 1, 2, 3
+_ACTS = {None: 0, "none": 0, "relu": 1, "gelu": 2, "silu": 3, 0: 0, 1: 1, 2: 2, 3: 3}
+
+
 def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, layout_a: int = LAYOUT_ROW,
-                   layout_b: int = LAYOUT_ROW) -> None:
+                   layout_b: int = LAYOUT_ROW, bias=None, row_scale=None, col_scale=None, activation=None) -> None:
+    """C = dq(A) @ dq(B).T; optionally fused, in fp32 before the output rounding:
+    C = act(acc * row_scale[:, None] * col_scale[None, :] + bias[None, :]) with bias [N] float32 or bfloat16,
+    row_scale [M] and col_scale [N] float32, activation one of None / "relu" / "gelu" / "silu"."""
     import torch
 
     A, B = _as_tensor(A, "A"), _as_tensor(B, "B")
@@ -105,13 +112,29 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
             raise RuntimeError(f"{name}: expected shape [{want[0]}, {want[1]}], got {tuple(t.shape)}")
     if _rows_cols(C, "C") != (M, N):
         raise RuntimeError(f"C: expected shape [{M}, {N}], got {tuple(C.shape)}")
-    devs = {t.device for t in (A, B, A_scale, B_scale, C)}
+    if activation not in _ACTS:
+        raise RuntimeError(f"activation must be None, 'relu', 'gelu' or 'silu', got {activation!r}")
+    extras = []
+    for t, name, n, dts in ((bias, "bias", N, (torch.float32, torch.bfloat16)), (row_scale, "row_scale", M, (torch.float32,)),
+                            (col_scale, "col_scale", N, (torch.float32,))):
+        if t is None:
+            continue
+        t = _as_tensor(t, name)
+        if t.dtype not in dts:
+            raise RuntimeError(f"{name}: expected dtype {' or '.join(str(d) for d in dts)}, got {t.dtype}")
+        if t.dim() != 1 or t.shape[0] != n or not t.is_contiguous():
+            raise RuntimeError(f"{name}: expected a contiguous vector of {n} elements, got shape {tuple(t.shape)}")
+        extras.append(t)
+    devs = {t.device for t in (A, B, A_scale, B_scale, C, *extras)}
     if len(devs) != 1:
         raise RuntimeError(f"all tensors must be on one device, got {sorted(map(str, devs))}")
     L = _lib.lib()
+    ptr = lambda t: 0 if t is None else t.data_ptr()
     with torch.cuda.device(C.device):
-        rc = L.mxfp6_gemm_ex(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
-                             fmt_a, fmt_b, layout_a, layout_b, int(C.dtype == torch.float32), _stream())
+        rc = L.mxfp6_gemm_fused(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
+                                fmt_a, fmt_b, layout_a, layout_b, int(C.dtype == torch.float32), ptr(bias),
+                                int(bias is not None and bias.dtype == torch.bfloat16), ptr(row_scale), ptr(col_scale),
+                                _ACTS[activation], _stream())
     _lib.check(rc, "dispatch_micro")
 
 

@@ -39,6 +39,13 @@ extern "C" {
 #define MXFP6_EINVAL_ALIGN (-4) /* a pointer violates the stated alignment                     */
 #define MXFP6_ENODEVICE (-5)    /* current device is not gfx950                                */
 #define MXFP6_EINVAL_LAYOUT (-6) /* layout code is not MXFP6_LAYOUT_ROW / MXFP6_LAYOUT_TILE    */
+#define MXFP6_EINVAL_EPILOGUE (-7) /* activation code is not one of MXFP6_ACT_*                */
+
+/* Activations of mxfp6_gemm_fused. */
+#define MXFP6_ACT_NONE 0
+#define MXFP6_ACT_RELU 1
+#define MXFP6_ACT_GELU 2 /* 0.5 y (1 + erf(y / sqrt 2)) */
+#define MXFP6_ACT_SILU 3 /* y / (1 + exp(-y))           */
 
 /*
  * The operator.  Replaces the reference's dispatch_micro(A, B, C) launcher
@@ -135,6 +142,23 @@ int mxfp6_gemm_ex(const void *A_packed, const void *B_packed, const void *A_scal
  * ceil(K/512) * 16 bytes, of which the padding bytes are not written). */
 int mxfp6_quantize_ex(const float *X, void *packed, void *scales, int rows, int K, int fmt, int layout,
                       void *hip_stream);
+
+/*
+ * mxfp6_gemm_ex with work fused into the epilogue, in fp32 on the accumulators before the output rounding:
+ *   C[m][n] = act(acc[m][n] * row_scale[m] * col_scale[n] + bias[n])
+ * Every vector is optional (NULL = leave out): bias [N] float (bias_bf16 == 0) or bf16 (!= 0), row_scale [M]
+ * float (e.g. a per-token activation scale), col_scale [N] float (e.g. a per-channel weight scale); activation
+ * is one of MXFP6_ACT_*.  With everything left out it is mxfp6_gemm_ex.  Alignment: bias and col_scale 16
+ * bytes (bf16 bias 8), row_scale 4.  gelu and silu are computed with the hardware exp2 / reciprocal and a
+ * five-term erf (absolute error <= 1.5e-7): results agree with a double-precision evaluation to about 1e-6 of
+ * the output range, not bit for bit.
+ * No counterpart in the reference, whose GEMMs store the accumulator tile as it is
+ * (analysis/bf16_gemm/mi325x/kernel_8192.cpp:223-224); it removes a pass over C for the usual linear-layer tail.
+ */
+int mxfp6_gemm_fused(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, void *C,
+                     int M, int N, int K, int fmt_a, int fmt_b, int layout_a, int layout_b, int out_f32,
+                     const void *bias, int bias_bf16, const float *row_scale, const float *col_scale, int activation,
+                     void *hip_stream);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

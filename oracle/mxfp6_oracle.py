@@ -208,6 +208,33 @@ def gemm_ref(a_packed, b_packed, a_scale, b_scale, fmt_a=E2M3, fmt_b=E2M3, acc=n
     return A @ B.T
 
 
+def epilogue_ref(acc, bias=None, row_scale=None, col_scale=None, activation=None) -> np.ndarray:
+    """The fused epilogue in float64: act(acc * row_scale[:, None] * col_scale[None, :] + bias[None, :]).
+    relu = max(y, 0); gelu = 0.5 y (1 + erf(y / sqrt 2)); silu = y / (1 + exp(-y)) -- the textbook forms
+    (torch.nn.functional.relu / gelu(approximate="none") / silu).  The reference has no fused epilogue for this
+    path (its kernels store the accumulator tile as it is, analysis/bf16_gemm/mi325x/kernel_8192.cpp:223-224), so
+    these definitions are pinned by closed forms only: tests/test_oracle.py checks them at points with known values
+    and against their defining identities."""
+    from scipy.special import erf
+
+    y = np.asarray(acc, dtype=np.float64).copy()
+    if row_scale is not None:
+        y *= np.asarray(row_scale, dtype=np.float64)[:, None]
+    if col_scale is not None:
+        y *= np.asarray(col_scale, dtype=np.float64)[None, :]
+    if bias is not None:
+        y += np.asarray(bias, dtype=np.float64)[None, :]
+    if activation in (None, "none"):
+        return y
+    if activation == "relu":
+        return np.maximum(y, 0.0)
+    if activation == "gelu":
+        return 0.5 * y * (1.0 + erf(y / np.sqrt(2.0)))
+    if activation == "silu":
+        return y / (1.0 + np.exp(-y))
+    raise ValueError(f"unknown activation {activation!r}")
+
+
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     """fp32 -> bf16 bit pattern (uint16), round-to-nearest-even; NaN stays NaN."""
     u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)

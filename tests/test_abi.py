@@ -30,7 +30,7 @@ def built_lib():
 
 def test_header_declares_the_operator():
     names = _declared_functions()
-    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_tile_operand", "mxfp6_tile_scales",
+    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_gemm_fused", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_tile_operand", "mxfp6_tile_scales",
                  "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout"):
         assert want in names
 
@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 104
+    assert L.mxfp6_abi_version() == 105
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -81,6 +81,13 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     assert L.mxfp6_gemm_ex(one, one, one, one, one, 32, 32, 128, 2, 2, 2, 0, 0, None) == -6      # unknown layout
     assert L.mxfp6_gemm_ex(one, one, one, one, one, 48, 32, 128, 2, 2, 1, 0, 0, None) == -2      # tile-major rows % 32
     assert L.mxfp6_gemm_ex(one, one, one, one, one, 32, 32, 96, 2, 2, 0, 1, 0, None) == -2       # tile-major K % 128
+    L.mxfp6_gemm_fused.restype = ci
+    L.mxfp6_gemm_fused.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, ci, vp, vp, ci, vp]
+    assert L.mxfp6_gemm_fused(one, one, one, one, one, 32, 32, 128, 2, 2, 0, 0, 0, None, 0, None, None, 4, None) == -7   # unknown activation
+    assert L.mxfp6_gemm_fused(one, one, one, one, one, 32, 32, 128, 2, 2, 0, 0, 0, ctypes.c_void_p(264), 0, None, None, 0, None) == -4  # float bias 16 B
+    assert L.mxfp6_gemm_fused(one, one, one, one, one, 32, 32, 128, 2, 2, 0, 0, 0, None, 0, None, ctypes.c_void_p(260), 0, None) == -4  # col_scale 16 B
+    assert L.mxfp6_gemm_fused(one, one, one, one, one, 32, 32, 96, 2, 2, 0, 1, 0, None, 0, None, None, 0, None) == -2    # the checks of gemm_ex
+    assert L.mxfp6_gemm_fused(one, one, one, one, one, 0, 32, 128, 2, 2, 0, 0, 0, None, 0, None, None, 1, None) == 0
     L.mxfp6_tile_operand.restype = ci
     L.mxfp6_tile_operand.argtypes = [vp, vp, ci, ci, ci, vp]
     assert L.mxfp6_tile_operand(one, one, 33, 128, 1, None) == -2

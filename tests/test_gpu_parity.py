@@ -337,6 +337,69 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
         assert torch.equal(ref[1:-1], got[1:-1])
 
 
+# ------------------------------------------------------------------ fused epilogue
+@pytest.mark.parametrize("kernel,M,N,K", [(1, 70, 40, 96), (3, 16, 96, 1024), (3, 32, 100, 512), (4, 64, 72, 1024), (4, 200, 136, 2048),
+                                          (5, 300, 264, 640), (6, 300, 264, 640), (5, 1024, 4104, 512), (6, 2304, 8200, 512)])
+@pytest.mark.parametrize("activation", [None, "relu", "gelu", "silu"])
+def test_fused_epilogue_every_kernel(hk, kernel, M, N, K, activation):
+    """act(acc * row_scale * col_scale + bias) fused into each kernel's epilogue (the last two shapes have more tiles than
+    CUs: the tiled kernel walks).  The accumulators are the same kernel's unfused fp32 output (bit-exact by the other tests),
+    so this isolates the epilogue: fp32 arithmetic against the float64 closed forms.  relu and the affine part are exact to
+    fp32 rounding of the terms (2e-5 of max(|ref|, 1 % rms) where scale * acc and bias cancel); silu uses the hardware exp2 / reciprocal and gelu a five-term erf with absolute error 1.5e-7,
+    held to 1e-4 of max(|ref|, 1 % rms) (the parity metric).  The bf16 output must be the RNE rounding of the fp32 output."""
+    rng = np.random.default_rng(M + N + K + kernel)
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=M + kernel)
+    dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
+    bias = rng.standard_normal(N).astype(np.float32) * 3
+    rs = (0.5 + rng.random(M)).astype(np.float32)
+    cs = (0.25 + rng.random(N)).astype(np.float32) * 0.2
+    prev = hk.tk_kernel.set_kernel(kernel)
+    prev_r = hk.tk_kernel.set_relayout(0)
+    try:
+        acc = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        hk.dispatch_micro(dA, dB, dAs, dBs, acc)
+        for use in ((True, True, True), (True, False, False), (False, True, False), (False, False, True), (False, False, False)):
+            if not any(use) and activation is None:
+                continue
+            kw = dict(bias=dev(bias) if use[0] else None, row_scale=dev(rs) if use[1] else None, col_scale=dev(cs) if use[2] else None,
+                      activation=activation)
+            C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(dA, dB, dAs, dBs, C, **kw)
+            ref = o.epilogue_ref(acc.cpu().numpy(), bias if use[0] else None, rs if use[1] else None, cs if use[2] else None, activation)
+            got = C.cpu().numpy()
+            assert np.isfinite(got).all()
+            assert o.rel_err(got, ref) <= (1e-4 if activation in ("gelu", "silu") else 2e-5), (use, o.rel_err(got, ref))
+            Cb = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+            hk.dispatch_micro(dA, dB, dAs, dBs, Cb, **kw)
+            assert torch.equal(Cb, C.to(torch.bfloat16))
+        # bf16 bias: the same as its float value
+        b16 = dev(bias).to(torch.bfloat16)
+        C1 = torch.empty(M, N, dtype=torch.float32, device="cuda"); C2 = torch.empty_like(C1)
+        hk.dispatch_micro(dA, dB, dAs, dBs, C1, bias=b16, activation=activation)
+        hk.dispatch_micro(dA, dB, dAs, dBs, C2, bias=b16.float(), activation=activation)
+        torch.cuda.synchronize()
+        assert torch.equal(C1, C2)
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+        hk.tk_kernel.set_relayout(prev_r)
+
+
+def test_fused_epilogue_automatic_path_with_relayout(hk):
+    """The automatic path of a large row-major problem (pre-pass + walking tiled kernel) carries the epilogue along."""
+    M = N = 4096; K = 8192
+    g = torch.Generator(device="cuda"); g.manual_seed(5)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.05, 2)
+    bias = torch.randn(N, device="cuda", generator=g)
+    rs = torch.rand(M, device="cuda", generator=g) + 0.5
+    acc = torch.empty(M, N, dtype=torch.float32, device="cuda"); C = torch.empty_like(acc)
+    hk.dispatch_micro(a, b, asc, bsc, acc)
+    hk.dispatch_micro(a, b, asc, bsc, C, bias=bias, row_scale=rs, activation="relu")
+    torch.cuda.synchronize()
+    want = torch.relu(torch.addcmul(bias[None, :].expand(M, N), acc, rs[:, None].expand(M, N)))  # fma(acc, rs, bias) like the kernel (cs = 1)
+    assert torch.allclose(C, want, rtol=2e-6, atol=1e-5)
+
+
 # ------------------------------------------------------------------ stream capture
 def test_graph_capture_replays_match_eager(hk):
     """A size at which the eager path takes the re-layout pre-pass (workspace from the stream-ordered allocator): under

@@ -304,3 +304,20 @@ def test_bf16_rounding_vs_torch():
     got_c = np.array([co.lib().mxfp6o_f32_to_bf16(float(v)) for v in x[-200:]], dtype=np.uint16)
     assert np.array_equal(got_c, exp[-200:])
     assert np.array_equal(o.bf16_bits_to_f32(exp).view(np.uint32) >> 16, exp.astype(np.uint32))
+
+
+def test_epilogue_closed_forms():
+    """The fused-epilogue definitions at points with known values and through their identities (a wrong sign,
+    a dropped 1/2 or sqrt 2, scale and bias applied in the wrong order or along the wrong axis all fail here)."""
+    y = np.array([[-3.0, -1.0, 0.0, 0.5, 2.0]])
+    assert np.array_equal(o.epilogue_ref(y, activation="relu"), [[0.0, 0.0, 0.0, 0.5, 2.0]])
+    g = o.epilogue_ref(y, activation="gelu")
+    # Phi(1) = 0.841344746068543, Phi(2) = 0.977249868051821, Phi(3) = 0.998650101968370 (standard normal CDF)
+    assert np.allclose(g, [[-3 * (1 - 0.998650101968370), -(1 - 0.841344746068543), 0.0, 0.5 * 0.691462461274013, 2 * 0.977249868051821]], atol=1e-14)
+    assert np.allclose(g - o.epilogue_ref(-y, activation="gelu"), y, atol=1e-14)        # gelu(y) - gelu(-y) = y
+    s = o.epilogue_ref(y, activation="silu")
+    assert np.allclose(s, y / (1 + np.exp(-y))) and np.allclose(s - o.epilogue_ref(-y, activation="silu"), y)  # silu(y) - silu(-y) = y
+    assert np.isclose(s[0, 4], 2 / (1 + np.exp(-2.0))) and np.isclose(s[0, 1], -0.2689414213699951)
+    acc = np.arange(6, dtype=np.float64).reshape(2, 3)
+    out = o.epilogue_ref(acc, bias=[10, 20, 30], row_scale=[1, 2], col_scale=[1, 10, 100])
+    assert np.array_equal(out, [[10, 30, 230], [16, 100, 1030]])  # (acc * rs * cs) + bias, bias per column, rs per row
