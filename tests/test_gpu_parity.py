@@ -451,6 +451,12 @@ def test_torch_op_and_linear_module(hk):
     got = y.view(torch.int16).cpu().numpy().view(np.uint16).reshape(48, 160)
     assert np.array_equal(got, o.f32_to_bf16_bits(torch.ops.hipkittensp.mxfp6_gemm(dev(xp), dev(wp), dev(xs), dev(ws), 2, 2, 0, 0, True).cpu().numpy()))
     assert o.rel_err(o.bf16_bits_to_f32(got), ref) <= 2 ** -7      # bf16 rounding of an in-tolerance result
+    # bias and activation ride in the GEMM's epilogue
+    b = rng.standard_normal(160).astype(np.float32)
+    lin2 = torch_op.MXFP6Linear(dev(w), bias=dev(b), activation="silu")
+    y2 = lin2(dev(x)).float().cpu().numpy().reshape(48, 160)
+    want = o.epilogue_ref(ref, bias=b, activation="silu")
+    assert o.rel_err(y2, want) <= 2 ** -7
 
 
 # ------------------------------------------------------------------ edge cases
