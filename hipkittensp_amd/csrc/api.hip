@@ -192,7 +192,7 @@ int mxfp6_quantize(const float* X, void* packed, void* scales, int rows, int K, 
   return mxfp6_quantize_ex(X, packed, scales, rows, K, fmt, MXFP6_LAYOUT_ROW, stream);
 }
 
-int mxfp6_quantize_ex(const float* X, void* packed, void* scales, int rows, int K, int fmt, int layout, void* stream) {
+static int quantize_common(const void* X, int x_bf16, void* packed, void* scales, int rows, int K, int fmt, int layout, void* stream) {
   if (rows < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
   if (layout != MXFP6_LAYOUT_ROW && layout != MXFP6_LAYOUT_TILE) return MXFP6_EINVAL_LAYOUT;
   if (layout == MXFP6_LAYOUT_TILE && (rows % 32 || K % 128)) return MXFP6_EINVAL_SHAPE;
@@ -202,8 +202,16 @@ int mxfp6_quantize_ex(const float* X, void* packed, void* scales, int rows, int 
   if (((uintptr_t)X & 15) || ((uintptr_t)packed & 3)) return MXFP6_EINVAL_ALIGN;
   int rc = check_device();
   if (rc) return rc;
-  hipError_t e = mxfp6::launch_quantize(X, (uint8_t*)packed, (uint8_t*)scales, rows, K, fmt, layout, (hipStream_t)stream);
+  hipError_t e = mxfp6::launch_quantize(X, x_bf16, (uint8_t*)packed, (uint8_t*)scales, rows, K, fmt, layout, (hipStream_t)stream);
   return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
+int mxfp6_quantize_ex(const float* X, void* packed, void* scales, int rows, int K, int fmt, int layout, void* stream) {
+  return quantize_common(X, 0, packed, scales, rows, K, fmt, layout, stream);
+}
+
+int mxfp6_quantize_bf16(const void* X, void* packed, void* scales, int rows, int K, int fmt, int layout, void* stream) {
+  return quantize_common(X, 1, packed, scales, rows, K, fmt, layout, stream);
 }
 
 const char* mxfp6_strerror(int code) {
@@ -222,7 +230,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 105; }
+int mxfp6_abi_version(void) { return 106; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -19,61 +19,72 @@ namespace mxfp6 {
 // 16 rows x one K-tile (512 input bytes per row, four whole lines), which is half of a 3 KB output tile and again
 // 1536 contiguous bytes; a block's 24 bytes are three 8-byte stores (an aligned 8-byte run never straddles the
 // 16-byte pieces the tile-major order permutes).
-constexpr int kQWaves = 4, kQChunk = 64 * 128;  // waves per workgroup; bytes a wave fetches at a time (64 blocks)
+constexpr int kQWaves = 4;  // waves per workgroup; a wave fetches 64 blocks at a time (8 KB of fp32, 4 KB of bf16)
 
 __device__ __forceinline__ void dma16_q(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_base), "v"(voff), "s"(rsrc) : "memory");
 }
 
-template <int FMT>
-__global__ __launch_bounds__(kQWaves * 64) void quantize_kernel(const float* __restrict__ X, uint8_t* __restrict__ packed,
+// In: float, or uint16_t for bf16 (the same values after the exact widening: the bf16 instruction
+// v_cvt_scalef32_pk32_{fp6,bf6}_bf16 was checked against the fp32 one on 1 M values per format, no difference).
+template <int FMT, typename In>
+__global__ __launch_bounds__(kQWaves * 64) void quantize_kernel(const In* __restrict__ X, uint8_t* __restrict__ packed,
                                                               uint8_t* __restrict__ scales, long nblocks, int nkb, int layout) {
   constexpr int EMAX = FMT == 2 ? 2 : 4;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[kQWaves * kQChunk];
+  constexpr int BB = 32 * (int)sizeof(In), P = BB / 16;  // bytes and 16-byte pieces of a block
+  constexpr int kChunk = 64 * BB, NLD = kChunk / 1024;   // bytes and direct loads of a chunk
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[kQWaves * kChunk];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kQChunk;
+  const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kChunk;
   const long nchunks = (nblocks + 63) / 64;
   const long stride = (long)gridDim.x * kQWaves;
   long chunk = (long)blockIdx.x * kQWaves + wave;
   const int nkt = nkb / 4;  // tile-major only: K-tiles per row
 
-  // slot s = q * 64 + lane of load q holds piece (s % 8) ^ (b & 7) of the chunk's block b = s / 8; tile-major:
+  // slot s = q * 64 + lane of load q holds piece (s % P) ^ (b % P) of the chunk's block b = s / P; tile-major:
   // block b is K-block b % 4 of row b / 4 of the chunk
-  int voff[8];
+  int voff[NLD];
 #pragma unroll
-  for (int q = 0; q < 8; q++) {
-    const int sl = q * 64 + lane, b = sl >> 3, c = (sl & 7) ^ (b & 7);
-    voff[q] = layout ? (b >> 2) * (nkb * 128) + (b & 3) * 128 + c * 16 : (b * 8 + c) * 16;
+  for (int q = 0; q < NLD; q++) {
+    const int sl = q * 64 + lane, b = sl / P, c = (sl % P) ^ (b % P);
+    voff[q] = layout ? (b >> 2) * (nkb * BB) + (b & 3) * BB + c * 16 : (b * P + c) * 16;
   }
   auto fetch = [&](long ch) __attribute__((always_inline)) {
     // the resource covers this chunk only (the whole input may exceed 4 GB); bytes past the end read as zero
     if (layout) {
       const long g16 = ch / nkt, kt = ch - g16 * nkt;
-      const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + (g16 * 16 * nkb + kt * 4) * 128, (uint32_t)(15 * nkb * 128 + 512));
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + (g16 * 16 * nkb + kt * 4) * BB, (uint32_t)(15 * nkb * BB + 4 * BB));
 #pragma unroll
-      for (int q = 0; q < 8; q++) dma16_q(r, buf + q * 1024, voff[q]);
+      for (int q = 0; q < NLD; q++) dma16_q(r, buf + q * 1024, voff[q]);
     } else {
-      const long left = nblocks * 128 - ch * kQChunk;
-      const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + ch * kQChunk, (uint32_t)(left < kQChunk ? left : kQChunk));
+      const long left = nblocks * BB - ch * kChunk;
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + ch * kChunk, (uint32_t)(left < kChunk ? left : kChunk));
 #pragma unroll
-      for (int q = 0; q < 8; q++) dma16_q(r, buf + q * 1024, voff[q]);
+      for (int q = 0; q < NLD; q++) dma16_q(r, buf + q * 1024, voff[q]);
     }
   };
   if (chunk < nchunks) fetch(chunk);
   for (; chunk < nchunks; chunk += stride) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    v4f x[8];
+    v4i x[P];
 #pragma unroll
-    for (int c = 0; c < 8; c++) x[c] = *reinterpret_cast<const v4f*>(smem + wave * kQChunk + lane * 128 + ((c ^ (lane & 7)) * 16));
+    for (int c = 0; c < P; c++) x[c] = *reinterpret_cast<const v4i*>(smem + wave * kChunk + lane * BB + ((c ^ (lane % P)) * 16));
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if (chunk + stride < nchunks) fetch(chunk + stride);  // the buffer is free again: the next chunk streams in under the arithmetic
 
     float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; i++)
+    for (int i = 0; i < P; i++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) amax = fmaxf(amax, fabsf(x[i][j]));
+      for (int j = 0; j < 4; j++) {
+        if constexpr (sizeof(In) == 4) {
+          amax = fmaxf(amax, fabsf(__int_as_float(x[i][j])));
+        } else {
+          amax = fmaxf(amax, fabsf(__int_as_float(x[i][j] << 16)));
+          amax = fmaxf(amax, fabsf(__int_as_float(x[i][j] & (int)0xffff0000)));
+        }
+      }
     int sb = 0;
     if (amax > 0.f) {
       const uint32_t u = __float_as_uint(amax);
@@ -82,14 +93,25 @@ __global__ __launch_bounds__(kQWaves * 64) void quantize_kernel(const float* __r
       sb = fl - EMAX + 127;
       sb = sb < 0 ? 0 : (sb > 254 ? 254 : sb);
     }
-    v16f ev, od;
-#pragma unroll
-    for (int i = 0; i < 16; i++) ev[i] = x[i / 2][(2 * i) & 3], od[i] = x[i / 2][(2 * i + 1) & 3];
     const float scale = __uint_as_float((uint32_t)sb << 23);  // 2^(sb - 127); the instruction uses the exponent field
     typedef unsigned v6u __attribute__((ext_vector_type(6)));
     v6u w;
-    if constexpr (FMT == 2) w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, scale);
-    else w = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(ev, od, scale);
+    if constexpr (sizeof(In) == 4) {
+      v16f ev, od;
+#pragma unroll
+      for (int i = 0; i < 16; i++) ev[i] = __int_as_float(x[i / 2][(2 * i) & 3]), od[i] = __int_as_float(x[i / 2][(2 * i + 1) & 3]);
+      if constexpr (FMT == 2) w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, scale);
+      else w = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(ev, od, scale);
+    } else {
+      typedef __bf16 v32bf __attribute__((ext_vector_type(32)));
+      typedef int v16i __attribute__((ext_vector_type(16)));
+      v16i raw;
+#pragma unroll
+      for (int i = 0; i < 16; i++) raw[i] = x[i / 4][i & 3];
+      const v32bf xb = __builtin_bit_cast(v32bf, raw);
+      if constexpr (FMT == 2) w = __builtin_amdgcn_cvt_scalef32_pk32_fp6_bf16(xb, scale);
+      else w = __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(xb, scale);
+    }
     if (layout == 0) {
       const long b = chunk * 64 + lane;
       if (b >= nblocks) continue;
@@ -110,15 +132,15 @@ __global__ __launch_bounds__(kQWaves * 64) void quantize_kernel(const float* __r
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-hipError_t launch_quantize(const float* X, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s) {
+hipError_t launch_quantize(const void* X, int x_bf16, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s) {
   const long nblocks = (long)rows * (K / 32);
   if (nblocks == 0) return hipSuccess;
   const long nchunks = (nblocks + 63) / 64, want = (nchunks + kQWaves - 1) / kQWaves;
   const unsigned grid = (unsigned)(want < 256 * 5 ? want : 256 * 5);  // five workgroups of 32 KB LDS fit a CU
-  if (fmt == 2)
-    quantize_kernel<2><<<grid, kQWaves * 64, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
-  else
-    quantize_kernel<3><<<grid, kQWaves * 64, 0, s>>>(X, packed, scales, nblocks, K / 32, layout);
+#define MXFP6_Q(FMT, T) quantize_kernel<FMT, T><<<grid, kQWaves * 64, 0, s>>>((const T*)X, packed, scales, nblocks, K / 32, layout)
+  if (fmt == 2) { if (x_bf16) MXFP6_Q(2, uint16_t); else MXFP6_Q(2, float); }
+  else { if (x_bf16) MXFP6_Q(3, uint16_t); else MXFP6_Q(3, float); }
+#undef MXFP6_Q
   return hipGetLastError();
 }
 

@@ -139,14 +139,14 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
 
 
 def quantize(X, fmt: int = E2M3, layout: int = LAYOUT_ROW):
-    """fp32 [rows, K] on the GPU -> (packed uint8 [rows, 3K/4], scales uint8 [rows, K/32]).
+    """fp32 or bf16 [rows, K] on the GPU -> (packed uint8 [rows, 3K/4], scales uint8 [rows, K/32]).
     With layout=LAYOUT_TILE packed bytes and scales are written tile-major (rows % 32 == 0, K % 128 == 0;
     scales [rows, ceil(K/512) * 16], padding zero)."""
     import torch
 
     X = _as_tensor(X, "X")
-    if X.dtype != torch.float32:
-        raise RuntimeError(f"X: expected dtype float32, got {X.dtype}")
+    if X.dtype not in (torch.float32, torch.bfloat16):
+        raise RuntimeError(f"X: expected dtype float32 or bfloat16, got {X.dtype}")
     if fmt not in (E2M3, E3M2):
         raise RuntimeError("fmt must be 2 (e2m3) or 3 (e3m2)")
     rows, K = _rows_cols(X, "X")
@@ -159,7 +159,8 @@ def quantize(X, fmt: int = E2M3, layout: int = LAYOUT_ROW):
     alloc = torch.zeros if sw != K // 32 else torch.empty  # the quantiser does not write padding bytes
     scales = alloc(*X.shape[:-1], sw, dtype=torch.uint8, device=X.device)
     with torch.cuda.device(X.device):
-        rc = _lib.lib().mxfp6_quantize_ex(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, layout, _stream())
+        fn = _lib.lib().mxfp6_quantize_bf16 if X.dtype == torch.bfloat16 else _lib.lib().mxfp6_quantize_ex
+        rc = fn(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, layout, _stream())
     _lib.check(rc, "quantize")
     return packed, scales
 

@@ -67,6 +67,6 @@ class MXFP6Linear(torch.nn.Module):
         self.register_buffer("weight_scale", scales)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        xp, xs = tk_kernel.quantize(x.to(torch.float32).contiguous(), self.fmt_x)
+        xp, xs = tk_kernel.quantize((x if x.dtype == torch.bfloat16 else x.to(torch.float32)).contiguous(), self.fmt_x)
         return mxfp6_gemm(xp, self.weight_packed, xs, self.weight_scale, self.fmt_x, self.fmt_w, tk_kernel.LAYOUT_ROW, self.layout_w,
                           bias=self.bias, activation=self.activation)

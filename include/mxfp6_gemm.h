@@ -143,6 +143,12 @@ int mxfp6_gemm_ex(const void *A_packed, const void *B_packed, const void *A_scal
 int mxfp6_quantize_ex(const float *X, void *packed, void *scales, int rows, int K, int fmt, int layout,
                       void *hip_stream);
 
+/* mxfp6_quantize_ex for bf16 input (X: rows x K bf16, 16-byte aligned): the values a float copy of X would give,
+ * without the copy.  Activations of bf16 models are the usual input; no counterpart in the reference, whose
+ * harness converts on the host side (kernels/gemm/bf16fp32/utils.py:28-34). */
+int mxfp6_quantize_bf16(const void *X_bf16, void *packed, void *scales, int rows, int K, int fmt, int layout,
+                        void *hip_stream);
+
 /*
  * mxfp6_gemm_ex with work fused into the epilogue, in fp32 on the accumulators before the output rounding:
  *   C[m][n] = act(acc[m][n] * row_scale[m] * col_scale[n] + bias[n])

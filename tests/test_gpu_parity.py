@@ -505,6 +505,14 @@ def test_gpu_quantiser_bit_exact(hk, fmt, kind):
     assert np.array_equal(packed.cpu().numpy(), ep)
     codes, s2 = o.quantise(x, fmt)
     assert np.array_equal(o.pack_fp6(codes), ep) and np.array_equal(s2, es)
+    # bf16 input: the quantisation of the same values widened to fp32, in both layouts
+    xb = dev(x[:288]).to(torch.bfloat16)
+    ep, es = co.quantise(xb.float().cpu().numpy(), fmt)
+    for layout in (0, 1):
+        packed, scales = hk.quantize(xb, fmt, layout=layout)
+        if layout:
+            packed, scales = hk.tile_operand(packed, untile=True), hk.tile_scales(scales, 1024, untile=True)
+        assert np.array_equal(scales.cpu().numpy(), es) and np.array_equal(packed.cpu().numpy(), ep)
 
 
 # ------------------------------------------------------------------ full-size configurations
