@@ -39,6 +39,8 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_gemm_ex.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp]
         L.mxfp6_gemm_fused.restype = ci
         L.mxfp6_gemm_fused.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, ci, vp, vp, ci, vp]
+        L.mxfp6_gemm_fused_fp6.restype = ci
+        L.mxfp6_gemm_fused_fp6.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, ci, vp, vp, ci, vp]
         L.mxfp6_quantize_ex.restype = ci
         L.mxfp6_quantize_ex.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.mxfp6_quantize_bf16.restype = ci

@@ -79,8 +79,10 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
   return true;
 }
 
-int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
-                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream, const mxfp6::Epilogue& ep = mxfp6::Epilogue()) {
+// The argument checks shared by the gemm entry points (c_align: alignment mask of C).  *empty: nothing to compute.
+int check_gemm_args(const void* A, const void* B, const void* As, const void* Bs, const void* C, int M, int N, int K, int fmt_a, int fmt_b,
+                    uintptr_t c_align, int layout_a, int layout_b, const mxfp6::Epilogue& ep, bool* empty) {
+  *empty = false;
   if (M < 0 || N < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
   if ((fmt_a != MXFP6_FMT_E2M3 && fmt_a != MXFP6_FMT_E3M2) || (fmt_b != MXFP6_FMT_E2M3 && fmt_b != MXFP6_FMT_E3M2))
     return MXFP6_EINVAL_FMT;
@@ -88,18 +90,29 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     return MXFP6_EINVAL_LAYOUT;
   if ((layout_a == MXFP6_LAYOUT_TILE && (M % 32 || K % 128)) || (layout_b == MXFP6_LAYOUT_TILE && (N % 32 || K % 128)))
     return MXFP6_EINVAL_SHAPE;
-  if (M == 0 || N == 0) return MXFP6_OK;
+  if (M == 0 || N == 0) {
+    *empty = true;
+    return MXFP6_OK;
+  }
   if (!C) return MXFP6_EINVAL_PTR;
   if (K > 0 && (!A || !B || !As || !Bs)) return MXFP6_EINVAL_PTR;
-  if (((uintptr_t)A & 3) || ((uintptr_t)B & 3) || ((uintptr_t)C & (f32out ? 3 : 1))) return MXFP6_EINVAL_ALIGN;
+  if (((uintptr_t)A & 3) || ((uintptr_t)B & 3) || ((uintptr_t)C & c_align)) return MXFP6_EINVAL_ALIGN;
   // the tiled kernel reads four floats (or four bf16) of the per-column vectors at a time
   if (((uintptr_t)ep.col_scale & 15) || ((uintptr_t)ep.row_scale & 3) || ((uintptr_t)ep.bias & (ep.bias_bf16 ? 7 : 15))) return MXFP6_EINVAL_ALIGN;
   if (ep.act < 0 || ep.act > 3) return MXFP6_EINVAL_EPILOGUE;
   if ((long)M * N >= (1L << 40) || (long)K / 4 * 3 * 256 >= (1L << 31)) return MXFP6_EINVAL_SHAPE;
-  int rc = check_device();
+  return MXFP6_OK;
+}
+
+int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
+                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream, const mxfp6::Epilogue& ep = mxfp6::Epilogue()) {
+  bool empty;
+  int rc = check_gemm_args(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, f32out ? 3 : 1, layout_a, layout_b, ep, &empty);
+  if (rc || empty) return rc;
+  rc = check_device();
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  if (K == 0) {
+  if (K == 0 && !mxfp6::epilogue_any(ep)) {
     hipError_t e = mxfp6::launch_fill_zero(C, (size_t)M * N * (f32out ? 4 : 2), s);
     return e == hipSuccess ? MXFP6_OK : (int)e;
   }
@@ -107,7 +120,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   g.ep = ep;
   const int force = g_force.load(std::memory_order_relaxed);
   hipError_t e;
-  if (force == 1) {
+  if (K == 0) {
+    e = mxfp6::launch_gemm_generic(g, s);  // act(bias) everywhere: the generic kernel's K loop runs zero times
+  } else if (force == 1) {
     e = mxfp6::launch_gemm_generic(g, s);
   } else if (force == 2 || force == 5 || force == 6) {
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
@@ -157,6 +172,50 @@ int mxfp6_gemm_fused(const void* A, const void* B, const void* As, const void* B
   mxfp6::Epilogue ep;
   ep.bias = bias, ep.bias_bf16 = bias_bf16 != 0, ep.row_scale = row_scale, ep.col_scale = col_scale, ep.act = activation;
   return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, out_f32 != 0, layout_a, layout_b, stream, ep);
+}
+
+int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const void* Bs, void* C_packed, void* C_scale, int M, int N,
+                         int K, int fmt_a, int fmt_b, int layout_a, int layout_b, int fmt_c, const void* bias, int bias_bf16,
+                         const float* row_scale, const float* col_scale, int activation, void* stream) {
+  if (fmt_c != MXFP6_FMT_E2M3 && fmt_c != MXFP6_FMT_E3M2) return MXFP6_EINVAL_FMT;
+  if (N < 0 || N % 32 != 0) return MXFP6_EINVAL_SHAPE;
+  mxfp6::Epilogue ep;
+  ep.bias = bias, ep.bias_bf16 = bias_bf16 != 0, ep.row_scale = row_scale, ep.col_scale = col_scale, ep.act = activation;
+  bool empty;
+  int rc = check_gemm_args(A, B, As, Bs, C_packed, M, N, K, fmt_a, fmt_b, 7, layout_a, layout_b, ep, &empty);
+  if (rc || empty) return rc;
+  if (!C_scale) return MXFP6_EINVAL_PTR;
+  rc = check_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  // the tiled kernel quantises its accumulators itself; where another kernel is the better one (few rows of A: C is
+  // small there) the product goes to an fp32 workspace of the stream-ordered allocator and through the quantiser
+  mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C_packed, M, N, K, fmt_a, fmt_b, false, layout_a, layout_b};
+  const int force = g_force.load(std::memory_order_relaxed);
+  const bool tiled = K > 0 && mxfp6::gemm_tiled_supports(g) &&
+                     (force == 2 || force == 5 || force == 6 ||
+                      (force == 0 && !mxfp6::gemm_skinny_supports(g) && !mxfp6::gemm_mid_preferred(g)));
+  if (tiled) {
+    g.ep = ep, g.C_scale = (uint8_t*)C_scale, g.fmt_c = fmt_c;
+    g.tile_rows = force == 5 ? 128 : force == 6 ? 256 : 0;
+    hipError_t e;
+    if (force != 0 || !relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
+    return e == hipSuccess ? MXFP6_OK : (int)e;
+  }
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return (int)hipErrorStreamCaptureUnsupported;
+  }
+  float* tmp = nullptr;
+  if (hipMallocAsync((void**)&tmp, (size_t)M * N * 4, s) != hipSuccess || !tmp) return (int)hipGetLastError();
+  rc = gemm_common(A, B, As, Bs, tmp, M, N, K, fmt_a, fmt_b, true, layout_a, layout_b, stream, ep);
+  if (rc == MXFP6_OK) {
+    const hipError_t e = mxfp6::launch_quantize(tmp, 0, (uint8_t*)C_packed, (uint8_t*)C_scale, M, N, fmt_c, MXFP6_LAYOUT_ROW, s);
+    rc = e == hipSuccess ? MXFP6_OK : (int)e;
+  }
+  const hipError_t fe = hipFreeAsync(tmp, s);
+  return rc != MXFP6_OK ? rc : (fe == hipSuccess ? MXFP6_OK : (int)fe);
 }
 
 int mxfp6_tile_operand(const void* src, void* dst, int rows, int K, int tile, void* stream) {
@@ -230,7 +289,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 106; }
+int mxfp6_abi_version(void) { return 107; }
 
 #pragma GCC visibility pop
 }  // extern "C"

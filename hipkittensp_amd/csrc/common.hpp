@@ -20,6 +20,17 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // unrounded accumulators, used to state the accuracy contract before the bf16 rounding).
 struct OutBf16 { typedef uint16_t type; };
 struct OutF32 { typedef float type; };
+struct OutFp6 { typedef uint8_t type; };  // C re-quantised to MXFP6: packed [M, 3N/4] + E8M0 [M, N/32] (tiled kernel only)
+
+// E8M0 byte of a 32-block with largest magnitude amax (floor(log2(amax)) - emax, clamped; 0 for an all-zero block)
+__device__ __forceinline__ int e8m0_of_amax(float amax, int emax) {
+  if (!(amax > 0.f)) return 0;
+  const uint32_t u = __float_as_uint(amax);
+  const int be = (int)(u >> 23);
+  const int fl = be ? be - 127 : (31 - __clz((int)u)) - 149;  // fp32 subnormals included
+  const int sb = fl - emax + 127;
+  return sb < 0 ? 0 : (sb > 254 ? 254 : sb);
+}
 
 // fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {

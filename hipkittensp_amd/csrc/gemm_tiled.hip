@@ -103,6 +103,8 @@ struct TiledArgs {
   void* C;
   int M, N, K, tiles_m, tiles_n, layout_a, layout_b;
   Epilogue ep;
+  uint8_t* C_scale;  // fp6 output only
+  int fmt_c;
 };
 
 // FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
@@ -446,6 +448,59 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   };
   auto epilogue = [&]<bool EDGE>(int rows_a, int rows_b) __attribute__((always_inline)) {
     const auto g = fresh_args();
+    if constexpr (sizeof(OutT) == 1) {
+      // C re-quantised to MXFP6 along N (the next GEMM's K): a 32-block of row m is the 16 values of lane (m, h = 0)
+      // and the 16 of lane (m, h = 1) of one 32x32 tile.  The wave's two tiles of a band (j = 0, 1) are traded with
+      // v_permlane32_swap, register by register, after which the lower lane holds all of block j = 0 and the upper
+      // lane all of block j = 1: P0[k] = column 8 (k / 4) + k % 4, P1[k] = that + 4.  Then exactly the quantiser:
+      // amax -> E8M0 -> hardware conversion -> 24 bytes and a scale byte per lane.
+      const int N = g->N, nkb = N / 32, fmt_c = g->fmt_c;
+      const long m0 = (long)(tile_cur & 0xffff) * kBM + wm * (TM * 32) + r32;
+      const int blk = (tile_cur >> 16) * (kBN / 32) + wn * TN + h;  // 32-block index along N of this lane's block
+      uint8_t* cp = reinterpret_cast<uint8_t*>(g->C);
+      uint8_t* sp = g->C_scale;
+      const int M = g->M;
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        float p0[16], p1[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+          const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[i][0][k]), __float_as_uint(acc[i][1][k]), false, false);
+          p0[k] = __uint_as_float(sw[0]), p1[k] = __uint_as_float(sw[1]);
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) amax = fmaxf(amax, fmaxf(fabsf(p0[k]), fabsf(p1[k])));
+        const int sb = e8m0_of_amax(amax, fmt_c == 2 ? 2 : 4);
+        const float scale = __uint_as_float((uint32_t)sb << 23);
+        v16f ev, od;  // even and odd columns of the block: column n = 8 q + r is p0[4 q + r] for r < 4, p1[4 q + r - 4] otherwise
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+          const int ne = 2 * t, no = 2 * t + 1;
+          ev[t] = (ne & 4) ? p1[4 * (ne >> 3) + (ne & 3)] : p0[4 * (ne >> 3) + (ne & 3)];
+          od[t] = (no & 4) ? p1[4 * (no >> 3) + (no & 3)] : p0[4 * (no >> 3) + (no & 3)];
+        }
+        typedef unsigned v6u __attribute__((ext_vector_type(6)));
+        // a real branch (the empty asm keeps it one): with both conversions issued on the same sources and a select
+        // behind them, the second one's result came out wrong from the third dword on
+        v6u w;
+        if (fmt_c == 2) {
+          w = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, scale);
+          asm volatile("" : "+v"(w));
+        } else {
+          w = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(ev, od, scale);
+          asm volatile("" : "+v"(w));
+        }
+        const long m = m0 + i * 32;
+        if (m < M && blk < nkb) {
+          u32x2* dst = reinterpret_cast<u32x2*>(cp + (m * nkb + blk) * 24);
+#pragma unroll
+          for (int c = 0; c < 3; c++) dst[c] = u32x2{w[2 * c], w[2 * c + 1]};
+          sp[m * nkb + blk] = (uint8_t)sb;
+        }
+      }
+      return;
+    }
     const int N = g->N, N2 = N * (int)sizeof(OutT);  // N2: bytes per row of C
     // the resource ends with the tile's last valid element
     const __amdgpu_buffer_rsrc_t rC = make_rsrc((OutT*)g->C + (size_t)(tile_cur & 0xffff) * kBM * N + (size_t)(tile_cur >> 16) * kBN,
@@ -608,9 +663,12 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int bm = tile_rows(g);
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + kBN - 1) / kBN;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep};
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c};
   const int grid = grid_size(g, tm * tn);
-  if (epilogue_any(g.ep)) {
+  if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
+    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, true><<<grid, NW * 64, 0, s>>>(ta);
+    else gemm_tiled_kernel<FA, FB, Out, 4, true><<<grid, NW * 64, 0, s>>>(ta);
+  } else if (epilogue_any(g.ep)) {
     if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, true><<<grid, NW * 64, 0, s>>>(ta);
     else gemm_tiled_kernel<FA, FB, Out, 4, true><<<grid, NW * 64, 0, s>>>(ta);
   } else {
@@ -622,7 +680,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
 
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s) {
 #define MXFP6_CASE(FA, FB) \
-  if (g.fmt_a == FA && g.fmt_b == FB) return g.f32out ? launch<FA, FB, OutF32>(g, s) : launch<FA, FB, OutBf16>(g, s);
+  if (g.fmt_a == FA && g.fmt_b == FB) return g.fmt_c ? launch<FA, FB, OutFp6>(g, s) : g.f32out ? launch<FA, FB, OutF32>(g, s) : launch<FA, FB, OutBf16>(g, s);
   MXFP6_CASE(2, 2) MXFP6_CASE(2, 3) MXFP6_CASE(3, 2) MXFP6_CASE(3, 3)
 #undef MXFP6_CASE
   return hipErrorInvalidValue;

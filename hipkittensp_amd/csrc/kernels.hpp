@@ -15,6 +15,8 @@ struct GemmArgs {
   int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (operand: 32 rows x 128 elements in LDS image order; scales: 32 rows x 16 bytes)
   int tile_rows = 0;               // tiled kernel: rows of A per output tile, 128 or 256; 0 = chosen per shape
   Epilogue ep;                     // fused bias / scales / activation (all optional)
+  uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
+  int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output
 };
 
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);

@@ -78,10 +78,13 @@ _ACTS = {None: 0, "none": 0, "relu": 1, "gelu": 2, "silu": 3, 0: 0, 1: 1, 2: 2, 
 
 
 def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, layout_a: int = LAYOUT_ROW,
-                   layout_b: int = LAYOUT_ROW, bias=None, row_scale=None, col_scale=None, activation=None) -> None:
+                   layout_b: int = LAYOUT_ROW, bias=None, row_scale=None, col_scale=None, activation=None, C_scale=None,
+                   fmt_c: int = E2M3) -> None:
     """C = dq(A) @ dq(B).T; optionally fused, in fp32 before the output rounding:
     C = act(acc * row_scale[:, None] * col_scale[None, :] + bias[None, :]) with bias [N] float32 or bfloat16,
-    row_scale [M] and col_scale [N] float32, activation one of None / "relu" / "gelu" / "silu"."""
+    row_scale [M] and col_scale [N] float32, activation one of None / "relu" / "gelu" / "silu".
+    With C_scale given, the result is re-quantised to MXFP6 (fmt_c) along N: C is then the packed operand
+    uint8 [M, 3N/4] and C_scale its E8M0 bytes uint8 [M, N/32] (N % 32 == 0), ready to be the next GEMM's A."""
     import torch
 
     A, B = _as_tensor(A, "A"), _as_tensor(B, "B")
@@ -90,7 +93,14 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
     for t, name in ((A, "A"), (B, "B"), (A_scale, "A_scale"), (B_scale, "B_scale")):
         if t.dtype != torch.uint8:
             raise RuntimeError(f"{name}: expected dtype uint8, got {t.dtype}")
-    if C.dtype not in (torch.bfloat16, torch.float32):
+    fp6_out = C_scale is not None
+    if fp6_out:
+        C_scale = _as_tensor(C_scale, "C_scale")
+        if C.dtype != torch.uint8 or C_scale.dtype != torch.uint8:
+            raise RuntimeError("C and C_scale: expected dtype uint8 for the MXFP6 output")
+        if fmt_c not in (E2M3, E3M2):
+            raise RuntimeError("fmt_c must be 2 (e2m3) or 3 (e3m2)")
+    elif C.dtype not in (torch.bfloat16, torch.float32):
         raise RuntimeError(f"C: expected dtype bfloat16 (or float32 for unrounded output), got {C.dtype}")
     if fmt_a not in (E2M3, E3M2) or fmt_b not in (E2M3, E3M2):
         raise RuntimeError("fmt_a / fmt_b must be 2 (e2m3) or 3 (e3m2)")
@@ -110,7 +120,12 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
         want = (rows, scale_width(K, lay))
         if _rows_cols(t, name) != want:
             raise RuntimeError(f"{name}: expected shape [{want[0]}, {want[1]}], got {tuple(t.shape)}")
-    if _rows_cols(C, "C") != (M, N):
+    if fp6_out:
+        if N % 32:
+            raise RuntimeError(f"the MXFP6 output needs N % 32 == 0, got N = {N}")
+        if _rows_cols(C, "C") != (M, N // 4 * 3) or _rows_cols(C_scale, "C_scale") != (M, N // 32):
+            raise RuntimeError(f"C / C_scale: expected shapes [{M}, {N // 4 * 3}] and [{M}, {N // 32}], got {tuple(C.shape)} and {tuple(C_scale.shape)}")
+    elif _rows_cols(C, "C") != (M, N):
         raise RuntimeError(f"C: expected shape [{M}, {N}], got {tuple(C.shape)}")
     if activation not in _ACTS:
         raise RuntimeError(f"activation must be None, 'relu', 'gelu' or 'silu', got {activation!r}")
@@ -125,11 +140,21 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
         if t.dim() != 1 or t.shape[0] != n or not t.is_contiguous():
             raise RuntimeError(f"{name}: expected a contiguous vector of {n} elements, got shape {tuple(t.shape)}")
         extras.append(t)
+    if fp6_out:
+        extras.append(C_scale)
     devs = {t.device for t in (A, B, A_scale, B_scale, C, *extras)}
     if len(devs) != 1:
         raise RuntimeError(f"all tensors must be on one device, got {sorted(map(str, devs))}")
     L = _lib.lib()
     ptr = lambda t: 0 if t is None else t.data_ptr()
+    if fp6_out:
+        with torch.cuda.device(C.device):
+            rc = L.mxfp6_gemm_fused_fp6(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), C_scale.data_ptr(),
+                                        M, N, K, fmt_a, fmt_b, layout_a, layout_b, fmt_c, ptr(bias),
+                                        int(bias is not None and bias.dtype == torch.bfloat16), ptr(row_scale), ptr(col_scale),
+                                        _ACTS[activation], _stream())
+        _lib.check(rc, "dispatch_micro")
+        return
     with torch.cuda.device(C.device):
         rc = L.mxfp6_gemm_fused(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
                                 fmt_a, fmt_b, layout_a, layout_b, int(C.dtype == torch.float32), ptr(bias),

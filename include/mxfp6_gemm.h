@@ -166,6 +166,21 @@ int mxfp6_gemm_fused(const void *A_packed, const void *B_packed, const void *A_s
                      const void *bias, int bias_bf16, const float *row_scale, const float *col_scale, int activation,
                      void *hip_stream);
 
+/*
+ * mxfp6_gemm_fused whose result is re-quantised to MXFP6 along N, i.e. written as the packed operand
+ * C_packed [M, 3N/4] and its E8M0 scales C_scale [M, N/32] (row-major) that the next layer's GEMM takes as A:
+ * exactly mxfp6_quantize(fmt_c) applied to the fp32 result of mxfp6_gemm_fused(out_f32 = 1), without that result
+ * ever reaching memory (0.78 instead of 2 or 4 bytes per output element).  N % 32 == 0; C_packed 8-byte aligned.
+ * The LDS-tiled kernel quantises its accumulators in its epilogue; shapes that run on another kernel (few rows of A,
+ * where C is small) go through an fp32 workspace taken from and returned to the stream-ordered allocator on
+ * hip_stream, and are refused under stream capture (hipErrorStreamCaptureUnsupported).
+ * No counterpart in the reference.
+ */
+int mxfp6_gemm_fused_fp6(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale,
+                         void *C_packed, void *C_scale, int M, int N, int K, int fmt_a, int fmt_b, int layout_a,
+                         int layout_b, int fmt_c, const void *bias, int bias_bf16, const float *row_scale,
+                         const float *col_scale, int activation, void *hip_stream);
+
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);
 

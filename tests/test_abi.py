@@ -30,7 +30,7 @@ def built_lib():
 
 def test_header_declares_the_operator():
     names = _declared_functions()
-    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_gemm_fused", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_quantize_bf16", "mxfp6_tile_operand", "mxfp6_tile_scales",
+    for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_gemm_fused", "mxfp6_gemm_fused_fp6", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_quantize_bf16", "mxfp6_tile_operand", "mxfp6_tile_scales",
                  "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout"):
         assert want in names
 
@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 106
+    assert L.mxfp6_abi_version() == 107
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"

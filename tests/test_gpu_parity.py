@@ -384,6 +384,35 @@ def test_fused_epilogue_every_kernel(hk, kernel, M, N, K, activation):
         hk.tk_kernel.set_relayout(prev_r)
 
 
+@pytest.mark.parametrize("kernel,M,N,K", [(0, 16, 96, 1024), (0, 64, 128, 1024), (0, 70, 64, 96), (5, 300, 288, 640), (6, 300, 288, 640),
+                                          (5, 1024, 4128, 512), (6, 2304, 8224, 896), (0, 4096, 4096, 8192)])
+@pytest.mark.parametrize("fmt_c", [2, 3])
+def test_fp6_requantised_output(hk, kernel, M, N, K, fmt_c):
+    """The GEMM's result written as the next layer's MXFP6 operand: bit for bit the quantiser applied to the fp32 result of
+    the same (fused) call.  Kernels 5 / 6 and the large automatic case quantise the accumulators in the tiled kernel's
+    epilogue (edge tiles, more tiles than CUs, the re-layout pre-pass); the small automatic cases run another kernel into
+    an fp32 workspace and the quantiser."""
+    g = torch.Generator(device="cuda"); g.manual_seed(M + N + K)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.05, 2)
+    bias = torch.randn(N, device="cuda", generator=g)
+    rs = torch.rand(M, device="cuda", generator=g) + 0.5
+    prev = hk.tk_kernel.set_kernel(kernel)
+    try:
+        for kw in (dict(), dict(bias=bias, row_scale=rs, activation="silu")):
+            C = torch.empty(M, N, dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(a, b, asc, bsc, C, **kw)
+            P = torch.full((M, N // 4 * 3), 0xAA, dtype=torch.uint8, device="cuda")
+            S = torch.full((M, N // 32), 0xAA, dtype=torch.uint8, device="cuda")
+            hk.dispatch_micro(a, b, asc, bsc, P, C_scale=S, fmt_c=fmt_c, **kw)
+            torch.cuda.synchronize()
+            ep, es = co.quantise(C.cpu().numpy(), fmt_c)
+            assert np.array_equal(S.cpu().numpy(), es)
+            assert np.array_equal(P.cpu().numpy(), ep)
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+
+
 def test_fused_epilogue_automatic_path_with_relayout(hk):
     """The automatic path of a large row-major problem (pre-pass + walking tiled kernel) carries the epilogue along."""
     M = N = 4096; K = 8192
