@@ -404,35 +404,40 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const bool affine = bias || row_scale || col_scale;
     const int M = g->M, N = g->N;
     const long m0 = (long)(tile_cur & 0xffff) * kBM + wm * (TM * 32) + r32, n0 = (long)(tile_cur >> 16) * kBN + wn * (TN * 32) + 4 * h;
-    // one 32x32 tile at a time, each with its own branches: a branch around all 128 accumulators at once makes the
-    // compiler keep a second copy of them
+    // 32 columns (j) at a time, each with its own branches: a branch around all 128 accumulators at once makes the
+    // compiler keep a second copy of them.  The column vectors of a j are loaded once for all rows (one round of load
+    // latency per j and output tile, not per 32x32 tile).
+    float rs[TM];
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < TM; i++) rs[i] = row_scale && m0 + i * 32 < M ? row_scale[m0 + i * 32] : 1.f;
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
-        if (affine) {
-          const float rs = row_scale && m0 + i * 32 < M ? row_scale[m0 + i * 32] : 1.f;
-          v4f cs[4], bi[4];
+    for (int j = 0; j < TN; j++) {
+      if (affine) {
+        v4f cs[4], bi[4];
 #pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const long n = n0 + j * 32 + q * 8;
-            cs[q] = v4f{1.f, 1.f, 1.f, 1.f}, bi[q] = v4f{0.f, 0.f, 0.f, 0.f};
-            if (n < N) {
-              if (col_scale) cs[q] = *reinterpret_cast<const v4f*>(col_scale + n);
-              if (bias && bias_bf16) {
-                const u32x2 b2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(bias) + n);
-                bi[q] = v4f{__uint_as_float(b2[0] << 16), __uint_as_float(b2[0] & 0xffff0000u), __uint_as_float(b2[1] << 16),
-                            __uint_as_float(b2[1] & 0xffff0000u)};
-              } else if (bias) {
-                bi[q] = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(bias) + n);
-              }
+        for (int q = 0; q < 4; q++) {
+          const long n = n0 + j * 32 + q * 8;
+          cs[q] = v4f{1.f, 1.f, 1.f, 1.f}, bi[q] = v4f{0.f, 0.f, 0.f, 0.f};
+          if (n < N) {
+            if (col_scale) cs[q] = *reinterpret_cast<const v4f*>(col_scale + n);
+            if (bias && bias_bf16) {
+              const u32x2 b2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(bias) + n);
+              bi[q] = v4f{__uint_as_float(b2[0] << 16), __uint_as_float(b2[0] & 0xffff0000u), __uint_as_float(b2[1] << 16),
+                          __uint_as_float(b2[1] & 0xffff0000u)};
+            } else if (bias) {
+              bi[q] = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(bias) + n);
             }
           }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; i++)
 #pragma unroll
           for (int q = 0; q < 4; q++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[i][j][4 * q + e] = fmaf(acc[i][j][4 * q + e] * rs, cs[q][e], bi[q][e]);
-        }
+            for (int e = 0; e < 4; e++) acc[i][j][4 * q + e] = fmaf(acc[i][j][4 * q + e] * rs[i], cs[q][e], bi[q][e]);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
         if (act == 1) {
 #pragma unroll
           for (int e = 0; e < 16; e++) acc[i][j][e] = act_relu(acc[i][j][e]);
@@ -445,6 +450,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
         }
         asm volatile("" : "+v"(acc[i][j]));
       }
+    }
   };
   auto epilogue = [&]<bool EDGE>(int rows_a, int rows_b) __attribute__((always_inline)) {
     const auto g = fresh_args();
