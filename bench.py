@@ -15,7 +15,8 @@ Prints ONE JSON line.  `value` is TFLOP/s of the whole job (wall clock between t
 synchronisations / steps; a step includes the library's re-layout pre-pass).  `roofline` prices the tiled
 GEMM kernel alone against the dense MXFP6 MFMA peak using the mean per-launch duration measured with device
 events on the launch stream; `decode` does
-the same for the M=16 skinny kernel (BASELINE.json configs[3]) against the HBM peak.  `cpu_baseline`
+the same for the M=16 skinny kernel (BASELINE.json configs[3]) against the HBM peak, `quantize` for the
+quantise+pack kernel (fp32 and bf16 sources).  `cpu_baseline`
 times the CPU oracle (oracle/mxfp6_oracle.c, an OpenMP port of dequantise-and-matmul) on a bounded
 sample of the same bytes; it is a reported baseline, not a target.
 """
@@ -195,6 +196,34 @@ def main():
             "achieved": dbytes / (dtev_ms * 1e-3) / 1e9, "unit": "GB/s", "frac": dbytes / (dtev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "launch_ms_mean": dtev_ms,
         }
+    # ---- the quantiser (the step in front of the GEMM at inference time): 8192 x 8192 activations -> packed fp6 + E8M0,
+    # fp32 and bf16 sources, into preallocated outputs through the C ABI (no allocation inside the timed region)
+    del dinputs
+    torch.cuda.empty_cache()
+    from hipkittensp_amd import _lib
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    quant = {"what": "fp32 / bf16 [8192, 8192] -> packed e2m3 + E8M0 scales (row-major), bytes read + written per launch", "bound": "hbm",
+             "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    qx = [torch.randn(8192, 8192, device="cuda") for _ in range(3)]
+    qp = torch.empty(8192, 6144, dtype=torch.uint8, device="cuda")
+    qs = torch.empty(8192, 256, dtype=torch.uint8, device="cuda")
+    for name, fn, xs in (("fp32", L.mxfp6_quantize_ex, qx), ("bf16", L.mxfp6_quantize_bf16, [x.to(torch.bfloat16) for x in qx])):
+        for i in range(args.warmup):
+            fn(xs[i % 3].data_ptr(), qp.data_ptr(), qs.data_ptr(), 8192, 8192, 2, 0, stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(args.steps):
+            rc = fn(xs[i % 3].data_ptr(), qp.data_ptr(), qs.data_ptr(), 8192, 8192, 2, 0, stream)
+        e1.record()
+        torch.cuda.synchronize()
+        assert rc == 0
+        ms = e0.elapsed_time(e1) / args.steps
+        qbytes = 8192 * 8192 * (xs[0].element_size() + 0.75 + 1 / 32)
+        quant[name] = {"launch_ms_mean": ms, "achieved": qbytes / (ms * 1e-3) / 1e9, "frac": qbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "algorithmic_bytes_per_launch": qbytes}
+    del qx, qp, qs
     decode = {
         "metric": "MXFP6 decode GEMM achieved GB/s @M=16,N=8192,K=28672",
         "value": dbytes / (dwall / args.steps) / 1e9,
@@ -236,6 +265,7 @@ def main():
         "tile_major": tile_major,
         "cpu_baseline": cpu,
         "decode": decode,
+        "quantize": quant,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(line))
