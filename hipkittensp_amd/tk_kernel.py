@@ -44,7 +44,7 @@ def _as_tensor(obj, name: str):
         raise RuntimeError(f"{name}: expected a torch Tensor, got {type(obj).__name__}")
     if not obj.is_contiguous():
         raise RuntimeError(f"{name}: tensor must be contiguous")
-    if obj.device.type == "cpu":
+    if not obj.is_cuda:
         raise RuntimeError(f"{name}: tensor must be on a GPU device")
     if obj.dim() > 4:
         raise RuntimeError(f"{name}: expected at most 4 dimensions, got {obj.dim()}")
@@ -65,7 +65,30 @@ def _rows_cols(t, name: str):
 def _stream():
     import torch
 
-    return torch.cuda.current_stream().cuda_stream
+    try:  # the raw handle, without building a Stream object per call
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    except AttributeError:
+        return torch.cuda.current_stream().cuda_stream
+
+
+class _on_device:
+    """`with _on_device(d)` that costs nothing when d is already the current device (the usual case)."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        import torch
+
+        self.ctx = None if device.index is None or device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 def scale_width(K: int, layout: int = LAYOUT_ROW) -> int:
@@ -148,14 +171,14 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
     L = _lib.lib()
     ptr = lambda t: 0 if t is None else t.data_ptr()
     if fp6_out:
-        with torch.cuda.device(C.device):
+        with _on_device(C.device):
             rc = L.mxfp6_gemm_fused_fp6(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), C_scale.data_ptr(),
                                         M, N, K, fmt_a, fmt_b, layout_a, layout_b, fmt_c, ptr(bias),
                                         int(bias is not None and bias.dtype == torch.bfloat16), ptr(row_scale), ptr(col_scale),
                                         _ACTS[activation], _stream())
         _lib.check(rc, "dispatch_micro")
         return
-    with torch.cuda.device(C.device):
+    with _on_device(C.device):
         rc = L.mxfp6_gemm_fused(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
                                 fmt_a, fmt_b, layout_a, layout_b, int(C.dtype == torch.float32), ptr(bias),
                                 int(bias is not None and bias.dtype == torch.bfloat16), ptr(row_scale), ptr(col_scale),
@@ -183,7 +206,7 @@ def quantize(X, fmt: int = E2M3, layout: int = LAYOUT_ROW):
     sw = scale_width(K, layout)
     alloc = torch.zeros if sw != K // 32 else torch.empty  # the quantiser does not write padding bytes
     scales = alloc(*X.shape[:-1], sw, dtype=torch.uint8, device=X.device)
-    with torch.cuda.device(X.device):
+    with _on_device(X.device):
         fn = _lib.lib().mxfp6_quantize_bf16 if X.dtype == torch.bfloat16 else _lib.lib().mxfp6_quantize_ex
         rc = fn(X.data_ptr(), packed.data_ptr(), scales.data_ptr(), rows, K, fmt, layout, _stream())
     _lib.check(rc, "quantize")
@@ -201,7 +224,7 @@ def tile_operand(packed, untile: bool = False):
     if w % 96 or rows % 32:
         raise RuntimeError("tile-major layout needs rows % 32 == 0 and K % 128 == 0")
     out = torch.empty_like(packed)
-    with torch.cuda.device(packed.device):
+    with _on_device(packed.device):
         rc = _lib.lib().mxfp6_tile_operand(packed.data_ptr(), out.data_ptr(), rows, w // 3 * 4, 0 if untile else 1, _stream())
     _lib.check(rc, "tile_operand")
     return out
@@ -221,7 +244,7 @@ def tile_scales(scales, K: int, untile: bool = False):
     if w != src_w:
         raise RuntimeError(f"scales: expected {src_w} bytes per row for K = {K}, got {w}")
     out = torch.empty(*scales.shape[:-1], dst_w, dtype=torch.uint8, device=scales.device)
-    with torch.cuda.device(scales.device):
+    with _on_device(scales.device):
         rc = _lib.lib().mxfp6_tile_scales(scales.data_ptr(), out.data_ptr(), rows, K, 0 if untile else 1, _stream())
     _lib.check(rc, "tile_scales")
     return out
