@@ -44,7 +44,7 @@ def _as_tensor(obj, name: str):
         raise RuntimeError(f"{name}: expected a torch Tensor, got {type(obj).__name__}")
     if not obj.is_contiguous():
         raise RuntimeError(f"{name}: tensor must be contiguous")
-    if not obj.is_cuda:
+    if obj.device.type == "cpu":
         raise RuntimeError(f"{name}: tensor must be on a GPU device")
     if obj.dim() > 4:
         raise RuntimeError(f"{name}: expected at most 4 dimensions, got {obj.dim()}")
