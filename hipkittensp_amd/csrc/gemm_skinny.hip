@@ -42,13 +42,15 @@ __device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt
 
 }  // namespace
 
-// AR = rows of A staged (16 or 32); NW = waves per workgroup
-template <int FA, int FB, typename Out, int AR, int NW>
+// AR = rows of A staged (16 or 32); NW = waves per workgroup; BR = rows of B per workgroup (32, or 16 so that a narrow
+// N still gives every CU a workgroup: the MFMA's other 16 rows then mirror the first and their outputs are dropped)
+template <int FA, int FB, typename Out, int AR, int NW, int BR>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                               typename Out::type* __restrict__ C, int M, int N, int K, int layout_b,
                                                               const Epilogue ep) {
-  constexpr int kBBuf = 32 * 384, kABuf = AR * 384, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then 2 x 1 KB of scales
+  static_assert(BR == 32 || BR == 16, "rows of B per workgroup");
+  constexpr int kBBuf = BR * 384, kABuf = AR * 384, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then 2 x 1 KB of scales
   constexpr int kBuf = kScOff + 2048;
   constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024;                    // direct loads per chunk: 12 and 6 or 12
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kBuf];
@@ -58,25 +60,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, r32 = lane & 31;
   const int nkt = K / 128, sbytes = K / 32, rowbytes = K / 4 * 3;
-  const int n0 = blockIdx.x * 32;
-  const int nrows = min(32, N - n0);
+  const int n0 = blockIdx.x * BR;
+  const int nrows = min(BR, N - n0);
+  const int rt = BR == 32 ? blockIdx.x : blockIdx.x >> 1, half = BR == 32 ? 0 : blockIdx.x & 1;  // tile-major B: row-tile, and which 16 rows of it
 
   // rows that do not exist (n >= N, m >= M) lie past the end of the resource and read as zeros
-  const __amdgpu_buffer_rsrc_t rB = make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
+  const __amdgpu_buffer_rsrc_t rB = layout_b ? make_rsrc(B + (size_t)rt * 32 * rowbytes, (uint32_t)32 * rowbytes)
+                                             : make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, (uint32_t)M * rowbytes);
   // tile-major B: this workgroup's 32 rows are one row-tile, whose scales are nk4 chunks of 512 bytes (row r at r * 16)
   const int nk4 = nkt / 4;
-  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)blockIdx.x * nk4 * 512, (uint32_t)nk4 * 512)
+  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)rt * nk4 * 512, (uint32_t)nk4 * 512)
                                               : make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
   const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * sbytes);
 
   // direct-load address maps: load i fills LDS bytes [i*1024, i*1024 + 1024) of the buffer; slot o = i*64 + lane holds
-  // piece (o % 24) ^ ((row >> 1) & 7) of row o / 24.  Tile-major B: four consecutive 3 KB tiles, copied as they are.
+  // piece (o % 24) ^ ((row >> 1) & 7) of row o / 24.  Tile-major B: four consecutive 3 KB tiles, copied as they are
+  // (BR = 16: the 1536 bytes that this workgroup's 16 rows have in each of them).
   int voff_b[NBL], voff_a[NAL];
 #pragma unroll
   for (int i = 0; i < NBL; i++) {
     const int o = i * 64 + lane, r = o / 24, p = (o - r * 24) ^ ((r >> 1) & 7);
-    voff_b[i] = layout_b ? o * 16 : r * rowbytes + p * 16;
+    constexpr int kPer = BR * 6;  // 16-byte pieces per K-tile of this workgroup's rows
+    voff_b[i] = layout_b ? (o / kPer) * 3072 + half * 1536 + (o % kPer) * 16 : r * rowbytes + p * 16;
   }
 #pragma unroll
   for (int i = 0; i < NAL; i++) {
@@ -84,9 +90,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     voff_a[i] = r * rowbytes + p * 16;
   }
   // scale loads: lane l fetches the 16 bytes of row l % 32 (both halves of the wave fetch the same rows)
-  const int voff_bs = layout_b ? r32 * 16 : r32 * sbytes;
-  const int voff_as = r32 * sbytes;
   const int ra = AR == 16 ? (r32 & 15) : r32;  // AR = 16: lanes 16-31 mirror rows 0-15 (their outputs are never stored)
+  const int rb = BR == 16 ? (r32 & 15) : r32;  // BR = 16: likewise for B
+  const int voff_bs = layout_b ? (half * 16 + rb) * 16 : rb * sbytes;
+  const int voff_as = r32 * sbytes;
 
   const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kBuf;
   const uint8_t* bufp = smem + wave * kBuf;
@@ -97,7 +104,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const int p = u * 6 + 3 * h + c;
-      b_rd[u][c] = layout_b ? u * 3072 + r32 * 96 + ((3 * h + c) ^ ((r32 >> 3) & 1)) * 16 : r32 * 384 + (p ^ ((r32 >> 1) & 7)) * 16;
+      b_rd[u][c] = layout_b ? u * (BR * 96) + rb * 96 + ((3 * h + c) ^ ((rb >> 3) & 1)) * 16 : rb * 384 + (p ^ ((rb >> 1) & 7)) * 16;
       a_rd[u][c] = kBBuf + ra * 384 + (p ^ ((ra >> 1) & 7)) * 16;
     }
 
@@ -126,7 +133,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     issue_chunk(wave);
     for (int j = 0; j < mine; j++) {
       wait_all_loads();
-      const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + r32 * 16);
+      const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + rb * 16);
       const v4i sc_a = *reinterpret_cast<const v4i*>(bufp + kScOff + 1024 + ra * 16);
       v4i fb[4][3], fa[4][3];
 #pragma unroll
@@ -167,8 +174,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 #pragma unroll
     for (int w = 0; w < NW; w++) s += part[(w * 16 + e) * 64 + l];
     const int m = l & 31;
-    const long nn = (long)n0 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
-    if (m < M && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, s, m, nn) : s);
+    const int nl = 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
+    const long nn = (long)n0 + nl;
+    if (m < M && nl < BR && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, s, m, nn) : s);
   }
 }
 
@@ -177,13 +185,22 @@ bool gemm_skinny_supports(const GemmArgs& g) {
   return g.layout_a == 0 && g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
 }
 
+// Geometry.  Few rows of B (N / 32 workgroups would leave half of the CUs idle): 16 rows per workgroup.  Many (N / 32
+// is several times the CU count): half as many waves per workgroup, so that two workgroups share a CU and one's first
+// loads run under the other's stream (a workgroup with a short K range is mostly load latency).
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  const unsigned grid = (g.N + 31) / 32;
-  if (g.M <= 16)
-    gemm_skinny_kernel<FA, FB, Out, 16, 8><<<grid, 8 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b, g.ep);
-  else
-    gemm_skinny_kernel<FA, FB, Out, 32, 6><<<grid, 6 * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_b, g.ep);
+  typedef typename Out::type T;
+  const unsigned wgs32 = (g.N + 31) / 32;
+#define MXFP6_SK(AR, NW, BR) \
+  gemm_skinny_kernel<FA, FB, Out, AR, NW, BR><<<(g.N + BR - 1) / BR, NW * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, g.layout_b, g.ep)
+  const int geo = g.skinny_geometry ? g.skinny_geometry : wgs32 <= 128 ? 2 : wgs32 >= 512 ? 3 : 1;
+  if (g.M <= 16) {
+    if (geo == 2) MXFP6_SK(16, 8, 16); else if (geo == 3) MXFP6_SK(16, 4, 32); else MXFP6_SK(16, 8, 32);
+  } else {
+    if (geo == 2) MXFP6_SK(32, 6, 16); else if (geo == 3) MXFP6_SK(32, 3, 32); else MXFP6_SK(32, 6, 32);
+  }
+#undef MXFP6_SK
   return hipGetLastError();
 }
 

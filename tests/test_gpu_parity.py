@@ -166,6 +166,33 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     check(got, ref, fa, fb, ap, asc, bp, bsc)
     cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=3)
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+    # every workgroup geometry (32 rows of B, 16 rows, 32 rows with half the waves) sums the same products; the order of the
+    # partial sums differs, so they agree to fp32 rounding, and each is held to the oracle
+    for kern in (hk.tk_kernel.KERNEL_SKINNY_32, hk.tk_kernel.KERNEL_SKINNY_16, hk.tk_kernel.KERNEL_SKINNY_HALF):
+        check(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kern), ref, fa, fb, ap, asc, bp, bsc)
+
+
+@pytest.mark.parametrize("kernel", [7, 8, 9])
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 2080, 1536), (5, 17408, 1024)])
+def test_skinny_geometries_tile_major_weights(hk, kernel, M, N, K):
+    """Each geometry with tile-major weights and scales (16 rows per workgroup read half of every 3 KB tile) against the
+    generic kernel on the row-major operands; ragged N only row-major."""
+    g = torch.Generator(device="cuda"); g.manual_seed(N + K)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2)
+    ref = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    prev = hk.tk_kernel.set_kernel(1)
+    try:
+        hk.dispatch_micro(a, b, asc, bsc, ref)
+        hk.tk_kernel.set_kernel(kernel)
+        for lb in ((0, 1) if N % 32 == 0 else (0,)):
+            B, Bs = (hk.tile_operand(b), hk.tile_scales(bsc, K)) if lb else (b, bsc)
+            C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(a, B, asc, Bs, C, layout_b=lb)
+            torch.cuda.synchronize()
+            assert o.rel_err(C.cpu().numpy(), ref.cpu().numpy()) <= TOL_TIGHT, (kernel, lb)
+    finally:
+        hk.tk_kernel.set_kernel(prev)
 
 
 # ------------------------------------------------------------------ mid-M kernel
