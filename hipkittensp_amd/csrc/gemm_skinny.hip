@@ -25,6 +25,9 @@
 // The reference has no kernel for this shape (its GEMMs need M, N multiples of the 256 tile,
 // analysis/bf16_gemm/mi325x/kernel_8192.cpp:24-32).  Algorithmic bytes per launch:
 // 0.75*K*(M+N) + (K/32)*(M+N) + 2*M*N.
+#include <map>
+#include <mutex>
+#include <utility>
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -48,7 +51,7 @@ template <int FA, int FB, typename Out, int AR, int NW, int BR>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                               typename Out::type* __restrict__ C, int M, int N, int K, int layout_b,
-                                                              const Epilogue ep) {
+                                                              const Epilogue ep, int nsplit, float* ws_part, int* ws_cnt) {
   static_assert(BR == 32 || BR == 16, "rows of B per workgroup");
   constexpr int kBBuf = BR * 384, kABuf = AR * 384, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then 2 x 1 KB of scales
   constexpr int kBuf = kScOff + 2048;
@@ -60,9 +63,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, r32 = lane & 31;
   const int nkt = K / 128, sbytes = K / 32, rowbytes = K / 4 * 3;
-  const int n0 = blockIdx.x * BR;
+  // nsplit > 1: the K range is split between nsplit workgroups per BR rows of B (workgroup = split * ntiles + tile)
+  const int ntiles = gridDim.x / nsplit;
+  const int tile = blockIdx.x % ntiles, split = blockIdx.x / ntiles;
+  const int n0 = tile * BR;
   const int nrows = min(BR, N - n0);
-  const int rt = BR == 32 ? blockIdx.x : blockIdx.x >> 1, half = BR == 32 ? 0 : blockIdx.x & 1;  // tile-major B: row-tile, and which 16 rows of it
+  const int rt = BR == 32 ? tile : tile >> 1, half = BR == 32 ? 0 : tile & 1;  // tile-major B: row-tile, and which 16 rows of it
 
   // rows that do not exist (n >= N, m >= M) lie past the end of the resource and read as zeros
   const __amdgpu_buffer_rsrc_t rB = layout_b ? make_rsrc(B + (size_t)rt * 32 * rowbytes, (uint32_t)32 * rowbytes)
@@ -108,9 +114,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
       a_rd[u][c] = kBBuf + ra * 384 + (p ^ ((ra >> 1) & 7)) * 16;
     }
 
-  // chunks of this wave: wave, wave + NW, ...
-  const int nchunks = nkt / 4;
-  const int mine = wave < nchunks ? (nchunks - wave + NW - 1) / NW : 0;
+  // chunks of this workgroup: [c0, c1); of this wave: c0 + wave, c0 + wave + NW, ...
+  const int nchunks = nkt / 4, cps = (nchunks + nsplit - 1) / nsplit;
+  const int c0 = split * cps, c1 = min(nchunks, c0 + cps);
+  const int mine = c0 + wave < c1 ? (c1 - c0 - wave + NW - 1) / NW : 0;
 
   auto issue_chunk = [&](int chunk) __attribute__((always_inline)) {
     const int sos = __builtin_amdgcn_readfirstlane(chunk * 16);
@@ -130,7 +137,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   for (int e = 0; e < 16; e++) acc[e] = 0.f;
 
   if (mine > 0) {
-    issue_chunk(wave);
+    issue_chunk(c0 + wave);
     for (int j = 0; j < mine; j++) {
       wait_all_loads();
       const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + rb * 16);
@@ -146,7 +153,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
       // the buffer is about to be refilled: its reads must have left LDS
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
-      if (j + 1 < mine) issue_chunk(wave + (j + 1) * NW);
+      if (j + 1 < mine) issue_chunk(c0 + wave + (j + 1) * NW);
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int sb = (uint32_t)sc_b[u] >> (16 * h), sa = (uint32_t)sc_a[u] >> (16 * h);
@@ -168,6 +175,39 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   for (int e = 0; e < 16; e++) part[(wave * 16 + e) * 64 + lane] = acc[e];
   __syncthreads();
   const bool has_ep = epilogue_any(ep);
+  if (nsplit > 1) {
+    // K split between workgroups: every workgroup leaves its partial tile in the workspace; the one that arrives last
+    // (a counter per tile) adds them up in split order, so the result does not depend on who that is.  The other
+    // workgroups may run on XCDs with L2s of their own: partial tiles and counter are written and read with
+    // device-scope atomic accesses, which go past those caches, instead of device-scope fences, which write back and
+    // invalidate a whole L2 per wave (measured: 0.2 us per workgroup, one after the other).
+    float* mine_ws = ws_part + ((size_t)tile * nsplit + split) * 1024;
+    for (int idx = tid; idx < 1024; idx += NW * 64) {
+      const int e = idx >> 6, l = idx & 63;
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; w++) t += part[(w * 16 + e) * 64 + l];
+      __hip_atomic_store(mine_ws + idx, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    wait_all_loads();  // stores count there too: the partial tile has arrived before the counter moves
+    __syncthreads();
+    int* flag = reinterpret_cast<int*>(smem + NW * 16 * 64 * 4);  // behind the partial tiles
+    if (tid == 0) *flag = __hip_atomic_fetch_add(ws_cnt + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1;
+    __syncthreads();
+    if (!*flag) return;
+    const float* all = ws_part + (size_t)tile * nsplit * 1024;
+    for (int idx = tid; idx < 1024; idx += NW * 64) {
+      const int e = idx >> 6, l = idx & 63;
+      float t = 0.f;
+      for (int q = 0; q < nsplit; q++) t += __hip_atomic_load(all + q * 1024 + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int m = l & 31;
+      const int nl = 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
+      const long nn = (long)n0 + nl;
+      if (m < M && nl < BR && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, t, m, nn) : t);
+    }
+    if (tid == 0) __hip_atomic_store(ws_cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    return;
+  }
   for (int idx = tid; idx < 1024; idx += NW * 64) {
     const int e = idx >> 6, l = idx & 63;
     float s = 0.f;
@@ -185,16 +225,78 @@ bool gemm_skinny_supports(const GemmArgs& g) {
   return g.layout_a == 0 && g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
 }
 
-// Geometry.  Few rows of B (N / 32 workgroups would leave half of the CUs idle): 16 rows per workgroup.  Many (N / 32
-// is several times the CU count): half as many waves per workgroup, so that two workgroups share a CU and one's first
-// loads run under the other's stream (a workgroup with a short K range is mostly load latency).
+// Workspace of the K split: 4 KB of partial tile per (tile, split) and a counter per tile that is zero between
+// launches.  One per stream, allocated at first use and kept: launches on one stream are ordered, so they can share it;
+// launches on different streams get different ones.  (Two graphs captured on one stream and replayed at the same time
+// on different streams would share theirs: replay them on one stream, or switch the split off with geometry 7 - 9.)
+// No allocation is possible while the stream is being captured: a capture without a workspace runs unsplit.
+namespace {
+constexpr int kWsSlots = 2048, kWsTiles = 1024;  // (tile, split) pairs and tiles a workspace holds
+struct SplitWs {
+  float* part = nullptr;
+  int* cnt = nullptr;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, SplitWs> g_ws;
+
+SplitWs split_workspace(hipStream_t s) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return {};
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_ws.find({dev, s});
+  if (it != g_ws.end()) return it->second;
+  if (g_ws.size() >= 64) return {};  // a process with this many streams runs unsplit on the later ones
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return {};
+  }
+  SplitWs w;
+  if (hipMalloc((void**)&w.part, (size_t)kWsSlots * 4096) != hipSuccess) { (void)hipGetLastError(); return {}; }
+  if (hipMalloc((void**)&w.cnt, kWsTiles * sizeof(int)) != hipSuccess || hipMemset(w.cnt, 0, kWsTiles * sizeof(int)) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(w.part);
+    return {};
+  }
+  g_ws[{dev, s}] = w;
+  return w;
+}
+}  // namespace
+
+// Geometry.  Few rows of B (N / 32 workgroups would leave CUs idle): a workgroup takes 16 rows of B, and the K range
+// is split between 2, 4 or 8 workgroups while that still fits the CUs and leaves every wave kMinChunks chunks.  Many
+// (N / 32 is several times the CU count): half as many waves per workgroup, so that two workgroups share a CU and
+// one's first loads run under the other's stream (a workgroup with a short K range is mostly load latency).
+// skinny_geometry: 1 - 3 fix the workgroup shape without a split; 4 + 3 * b + log2(split) - 1 (b = 0: 32 rows of B,
+// b = 1: 16 rows) fixes both.
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   typedef typename Out::type T;
   const unsigned wgs32 = (g.N + 31) / 32;
+  const int nchunks = g.K / 512, nw = g.M <= 16 ? 8 : 6;
+  int geo, want = 1;
+  if (g.skinny_geometry >= 4) {
+    geo = 1 + (g.skinny_geometry - 4) / 3;
+    want = 2 << ((g.skinny_geometry - 4) % 3);
+  } else if (g.skinny_geometry) {
+    geo = g.skinny_geometry;
+  } else {
+    geo = wgs32 <= 128 ? 2 : wgs32 >= 512 ? 3 : 1;
+    constexpr int kMinChunks = 3;  // measured: below this the 2.5 us of the second phase outweigh the wider stream
+    const unsigned tiles = geo == 2 ? (g.N + 15) / 16 : wgs32;
+    if (geo != 3)
+      while (want < 8 && tiles * want * 2 <= 256 && nchunks / (want * 2) >= kMinChunks * nw) want *= 2;
+  }
+  int nsplit = 1;
+  SplitWs ws;
+  const unsigned tiles = geo == 2 ? (g.N + 15) / 16 : wgs32;
+  if (want > 1 && tiles <= (unsigned)kWsTiles && tiles * want <= (unsigned)kWsSlots) {
+    ws = split_workspace(s);
+    if (ws.part) nsplit = want;
+  }
 #define MXFP6_SK(AR, NW, BR) \
-  gemm_skinny_kernel<FA, FB, Out, AR, NW, BR><<<(g.N + BR - 1) / BR, NW * 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, g.layout_b, g.ep)
-  const int geo = g.skinny_geometry ? g.skinny_geometry : wgs32 <= 128 ? 2 : wgs32 >= 512 ? 3 : 1;
+  gemm_skinny_kernel<FA, FB, Out, AR, NW, BR><<<(g.N + BR - 1) / BR * nsplit, NW * 64, 0, s>>>( \
+      g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, g.layout_b, g.ep, nsplit, ws.part, ws.cnt)
   if (g.M <= 16) {
     if (geo == 2) MXFP6_SK(16, 8, 16); else if (geo == 3) MXFP6_SK(16, 4, 32); else MXFP6_SK(16, 8, 32);
   } else {

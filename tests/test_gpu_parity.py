@@ -170,9 +170,14 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     # partial sums differs, so they agree to fp32 rounding, and each is held to the oracle
     for kern in (hk.tk_kernel.KERNEL_SKINNY_32, hk.tk_kernel.KERNEL_SKINNY_16, hk.tk_kernel.KERNEL_SKINNY_HALF):
         check(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kern), ref, fa, fb, ap, asc, bp, bsc)
+    # the K range split between 2 / 4 / 8 workgroups per tile of C (more splits than chunks leaves some without work);
+    # twice each: the tile counters must be back at zero after a launch
+    for kern in hk.tk_kernel.KERNEL_SKINNY_32_SPLIT + hk.tk_kernel.KERNEL_SKINNY_16_SPLIT:
+        for _ in range(2):
+            check(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kern), ref, fa, fb, ap, asc, bp, bsc)
 
 
-@pytest.mark.parametrize("kernel", [7, 8, 9])
+@pytest.mark.parametrize("kernel", [7, 8, 9, 11, 13])
 @pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 2080, 1536), (5, 17408, 1024)])
 def test_skinny_geometries_tile_major_weights(hk, kernel, M, N, K):
     """Each geometry with tile-major weights and scales (16 rows per workgroup read half of every 3 KB tile) against the
@@ -193,6 +198,59 @@ def test_skinny_geometries_tile_major_weights(hk, kernel, M, N, K):
             assert o.rel_err(C.cpu().numpy(), ref.cpu().numpy()) <= TOL_TIGHT, (kernel, lb)
     finally:
         hk.tk_kernel.set_kernel(prev)
+
+
+def test_skinny_k_split_chosen_by_shape_streams_and_capture(hk):
+    """Few rows of B and a long K: the automatic choice splits K between workgroups (partial tiles in a per-stream
+    workspace, summed by the last workgroup to arrive).  Against the generic kernel; tile-major weights; fused epilogue;
+    two streams at once, each with its own workspace; under stream capture (a workspace exists or the launch runs
+    unsplit: the same sums up to fp32 rounding either way)."""
+    M, N, K = 16, 1024, 28672
+    g = torch.Generator(device="cuda"); g.manual_seed(5)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2)
+    bias = torch.randn(N, device="cuda", generator=g)
+    bt, bst = hk.tile_operand(b), hk.tile_scales(bsc, K)
+    ref = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    prev = hk.tk_kernel.set_kernel(1)
+    try:
+        hk.dispatch_micro(a, b, asc, bsc, ref)
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+    torch.cuda.synchronize()
+    refn = ref.cpu().numpy()
+    for rep in range(3):
+        for B, Bs, lb in ((b, bsc, 0), (bt, bst, 1)):
+            C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(a, B, asc, Bs, C, layout_b=lb)
+            assert o.rel_err(C.cpu().numpy(), refn) <= TOL_TIGHT, (rep, lb)
+    C = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    hk.dispatch_micro(a, bt, asc, bst, C, layout_b=1, bias=bias, activation="relu")
+    assert torch.allclose(C, torch.relu(ref + bias[None, :]), rtol=2e-6, atol=1e-5)
+    # two streams, launches interleaved
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda") for _ in range(6)] for _ in streams]
+    torch.cuda.synchronize()
+    for i in range(6):
+        for st, out in zip(streams, outs):
+            with torch.cuda.stream(st):
+                hk.dispatch_micro(a, bt, asc, bst, out[i], layout_b=1)
+    torch.cuda.synchronize()
+    for out in outs:
+        for C in out:
+            assert o.rel_err(C.cpu().numpy(), refn) <= TOL_TIGHT
+    # capture and replays
+    Cg = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hk.dispatch_micro(a, bt, asc, bst, Cg, layout_b=1)
+    for rep in range(3):
+        Cg.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert o.rel_err(Cg.cpu().numpy(), refn) <= TOL_TIGHT, f"replay {rep}"
+        hk.dispatch_micro(a, bt, asc, bst, torch.empty_like(Cg), layout_b=1)
+        torch.cuda.synchronize()
 
 
 # ------------------------------------------------------------------ mid-M kernel
