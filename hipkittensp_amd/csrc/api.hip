@@ -135,7 +135,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 4) {
     if (!mxfp6::gemm_mid_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_mid(g, s);
-  } else if (mxfp6::gemm_skinny_supports(g)) {
+  } else if (mxfp6::gemm_skinny_preferred(g)) {
     e = mxfp6::launch_gemm_skinny(g, s);
   } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
     e = mxfp6::launch_gemm_mid(g, s);
@@ -195,7 +195,7 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
   const int force = g_force.load(std::memory_order_relaxed);
   const bool tiled = K > 0 && mxfp6::gemm_tiled_supports(g) &&
                      (force == 2 || force == 5 || force == 6 ||
-                      (force == 0 && !mxfp6::gemm_skinny_supports(g) && !mxfp6::gemm_mid_preferred(g)));
+                      (force == 0 && !mxfp6::gemm_skinny_preferred(g) && !mxfp6::gemm_mid_preferred(g)));
   if (tiled) {
     g.ep = ep, g.C_scale = (uint8_t*)C_scale, g.fmt_c = fmt_c;
     g.tile_rows = force == 5 ? 128 : force == 6 ? 256 : 0;

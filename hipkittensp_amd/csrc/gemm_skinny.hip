@@ -1,4 +1,4 @@
-// Skinny-M (decode-shaped) MXFP6 GEMM for gfx950: M <= 32, bound by HBM.
+// Skinny-M (decode-shaped) MXFP6 GEMM for gfx950: M <= 128, bound by HBM.
 //
 // Every byte of B (weights) is read from HBM once.  One workgroup owns 32 consecutive rows of B (32 output
 // columns) and splits K over its waves in chunks of four K-tiles (4 x 128 elements = 384 bytes per row = three
@@ -16,7 +16,9 @@
 // which spreads the 16 rows of a ds_read_b128 phase over all 64 banks (rows r and r+16 share banks and are never
 // in the same phase, analysis/paper_experiments/phases/ds_read_b128/phase_results.txt:4-7); the permutation is
 // applied by choosing which global bytes each lane fetches, as in the tiled kernel.  A tile-major B arrives as
-// four 3 KB tiles in the tiled kernel's image.  A's rows (M <= 32) are staged like a row-major B, from L2.  The
+// four 3 KB tiles in the tiled kernel's image.  A's rows are staged like a row-major B, from L2: 16 or 32 of them
+// feed one 32x32 accumulator tile per wave; 64 feed two and 128 four (against the same fragments of B), with four
+// waves per workgroup, and 128 in chunks of two K-tiles (192-byte rows), so that the buffers still fit LDS.  The
 // E8M0 bytes of a chunk are 16 bytes per row: one more direct load each for B and A (no load of this kernel has a
 // register destination, so nothing can read a register before its load has landed).  All loads are issued from
 // inline assembly and waited for with vmcnt by hand.  The partial 32x32 tiles of the waves are summed
@@ -45,19 +47,26 @@ __device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt
 
 }  // namespace
 
-// AR = rows of A staged (16 or 32); NW = waves per workgroup; BR = rows of B per workgroup (32, or 16 so that a narrow
-// N still gives every CU a workgroup: the MFMA's other 16 rows then mirror the first and their outputs are dropped)
+// AR = rows of A staged (16, 32 or 64: one or two 32-row accumulator tiles per wave); NW = waves per workgroup;
+// BR = rows of B per workgroup (32, or 16 so that a narrow N still gives every CU a workgroup: the MFMA's other 16
+// rows then mirror the first and their outputs are dropped)
 template <int FA, int FB, typename Out, int AR, int NW, int BR>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                               typename Out::type* __restrict__ C, int M, int N, int K, int layout_b,
                                                               const Epilogue ep, int nsplit, float* ws_part, int* ws_cnt) {
   static_assert(BR == 32 || BR == 16, "rows of B per workgroup");
-  constexpr int kBBuf = BR * 384, kABuf = AR * 384, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then 2 x 1 KB of scales
-  constexpr int kBuf = kScOff + 2048;
-  constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024;                    // direct loads per chunk: 12 and 6 or 12
+  static_assert(AR == 16 || AR == 32 || AR == 64 || AR == 128, "rows of A");
+  constexpr int TA = AR > 32 ? AR / 32 : 1;   // accumulator tiles per wave
+  constexpr int KT = AR == 128 ? 2 : 4;       // K-tiles per chunk (128 rows of A: half chunks, so that four waves' buffers fit)
+  constexpr int kRow = 96 * KT, kPieces = 6 * KT;  // bytes and 16-byte pieces of a row in a chunk
+  constexpr int kBBuf = BR * kRow, kABuf = AR * kRow, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then the scales:
+  constexpr int kASc = AR <= 64 ? 1024 : AR * 16;                              // 1 KB for B, 16 bytes per row of A
+  constexpr int kBuf = kScOff + 1024 + kASc;
+  constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024, NAS = kASc / 1024;  // direct loads per chunk: 12 or 6; 6, 12 or 24; 1 or 2
+  static_assert(kBBuf % 1024 == 0 && kABuf % 1024 == 0, "whole direct loads");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kBuf];
-  static_assert(NW * kBuf <= 163840 && NW * kBuf >= NW * 16 * 64 * 4, "LDS budget (the buffers double as the reduction buffer)");
+  static_assert(NW * kBuf <= 163840 && NW * kBuf >= NW * TA * 16 * 64 * 4 + 64, "LDS budget (the buffers double as the reduction buffer)");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -81,101 +90,119 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * sbytes);
 
   // direct-load address maps: load i fills LDS bytes [i*1024, i*1024 + 1024) of the buffer; slot o = i*64 + lane holds
-  // piece (o % 24) ^ ((row >> 1) & 7) of row o / 24.  Tile-major B: four consecutive 3 KB tiles, copied as they are
-  // (BR = 16: the 1536 bytes that this workgroup's 16 rows have in each of them).
+  // piece swz(o % kPieces, row) of row o / kPieces, where swz permutes the pieces of a row inside groups of eight
+  // (384-byte rows) or four (192-byte rows) so that the 16 rows of a ds_read_b128 phase fall into different banks.
+  // Tile-major B: KT consecutive 3 KB tiles, copied as they are (BR = 16: the 1536 bytes that this workgroup's 16 rows
+  // have in each of them).
+  auto swz = [](int p, int r) __attribute__((always_inline)) { return KT == 4 ? p ^ ((r >> 1) & 7) : p ^ ((r >> 2) & 3); };
   int voff_b[NBL], voff_a[NAL];
 #pragma unroll
   for (int i = 0; i < NBL; i++) {
-    const int o = i * 64 + lane, r = o / 24, p = (o - r * 24) ^ ((r >> 1) & 7);
+    const int o = i * 64 + lane, r = o / kPieces, p = swz(o - r * kPieces, r);
     constexpr int kPer = BR * 6;  // 16-byte pieces per K-tile of this workgroup's rows
     voff_b[i] = layout_b ? (o / kPer) * 3072 + half * 1536 + (o % kPer) * 16 : r * rowbytes + p * 16;
   }
 #pragma unroll
   for (int i = 0; i < NAL; i++) {
-    const int o = i * 64 + lane, r = o / 24, p = (o - r * 24) ^ ((r >> 1) & 7);
+    const int o = i * 64 + lane, r = o / kPieces, p = swz(o - r * kPieces, r);
     voff_a[i] = r * rowbytes + p * 16;
   }
-  // scale loads: lane l fetches the 16 bytes of row l % 32 (both halves of the wave fetch the same rows)
+  // scale loads: lane l fetches the 16 bytes (four K-tiles) of row l % 32 (both halves of the wave fetch the same rows;
+  // 64 or more rows of A: of row l, l + 64)
   const int ra = AR == 16 ? (r32 & 15) : r32;  // AR = 16: lanes 16-31 mirror rows 0-15 (their outputs are never stored)
   const int rb = BR == 16 ? (r32 & 15) : r32;  // BR = 16: likewise for B
   const int voff_bs = layout_b ? (half * 16 + rb) * 16 : rb * sbytes;
-  const int voff_as = r32 * sbytes;
+  const int voff_as = (AR >= 64 ? lane : r32) * sbytes;
 
   const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kBuf;
   const uint8_t* bufp = smem + wave * kBuf;
   // LDS read offsets of this lane: K-tile u, piece c of its half (pieces 3h .. 3h+2 of the K-tile)
-  int b_rd[4][3], a_rd[4][3];
+  int b_rd[KT][3], a_rd[KT][3];
 #pragma unroll
-  for (int u = 0; u < 4; u++)
+  for (int u = 0; u < KT; u++)
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const int p = u * 6 + 3 * h + c;
-      b_rd[u][c] = layout_b ? u * (BR * 96) + rb * 96 + ((3 * h + c) ^ ((rb >> 3) & 1)) * 16 : rb * 384 + (p ^ ((rb >> 1) & 7)) * 16;
-      a_rd[u][c] = kBBuf + ra * 384 + (p ^ ((ra >> 1) & 7)) * 16;
+      b_rd[u][c] = layout_b ? u * (BR * 96) + rb * 96 + ((3 * h + c) ^ ((rb >> 3) & 1)) * 16 : rb * kRow + swz(p, rb) * 16;
+      a_rd[u][c] = kBBuf + ra * kRow + swz(p, ra) * 16;
     }
 
   // chunks of this workgroup: [c0, c1); of this wave: c0 + wave, c0 + wave + NW, ...
-  const int nchunks = nkt / 4, cps = (nchunks + nsplit - 1) / nsplit;
+  const int nchunks = nkt / KT, cps = (nchunks + nsplit - 1) / nsplit;
   const int c0 = split * cps, c1 = min(nchunks, c0 + cps);
   const int mine = c0 + wave < c1 ? (c1 - c0 - wave + NW - 1) / NW : 0;
 
   auto issue_chunk = [&](int chunk) __attribute__((always_inline)) {
-    const int sos = __builtin_amdgcn_readfirstlane(chunk * 16);
-    const int sosb = __builtin_amdgcn_readfirstlane(layout_b ? chunk * 512 : chunk * 16);
+    const int sg = KT == 4 ? chunk : chunk >> 1;  // the scales come in groups of four K-tiles
+    const int sos = __builtin_amdgcn_readfirstlane(sg * 16);
+    const int sosb = __builtin_amdgcn_readfirstlane(layout_b ? sg * 512 : sg * 16);
     dma16_sk(rBs, buf + kScOff, voff_bs, sosb);
-    dma16_sk(rAs, buf + kScOff + 1024, voff_as, sos);
-    const int so = __builtin_amdgcn_readfirstlane(chunk * 384);
-    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * (4 * 3072) : chunk * 384);
+#pragma unroll
+    for (int i = 0; i < NAS; i++) dma16_sk(rAs, buf + kScOff + 1024 + i * 1024, voff_as + i * 64 * sbytes, sos);
+    const int so = __builtin_amdgcn_readfirstlane(chunk * kRow);
+    const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * (KT * 3072) : chunk * kRow);
 #pragma unroll
     for (int i = 0; i < NBL; i++) dma16_sk(rB, buf + i * 1024, voff_b[i], sob);
 #pragma unroll
     for (int i = 0; i < NAL; i++) dma16_sk(rA, buf + kBBuf + i * 1024, voff_a[i], so);
   };
 
-  v16f acc;
+  v16f acc[TA];
 #pragma unroll
-  for (int e = 0; e < 16; e++) acc[e] = 0.f;
+  for (int t = 0; t < TA; t++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
 
   if (mine > 0) {
     issue_chunk(c0 + wave);
     for (int j = 0; j < mine; j++) {
       wait_all_loads();
       const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + rb * 16);
-      const v4i sc_a = *reinterpret_cast<const v4i*>(bufp + kScOff + 1024 + ra * 16);
-      v4i fb[4][3], fa[4][3];
+      v4i sc_a[TA];
+      v4i fb[KT][3], fa[TA][KT][3];
+      const bool odd = KT == 2 && ((c0 + wave + j * NW) & 1);  // half chunks: which two of the four scale bytes
 #pragma unroll
-      for (int u = 0; u < 4; u++)
+      for (int t = 0; t < TA; t++) sc_a[t] = *reinterpret_cast<const v4i*>(bufp + kScOff + 1024 + (t * 32 + ra) * 16);
+#pragma unroll
+      for (int u = 0; u < KT; u++)
 #pragma unroll
         for (int c = 0; c < 3; c++) {
           fb[u][c] = *reinterpret_cast<const v4i*>(bufp + b_rd[u][c]);
-          fa[u][c] = *reinterpret_cast<const v4i*>(bufp + a_rd[u][c]);
+#pragma unroll
+          for (int t = 0; t < TA; t++) fa[t][u][c] = *reinterpret_cast<const v4i*>(bufp + a_rd[u][c] + t * (32 * kRow));
         }
       // the buffer is about to be refilled: its reads must have left LDS
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
       if (j + 1 < mine) issue_chunk(c0 + wave + (j + 1) * NW);
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        const int sb = (uint32_t)sc_b[u] >> (16 * h), sa = (uint32_t)sc_a[u] >> (16 * h);
+      for (int u = 0; u < KT; u++) {
+        const int sb = (uint32_t)(KT == 4 ? sc_b[u] : odd ? sc_b[u + 2] : sc_b[u]) >> (16 * h);
         const v8i b0 = __builtin_shufflevector(fb[u][0], fb[u][1], 0, 1, 2, 3, 4, 5, -1, -1);
         const v8i b1 = __builtin_shufflevector(fb[u][1], fb[u][2], 2, 3, 4, 5, 6, 7, -1, -1);
-        const v8i a0 = __builtin_shufflevector(fa[u][0], fa[u][1], 0, 1, 2, 3, 4, 5, -1, -1);
-        const v8i a1 = __builtin_shufflevector(fa[u][1], fa[u][2], 2, 3, 4, 5, 6, 7, -1, -1);
-        acc = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc, sb, sa);
-        acc = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc, sb, sa);
+#pragma unroll
+        for (int t = 0; t < TA; t++) {
+          const int sa = (uint32_t)(KT == 4 ? sc_a[t][u] : odd ? sc_a[t][u + 2] : sc_a[t][u]) >> (16 * h);
+          const v8i a0 = __builtin_shufflevector(fa[t][u][0], fa[t][u][1], 0, 1, 2, 3, 4, 5, -1, -1);
+          const v8i a1 = __builtin_shufflevector(fa[t][u][1], fa[t][u][2], 2, 3, 4, 5, 6, 7, -1, -1);
+          acc[t] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[t], sb, sa);
+          acc[t] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[t], sb, sa);
+        }
       }
     }
   }
 
-  // sum the K-slices: register e of lane l is C[m = l % 32][n = 8*(e/4) + 4*(l/32) + e%4].
+  // sum the K-slices: register e of lane l is C[m = 32 t + l % 32][n = 8*(e/4) + 4*(l/32) + e%4] of accumulator tile t.
   // The buffers double as the reduction buffer once every wave has drained its loads.
   __syncthreads();
   float* part = reinterpret_cast<float*>(smem);
 #pragma unroll
-  for (int e = 0; e < 16; e++) part[(wave * 16 + e) * 64 + lane] = acc[e];
+  for (int t = 0; t < TA; t++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) part[((wave * TA + t) * 16 + e) * 64 + lane] = acc[t][e];
   __syncthreads();
   const bool has_ep = epilogue_any(ep);
-  if (nsplit > 1) {
+  if (TA == 1 && nsplit > 1) {
     // K split between workgroups: every workgroup leaves its partial tile in the workspace; the one that arrives last
     // (a counter per tile) adds them up in split order, so the result does not depend on who that is.  The other
     // workgroups may run on XCDs with L2s of their own: partial tiles and counter are written and read with
@@ -208,12 +235,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     if (tid == 0) __hip_atomic_store(ws_cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     return;
   }
-  for (int idx = tid; idx < 1024; idx += NW * 64) {
-    const int e = idx >> 6, l = idx & 63;
+  for (int idx = tid; idx < TA * 1024; idx += NW * 64) {
+    const int t = idx >> 10, e = (idx >> 6) & 15, l = idx & 63;
     float s = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; w++) s += part[(w * 16 + e) * 64 + l];
-    const int m = l & 31;
+    for (int w = 0; w < NW; w++) s += part[((w * TA + t) * 16 + e) * 64 + l];
+    const int m = t * 32 + (l & 31);
     const int nl = 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
     const long nn = (long)n0 + nl;
     if (m < M && nl < BR && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, s, m, nn) : s);
@@ -222,7 +249,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 
 bool gemm_skinny_supports(const GemmArgs& g) {
   // K % 512: chunks of four K-tiles are whole (three 128-byte lines per row, 16 scale bytes per row)
-  return g.layout_a == 0 && g.M >= 1 && g.M <= 32 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)32 * (g.K / 4 * 3) < (1L << 31);
+  return g.layout_a == 0 && g.M >= 1 && g.M <= 128 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31);
+}
+
+// Automatic choice.  Up to 64 rows of A this kernel is the fastest everywhere (measured against the mid-M kernel: 18 us
+// against 22 at 64 x 8192 x 8192, 48 against 66 at K = 28672, level at N = 28672).  With 65 - 128 rows a wave's chunk is
+// mostly A (24 KB of 30), so few bytes of B are in flight per CU: it wins by 10 - 15 % while one round of workgroups covers
+// N and loses by 25 % beyond, where the mid-M kernel's 64 rows of B per workgroup halve the traffic of A.
+bool gemm_skinny_preferred(const GemmArgs& g) {
+  if (!gemm_skinny_supports(g)) return false;
+  return g.M <= 64 || (g.N + 31) / 32 <= 256 || !gemm_mid_supports(g);
 }
 
 // Workspace of the K split: 4 KB of partial tile per (tile, split) and a counter per tile that is zero between
@@ -275,7 +311,10 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const unsigned wgs32 = (g.N + 31) / 32;
   const int nchunks = g.K / 512, nw = g.M <= 16 ? 8 : 6;
   int geo, want = 1;
-  if (g.skinny_geometry >= 4) {
+  if (g.M > 32) {
+    // 33 - 128 rows of A: two or four accumulator tiles per wave, four waves or two (two workgroups per CU), no K split
+    geo = g.skinny_geometry == 3 || (g.skinny_geometry == 0 && wgs32 > 256) ? 3 : 1;
+  } else if (g.skinny_geometry >= 4) {
     geo = 1 + (g.skinny_geometry - 4) / 3;
     want = 2 << ((g.skinny_geometry - 4) % 3);
   } else if (g.skinny_geometry) {
@@ -297,7 +336,11 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
 #define MXFP6_SK(AR, NW, BR) \
   gemm_skinny_kernel<FA, FB, Out, AR, NW, BR><<<(g.N + BR - 1) / BR * nsplit, NW * 64, 0, s>>>( \
       g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, g.layout_b, g.ep, nsplit, ws.part, ws.cnt)
-  if (g.M <= 16) {
+  if (g.M > 64) {
+    if (geo == 3) MXFP6_SK(128, 2, 32); else MXFP6_SK(128, 4, 32);
+  } else if (g.M > 32) {
+    if (geo == 3) MXFP6_SK(64, 2, 32); else MXFP6_SK(64, 4, 32);
+  } else if (g.M <= 16) {
     if (geo == 2) MXFP6_SK(16, 8, 16); else if (geo == 3) MXFP6_SK(16, 4, 32); else MXFP6_SK(16, 8, 32);
   } else {
     if (geo == 2) MXFP6_SK(32, 6, 16); else if (geo == 3) MXFP6_SK(32, 3, 32); else MXFP6_SK(32, 6, 32);

@@ -29,6 +29,7 @@ double tiled_estimate_us(const GemmArgs& g, int rows);  // estimated time of the
 double mid_estimate_us(const GemmArgs& g);
 hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
+bool gemm_skinny_preferred(const GemmArgs& g);  // over the mid-M kernel, by shape
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 hipError_t launch_quantize(const void* X, int x_bf16, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);
 hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);

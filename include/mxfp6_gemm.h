@@ -71,7 +71,7 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
 /*
  * Kernel selection override for measurement and tests: 0 = automatic (default), 1 = generic
  * one-wave-per-tile kernel, 2 = LDS-tiled MFMA kernel (needs N % 8 == 0, K % 128 == 0; 128 or 256 rows of A
- * per output tile, whichever fills the GPU better), 3 = skinny-M streaming kernel (needs M <= 32,
+ * per output tile, whichever fills the GPU better), 3 = skinny-M streaming kernel (needs M <= 128,
  * K % 512 == 0; its workgroup geometry follows N), 4 = mid-M kernel (needs 32 < M <= 512, K % 1024 == 0,
  * row-major A), 5 / 6 = the tiled kernel with 128- / 256-row tiles, 7 / 8 / 9 = the skinny kernel with 32 rows of B
  * per workgroup / 16 rows / 32 rows and half the waves (none of them splitting K), 10 / 11 / 12 = 32 rows of B with

@@ -144,8 +144,9 @@ def test_forced_kernels_reject_shapes_they_cannot_take(hk):
     ap, asc, bp, bsc = operands(64, 64, 64, 2, 2, seed=1)
     with pytest.raises(RuntimeError, match="bad shape"):
         gemm(hk, ap, bp, asc, bsc, kernel=2)
+    ap, asc, bp, bsc = operands(129, 64, 512, 2, 2, seed=1)
     with pytest.raises(RuntimeError, match="bad shape"):
-        gemm(hk, ap, bp, asc, bsc, kernel=3)          # M > 32
+        gemm(hk, ap, bp, asc, bsc, kernel=3)          # M > 128
     ap, asc, bp, bsc = operands(16, 64, 384, 2, 2, seed=1)
     with pytest.raises(RuntimeError, match="bad shape"):
         gemm(hk, ap, bp, asc, bsc, kernel=3)          # K % 512
@@ -157,7 +158,9 @@ def test_forced_kernels_reject_shapes_they_cannot_take(hk):
 
 
 # ------------------------------------------------------------------ skinny kernel
-@pytest.mark.parametrize("M,N,K", [(16, 64, 512), (1, 32, 1024), (7, 100, 2048), (16, 512, 3584), (32, 96, 1536), (13, 33, 512 * 9), (17, 31, 512 * 13), (16, 1000, 512 * 20)])
+@pytest.mark.parametrize("M,N,K", [(16, 64, 512), (1, 32, 1024), (7, 100, 2048), (16, 512, 3584), (32, 96, 1536), (13, 33, 512 * 9), (17, 31, 512 * 13), (16, 1000, 512 * 20),
+                                   (33, 40, 1024), (64, 96, 512 * 5), (48, 1000, 2048), (50, 31, 512 * 11),    # 33 - 64 rows of A: two accumulator tiles
+                                   (65, 40, 1024), (128, 96, 512 * 5), (100, 1000, 2048), (96, 31, 512 * 11)])  # 65 - 128: four, half chunks
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
 def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + 2 * N + K, kind_b="weights")
@@ -178,7 +181,7 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
 
 
 @pytest.mark.parametrize("kernel", [7, 8, 9, 11, 13])
-@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 2080, 1536), (5, 17408, 1024)])
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 2080, 1536), (5, 17408, 1024), (64, 4096, 2048), (100, 2080, 1536), (128, 17408, 1024)])
 def test_skinny_geometries_tile_major_weights(hk, kernel, M, N, K):
     """Each geometry with tile-major weights and scales (16 rows per workgroup read half of every 3 KB tile) against the
     generic kernel on the row-major operands; ragged N only row-major."""
@@ -268,9 +271,13 @@ def test_mid_kernel_vs_oracle(hk, M, N, K, fa, fb):
 
 
 def test_mid_kernel_is_chosen_and_rejects_other_shapes(hk):
-    # few 256x256 tiles, K in whole B slots: the automatic choice is the mid kernel and agrees with the forced one bit for bit
-    ap, asc, bp, bsc = operands(96, 288, 2048, 2, 2, seed=9, kind_b="weights")
+    # more than 128 rows of A, few 256x256 tiles, K in whole B slots: the automatic choice is the mid kernel and agrees with
+    # the forced one bit for bit; up to 128 rows (and N within one round of workgroups) it is the skinny kernel
+    ap, asc, bp, bsc = operands(160, 288, 2048, 2, 2, seed=9, kind_b="weights")
     assert np.array_equal(gemm(hk, ap, bp, asc, bsc, kernel=0), gemm(hk, ap, bp, asc, bsc, kernel=4))
+    check(gemm(hk, ap, bp, asc, bsc, kernel=4), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)
+    ap, asc, bp, bsc = operands(96, 288, 2048, 2, 2, seed=9, kind_b="weights")
+    assert np.array_equal(gemm(hk, ap, bp, asc, bsc, kernel=0), gemm(hk, ap, bp, asc, bsc, kernel=3))
     check(gemm(hk, ap, bp, asc, bsc, kernel=4), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)
     for M, N, K in ((32, 64, 1024), (520, 64, 1024), (64, 64, 1536)):   # M <= 32, M > 512, K % 1024
         ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=5)
