@@ -186,11 +186,21 @@ def main():
     dwall, dev_ms = timed_loop(hk, torch, dinputs, dC, args.steps, args.warmup)
     dbytes = algorithmic_bytes(dM, dN, dK)
     d_achieved = dbytes / (dev_ms * 1e-3) / 1e9
-    dtile = None
+    dtile = dbatched = None
     if args.layouts == "both":
         dtin = [(ap, hk.tile_operand(bp), asc, hk.tile_scales(bsc, dK)) for ap, bp, asc, bsc in dinputs]
         dtwall, dtev_ms = timed_loop(hk, torch, dtin, dC, args.steps, args.warmup, 0, 1)
+        # batched decode: 64 rows of A against the same tile-major weights (the skinny kernel with two accumulator tiles)
+        bM = 64
+        ba, bas = hk.quantize(torch.randn(bM, dK, device="cuda"), 2)
+        bC = torch.empty(bM, dN, dtype=torch.bfloat16, device="cuda")
+        bwall, bev_ms = timed_loop(hk, torch, [(ba, bt, bas, bst) for _, bt, _, bst in dtin], bC, args.steps, args.warmup, 0, 1)
+        bbytes = algorithmic_bytes(bM, dN, dK)
         del dtin
+        dbatched = {
+            "what": "M=64 against the same tile-major weights", "achieved": bbytes / (bev_ms * 1e-3) / 1e9, "unit": "GB/s",
+            "frac": bbytes / (bev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "launch_ms_mean": bev_ms, "algorithmic_bytes_per_launch": bbytes,
+        }
         dtile = {
             "what": "same decode workload, weights (B) and their scales tile-major",
             "achieved": dbytes / (dtev_ms * 1e-3) / 1e9, "unit": "GB/s", "frac": dbytes / (dtev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -241,6 +251,7 @@ def main():
             "algorithmic_bytes_per_launch": dbytes,
         },
         "tile_major_weights": dtile,
+        "batched_m64": dbatched,
     }
 
     line = {
