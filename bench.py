@@ -84,9 +84,11 @@ def timed_loop(hk, torch, inputs, C, steps, warmup, layout_a=0, layout_b=0):
     return wall, e0.elapsed_time(e1) / steps
 
 
-def cpu_baseline(inputs, M_sample):
-    """The C oracle (OpenMP) on the first M_sample rows of A against all of B: same bytes as the GPU run."""
+def cpu_baseline(inputs, M_sample, gpu_f32):
+    """The C oracle (OpenMP) on the first M_sample rows of A against all of B: same bytes as the GPU run.  gpu_f32 is the
+    library's result for the same rows before the bf16 rounding: the two are compared with the parity metric."""
     from oracle import c_oracle as co
+    from oracle import mxfp6_oracle as o
 
     ap, bp, asc, bsc = inputs
     ap_h = ap[:M_sample].cpu().numpy()
@@ -94,9 +96,11 @@ def cpu_baseline(inputs, M_sample):
     bp_h, bsc_h = bp.cpu().numpy(), bsc.cpu().numpy()
     N, K = bp_h.shape[0], bp_h.shape[1] // 3 * 4
     t0 = time.perf_counter()
-    co.gemm_f32(ap_h, bp_h, asc_h, bsc_h, 2, 2)
+    ref = co.gemm_f32(ap_h, bp_h, asc_h, bsc_h, 2, 2)
     dt = time.perf_counter() - t0
     return {
+        "max_rel_err_gpu_vs_cpu": o.rel_err(gpu_f32, ref),
+        "max_rel_err_bar": 2e-3,
         "value": 2.0 * M_sample * N * K / dt / 1e12,
         "unit": "TFLOPS",
         "cores": co.num_threads(),
@@ -166,7 +170,14 @@ def main():
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(inputs[0], args.cpu_rows)
+        ap0, bp0, asc0, bsc0 = inputs[0]
+        c32 = torch.empty(args.cpu_rows, N, dtype=torch.float32, device="cuda")
+        hk.dispatch_micro(ap0[: args.cpu_rows], bp0, asc0[: args.cpu_rows], bsc0, c32)
+        torch.cuda.synchronize()
+        gpu_f32 = c32.cpu().numpy()
+        del c32
+        cpu = cpu_baseline(inputs[0], args.cpu_rows, gpu_f32)
+        del gpu_f32
 
     # callers that keep their operands tile-major (MXFP6_LAYOUT_TILE; weights converted once, activations straight
     # from the quantiser) skip the pre-pass: that is the kernel-only figure above
