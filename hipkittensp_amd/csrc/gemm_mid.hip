@@ -85,8 +85,12 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
   const bool a_wave = wave < 4;                  // waves 0-3 load A and the scales, waves 4-7 load B
   const int lw = wave & 3;
   const int nkt = K / 128, sbytes = K / 32, rowbytes = K / 4 * 3, nk4 = nkt / 4;
-  // consecutive workgroups share their rows of B (they hit in L2 / the last-level cache together)
-  const int nb = blockIdx.x / mblocks, mb = blockIdx.x - nb * mblocks;
+  // The mblocks workgroups that share rows of B are 8 apart in launch order: workgroups go round-robin over the 8 XCDs,
+  // so these land on one XCD at about the same time and the later ones find B in that XCD's L2.  (The last, incomplete
+  // group of 8 * mblocks workgroups is numbered consecutively.)
+  const int chunk = 8 * mblocks, bid = blockIdx.x, full = (int)(gridDim.x / chunk) * chunk;
+  const int nb = bid < full ? (bid / chunk) * 8 + (bid & 7) : bid / mblocks;
+  const int mb = bid < full ? (bid % chunk) >> 3 : bid % mblocks;
   const int n0 = nb * BN, m0 = mb * BM;
   const int nrows = min(BN, N - n0), mrows = min(BM, M - m0);
 
