@@ -289,7 +289,9 @@ SplitWs split_workspace(hipStream_t s) {
   }
   SplitWs w;
   if (hipMalloc((void**)&w.part, (size_t)kWsSlots * 4096) != hipSuccess) { (void)hipGetLastError(); return {}; }
-  if (hipMalloc((void**)&w.cnt, kWsTiles * sizeof(int)) != hipSuccess || hipMemset(w.cnt, 0, kWsTiles * sizeof(int)) != hipSuccess) {
+  // cleared on the caller's stream (not being captured here): ordered before the launch that follows, whatever that
+  // stream's relation to the null stream is
+  if (hipMalloc((void**)&w.cnt, kWsTiles * sizeof(int)) != hipSuccess || hipMemsetAsync(w.cnt, 0, kWsTiles * sizeof(int), s) != hipSuccess) {
     (void)hipGetLastError();
     (void)hipFree(w.part);
     return {};
