@@ -290,7 +290,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 109; }
+int mxfp6_abi_version(void) { return 110; }
 
 #pragma GCC visibility pop
 }  // extern "C"
