@@ -128,7 +128,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.tile_rows = force == 5 ? 128 : force == 6 ? 256 : 0;
     e = mxfp6::launch_gemm_tiled(g, s);
-  } else if (force == 3 || (force >= 7 && force <= 15)) {
+  } else if (force == 3 || (force >= 7 && force <= 16)) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.skinny_geometry = force == 3 ? 0 : force - 6;
     e = mxfp6::launch_gemm_skinny(g, s);
@@ -244,7 +244,7 @@ int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, voi
 int mxfp6_set_relayout(int on) { return g_relayout.exchange(on ? 1 : 0); }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 15) return g_force.load();
+  if (which < 0 || which > 16) return g_force.load();
   return g_force.exchange(which);
 }
 
@@ -290,7 +290,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 110; }
+int mxfp6_abi_version(void) { return 111; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -302,11 +302,13 @@ SplitWs split_workspace(hipStream_t s) {
 }  // namespace
 
 // Geometry.  Few rows of B (N / 32 workgroups would leave CUs idle): a workgroup takes 16 rows of B, and the K range
-// is split between 2, 4 or 8 workgroups while that still fits the CUs and leaves every wave kMinChunks chunks.  Many
-// (N / 32 is several times the CU count): half as many waves per workgroup, so that two workgroups share a CU and
-// one's first loads run under the other's stream (a workgroup with a short K range is mostly load latency).
+// is split between 2, 4 or 8 workgroups while that still fits the CUs and leaves every wave kMinChunks chunks.  More
+// than one workgroup per CU (N / 32 above the CU count): half as many waves per workgroup, so that two workgroups share
+// a CU and one's first loads run under the other's stream (a workgroup with a short K range is mostly load latency);
+// with at most 16 chunks of K and up to 16 rows of A, two waves per workgroup (eight workgroups share a CU, each wave
+// streams a longer part of K: measured 5 - 13 % at N = 14336 .. 28672, K = 4096 .. 8192, nothing beyond N = 32768).
 // skinny_geometry: 1 - 3 fix the workgroup shape without a split; 4 + 3 * b + log2(split) - 1 (b = 0: 32 rows of B,
-// b = 1: 16 rows) fixes both.
+// b = 1: 16 rows) fixes both; 10 = two waves per workgroup.
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   typedef typename Out::type T;
@@ -316,13 +318,15 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   if (g.M > 32) {
     // 33 - 128 rows of A: two or four accumulator tiles per wave, four waves or two (two workgroups per CU), no K split
     geo = g.skinny_geometry == 3 || (g.skinny_geometry == 0 && wgs32 > 256) ? 3 : 1;
+  } else if (g.skinny_geometry == 10) {
+    geo = g.M <= 16 ? 5 : 3;  // two waves per workgroup (up to 16 rows of A)
   } else if (g.skinny_geometry >= 4) {
     geo = 1 + (g.skinny_geometry - 4) / 3;
     want = 2 << ((g.skinny_geometry - 4) % 3);
   } else if (g.skinny_geometry) {
     geo = g.skinny_geometry;
   } else {
-    geo = wgs32 <= 128 ? 2 : wgs32 >= 512 ? 3 : 1;
+    geo = wgs32 <= 128 ? 2 : wgs32 <= 256 ? 1 : g.M <= 16 && wgs32 <= 1024 && nchunks <= 16 ? 5 : 3;
     constexpr int kMinChunks = 3;  // measured: below this the 2.5 us of the second phase outweigh the wider stream
     const unsigned tiles = geo == 2 ? (g.N + 15) / 16 : wgs32;
     if (geo != 3)
@@ -343,7 +347,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   } else if (g.M > 32) {
     if (geo == 3) MXFP6_SK(64, 2, 32); else MXFP6_SK(64, 4, 32);
   } else if (g.M <= 16) {
-    if (geo == 2) MXFP6_SK(16, 8, 16); else if (geo == 3) MXFP6_SK(16, 4, 32); else MXFP6_SK(16, 8, 32);
+    if (geo == 2) MXFP6_SK(16, 8, 16); else if (geo == 3) MXFP6_SK(16, 4, 32); else if (geo == 5) MXFP6_SK(16, 2, 32); else MXFP6_SK(16, 8, 32);
   } else {
     if (geo == 2) MXFP6_SK(32, 6, 16); else if (geo == 3) MXFP6_SK(32, 3, 32); else MXFP6_SK(32, 6, 32);
   }

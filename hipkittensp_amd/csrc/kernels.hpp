@@ -14,7 +14,7 @@ struct GemmArgs {
   bool f32out;
   int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (operand: 32 rows x 128 elements in LDS image order; scales: 32 rows x 16 bytes)
   int tile_rows = 0;               // tiled kernel: rows of A per output tile, 128 or 256; 0 = chosen per shape
-  int skinny_geometry = 0;         // skinny kernel: 1 = 32 rows of B and all waves, 2 = 16 rows of B, 3 = half the waves, 4 - 9 = 1 or 2 with the K range split between 2 / 4 / 8 workgroups; 0 = by shape
+  int skinny_geometry = 0;         // skinny kernel: 1 = 32 rows of B and all waves, 2 = 16 rows of B, 3 = half the waves, 4 - 9 = 1 or 2 with the K range split between 2 / 4 / 8 workgroups, 10 = two waves; 0 = by shape
   Epilogue ep;                     // fused bias / scales / activation (all optional)
   uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
   int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output

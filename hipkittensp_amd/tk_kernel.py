@@ -39,6 +39,7 @@ KERNEL_AUTO, KERNEL_GENERIC, KERNEL_TILED, KERNEL_SKINNY, KERNEL_MID, KERNEL_TIL
 KERNEL_SKINNY_32, KERNEL_SKINNY_16, KERNEL_SKINNY_HALF = 7, 8, 9  # skinny kernel: rows of B per workgroup 32 / 16, or 32 with half the waves
 KERNEL_SKINNY_32_SPLIT = (10, 11, 12)  # 32 rows of B, K range split between 2 / 4 / 8 workgroups
 KERNEL_SKINNY_16_SPLIT = (13, 14, 15)  # 16 rows of B, likewise
+KERNEL_SKINNY_2WAVES = 16  # 32 rows of B, two waves per workgroup (wide N, short K)
 
 
 def _as_tensor(obj, name: str):

@@ -75,7 +75,7 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  * K % 512 == 0; its workgroup geometry follows N), 4 = mid-M kernel (needs 32 < M <= 512, K % 1024 == 0,
  * row-major A), 5 / 6 = the tiled kernel with 128- / 256-row tiles, 7 / 8 / 9 = the skinny kernel with 32 rows of B
  * per workgroup / 16 rows / 32 rows and half the waves (none of them splitting K), 10 / 11 / 12 = 32 rows of B with
- * the K range split between 2 / 4 / 8 workgroups, 13 / 14 / 15 = the same with 16 rows of B (the split takes a
+ * the K range split between 2 / 4 / 8 workgroups, 13 / 14 / 15 = the same with 16 rows of B, 16 = 32 rows of B and two waves per workgroup (the split takes a
  * workspace of 8 MB per stream at first use; without one, e.g. first use under stream capture, the launch runs
  * unsplit).  A forced kernel that cannot run the given
  * shape makes the gemm calls return MXFP6_EINVAL_SHAPE.  Returns the previous value.
