@@ -166,3 +166,13 @@ def test_torch_op_fake_shapes():
     import pytest
     with pytest.raises(RuntimeError):
         torch.ops.hipkittensp.mxfp6_gemm(A, B, As, Bs[:, :7], 2, 2, 0, 0, False)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in (r.stdout + r.stderr)
