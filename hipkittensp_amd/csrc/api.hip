@@ -124,9 +124,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     e = mxfp6::launch_gemm_generic(g, s);  // act(bias) everywhere: the generic kernel's K loop runs zero times
   } else if (force == 1) {
     e = mxfp6::launch_gemm_generic(g, s);
-  } else if (force == 2 || force == 5 || force == 6) {
+  } else if (force == 2 || force == 5 || force == 6 || force == 17) {
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
-    g.tile_rows = force == 5 ? 128 : force == 6 ? 256 : 0;
+    g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
     e = mxfp6::launch_gemm_tiled(g, s);
   } else if (force == 3 || (force >= 7 && force <= 16)) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
@@ -194,11 +194,11 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C_packed, M, N, K, fmt_a, fmt_b, false, layout_a, layout_b};
   const int force = g_force.load(std::memory_order_relaxed);
   const bool tiled = K > 0 && mxfp6::gemm_tiled_supports(g) &&
-                     (force == 2 || force == 5 || force == 6 ||
+                     (force == 2 || force == 5 || force == 6 || force == 17 ||
                       (force == 0 && !mxfp6::gemm_skinny_preferred(g) && !mxfp6::gemm_mid_preferred(g)));
   if (tiled) {
     g.ep = ep, g.C_scale = (uint8_t*)C_scale, g.fmt_c = fmt_c;
-    g.tile_rows = force == 5 ? 128 : force == 6 ? 256 : 0;
+    g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
     hipError_t e;
     if (force != 0 || !relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
     return e == hipSuccess ? MXFP6_OK : (int)e;
@@ -244,7 +244,7 @@ int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, voi
 int mxfp6_set_relayout(int on) { return g_relayout.exchange(on ? 1 : 0); }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 16) return g_force.load();
+  if (which < 0 || which > 17) return g_force.load();
   return g_force.exchange(which);
 }
 
@@ -290,7 +290,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 111; }
+int mxfp6_abi_version(void) { return 112; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -299,7 +299,7 @@ bool gemm_mid_preferred(const GemmArgs& g) {
   if (!gemm_mid_supports(g)) return false;
   if (!gemm_tiled_supports(g)) return true;
   const double t = mid_estimate_us(g);
-  return t < tiled_estimate_us(g, 128) && t < tiled_estimate_us(g, 256);
+  return t < tiled_estimate_us(g, 128) && t < tiled_estimate_us(g, 256) && t < tiled_estimate_us(g, 128, 128);
 }
 
 template <int FA, int FB, typename Out>

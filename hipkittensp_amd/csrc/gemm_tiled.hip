@@ -51,24 +51,25 @@ namespace mxfp6 {
 
 int g_tiled_walk = 1;  // 0: always one workgroup per output tile (development switch)
 
-constexpr int kBN = 256, kBK = 128;  // the tile has 256 (TM = 4) or 128 (TM = 2) rows of A
+constexpr int kBK = 128;  // the tile has 256 (TM = 4) or 128 (TM = 2) rows of A and 256 (TN = 2) or 128 (TN = 1) rows of B
 constexpr int kScStage = 256 * 16;   // bytes of one operand's scales for four K-tiles
 constexpr int kGroupM = 4;          // tile rows per raster group
 constexpr int kStages = 3;          // operand ring depth
 constexpr int kScaleBuf = 2 * kScStage;
-constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile (TM * 32) x 64
-constexpr int TN = 8 / WN;                   // 32x32 MFMA tiles per wave in N; in M: TM, a template parameter (4 or 2)
-constexpr int OPB = 24 / NW;                 // direct loads per wave and K-tile for B's 256 rows
+constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile (TM * 32) x (TN * 32)
 constexpr int SCL = 1;                       // scale direct loads per wave per slot that carries scales
-constexpr int kLoadsInCompute = 4;           // of the operand loads per wave and K-tile: issued between MFMAs
-// Per tile height.  A's 128 rows are 12 loads of 1 KB for 8 waves: every wave issues two, and the last four of
-// the sixteen lie past the end of A's buffer resource (they fetch nothing and fill padding behind the A tile).
-template <int TM>
+// Per tile shape: TM (4 or 2) and TN (2 or 1) 32x32 MFMA tiles per wave in M and N.  An operand tile of 128 rows is
+// 12 loads of 1 KB for 8 waves: every wave issues two, and the last four of the sixteen lie past the end of the
+// operand's buffer resource (they fetch nothing and fill padding behind the tile).
+template <int TM, int TN>
 struct Shape {
-  static constexpr int BM = WM * TM * 32;
+  static constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   static constexpr int OPA = (BM * 96 / 1024 + NW - 1) / NW;  // direct loads per wave and K-tile for A
+  static constexpr int OPB = (BN * 96 / 1024 + NW - 1) / NW;  // ... and for B
   static constexpr int NL = OPA + OPB;                        // operand loads per wave and K-tile
-  static constexpr int kAStage = OPA * NW * 1024, kStage = kAStage + kBN * 96;  // LDS bytes of A's tile (padded), of a ring slot
+  // of the operand loads per wave and K-tile: issued between MFMAs, one after every second of the 2 TM TN
+  static constexpr int kLoadsInCompute = TM * TN < 4 ? TM * TN : 4;
+  static constexpr int kAStage = OPA * NW * 1024, kStage = kAStage + OPB * NW * 1024;  // LDS bytes of A's tile (padded), of a ring slot
   static constexpr int kScaleBase = kStages * kStage, kLdsBytes = kScaleBase + 2 * kScaleBuf;
   static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= NL && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
   static_assert(kLdsBytes <= 163840, "LDS budget");
@@ -110,10 +111,12 @@ struct TiledArgs {
 // FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
 // around updates of all accumulators make the compiler copy them at every output tile, taken or not (3-4 % of an
 // unfused 8192^3 GEMM).
-template <int FA, int FB, typename Out, int TM, bool FUSED>
+template <int FA, int FB, typename Out, int TM, int TN, bool FUSED>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
-  typedef Shape<TM> S;
-  constexpr int kBM = S::BM, OPA = S::OPA, NL = S::NL, kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase;
+  typedef Shape<TM, TN> S;
+  constexpr int kBM = S::BM, kBN = S::BN, OPA = S::OPA, OPB = S::OPB, NL = S::NL, kLoadsInCompute = S::kLoadsInCompute;
+  constexpr int kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase;
+  static_assert(TN == 2 || sizeof(typename Out::type) != 1, "the fp6 epilogue pairs a wave's two tiles of a band");
   // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
   __shared__ __attribute__((aligned(1024))) uint8_t smem[S::kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
@@ -640,15 +643,15 @@ static int grid_size(const GemmArgs& g, int tiles) {
 // dealt to the CUs in rounds, and a K-tile of a round takes longer the fuller the round is (fewer active CUs run
 // at a higher clock and meet less L2 contention).  Constants measured on MI355X with tile-major B: 8192-wide
 // problems of 64 K-tiles took 57.7 / 62.7 / 70.1 / 86.9 us with 64 / 128 / 192 / 256 tiles of 256 rows and
-// 43.5 / 46.5 / 53.9 us with 128 / 192 / 256 tiles of 128 rows; row-major B costs about 28 % more, and no shape
-// runs faster than its bytes stream.
-double tiled_estimate_us(const GemmArgs& g, int rows) {
+// 43.5 / 46.5 / 53.9 us with 128 / 192 / 256 tiles of 128 rows, 34.1 / 38.9 / 73.8 us with 128 / 256 / 512 tiles of
+// 128 x 128; row-major B costs about 28 % more, and no shape runs faster than its bytes stream.
+double tiled_estimate_us(const GemmArgs& g, int rows, int cols) {
   int cus = cu_count();
   if (cus <= 0) cus = 256;
-  const long tiles = (long)((g.M + rows - 1) / rows) * ((g.N + kBN - 1) / kBN);
+  const long tiles = (long)((g.M + rows - 1) / rows) * ((g.N + cols - 1) / cols);
   const long full = tiles / cus;
   const double f = (double)(tiles % cus) / cus;
-  const double c0 = rows == 128 ? 0.62 : 0.85, c1 = rows == 128 ? 0.22 : 0.50;
+  const double c0 = cols == 128 ? 0.45 : rows == 128 ? 0.62 : 0.85, c1 = cols == 128 ? 0.10 : rows == 128 ? 0.22 : 0.50;
   const double per_ktile = full * (c0 + c1) + (f > 0 ? c0 + c1 * f * f : 0.0);
   const double layout = 1.0 + (g.layout_b ? 0.0 : 0.28) - (g.layout_a ? 0.05 : 0.0);
   // few rows of A against a large B is a streaming problem: measured 3.5 / 3.3 TB/s (tile-major B, 128- / 256-row
@@ -659,27 +662,33 @@ double tiled_estimate_us(const GemmArgs& g, int rows) {
   return compute > stream ? compute : stream;
 }
 
-// Tile height: 256 rows of A per tile unless tiles of 128 rows fill the machine better.
-static int tile_rows(const GemmArgs& g) {
-  if (g.tile_rows == 128 || g.tile_rows == 256) return g.tile_rows;
-  return tiled_estimate_us(g, 128) < tiled_estimate_us(g, 256) ? 128 : 256;
+// Tile shape: 256 x 256 unless tiles of 128 rows of A, or of 128 x 128, fill the machine better (the fp6 output needs
+// 256 columns).  Returns rows | cols << 16.
+static int tile_shape(const GemmArgs& g) {
+  if (g.tile_rows == 128 || g.tile_rows == 256) return g.tile_rows | (g.tile_cols == 128 && g.tile_rows == 128 && !g.fmt_c ? 128 : 256) << 16;
+  const double t256 = tiled_estimate_us(g, 256, 256), t128 = tiled_estimate_us(g, 128, 256);
+  const double t128n = g.fmt_c ? 1e30 : tiled_estimate_us(g, 128, 128);
+  if (t128n < t128 && t128n < t256) return 128 | 128 << 16;
+  return (t128 < t256 ? 128 : 256) | 256 << 16;
 }
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  const int bm = tile_rows(g);
-  const int tm = (g.M + bm - 1) / bm, tn = (g.N + kBN - 1) / kBN;
+  const int shape = tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
+  const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
   const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c};
   const int grid = grid_size(g, tm * tn);
   if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
-    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, true><<<grid, NW * 64, 0, s>>>(ta);
-    else gemm_tiled_kernel<FA, FB, Out, 4, true><<<grid, NW * 64, 0, s>>>(ta);
+    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
+    else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
   } else if (epilogue_any(g.ep)) {
-    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, true><<<grid, NW * 64, 0, s>>>(ta);
-    else gemm_tiled_kernel<FA, FB, Out, 4, true><<<grid, NW * 64, 0, s>>>(ta);
+    if (bn == 128) gemm_tiled_kernel<FA, FB, Out, 2, 1, true><<<grid, NW * 64, 0, s>>>(ta);
+    else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
+    else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
   } else {
-    if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, false><<<grid, NW * 64, 0, s>>>(ta);
-    else gemm_tiled_kernel<FA, FB, Out, 4, false><<<grid, NW * 64, 0, s>>>(ta);
+    if (bn == 128) gemm_tiled_kernel<FA, FB, Out, 2, 1, false><<<grid, NW * 64, 0, s>>>(ta);
+    else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, false><<<grid, NW * 64, 0, s>>>(ta);
+    else gemm_tiled_kernel<FA, FB, Out, 4, 2, false><<<grid, NW * 64, 0, s>>>(ta);
   }
   return hipGetLastError();
 }

@@ -14,6 +14,7 @@ struct GemmArgs {
   bool f32out;
   int layout_a = 0, layout_b = 0;  // 0 = row-major, 1 = tile-major (operand: 32 rows x 128 elements in LDS image order; scales: 32 rows x 16 bytes)
   int tile_rows = 0;               // tiled kernel: rows of A per output tile, 128 or 256; 0 = chosen per shape
+  int tile_cols = 0;               // ... and rows of B: 128 (with 128 rows of A only) or 256; 0 with tile_rows set = 256
   int skinny_geometry = 0;         // skinny kernel: 1 = 32 rows of B and all waves, 2 = 16 rows of B, 3 = half the waves, 4 - 9 = 1 or 2 with the K range split between 2 / 4 / 8 workgroups, 10 = two waves; 0 = by shape
   Epilogue ep;                     // fused bias / scales / activation (all optional)
   uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
@@ -25,7 +26,7 @@ bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
 bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
-double tiled_estimate_us(const GemmArgs& g, int rows);  // estimated time of the tiled kernel with 128- or 256-row tiles
+double tiled_estimate_us(const GemmArgs& g, int rows, int cols = 256);  // estimated time of the tiled kernel with tiles of rows x cols
 double mid_estimate_us(const GemmArgs& g);
 hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);

@@ -40,6 +40,7 @@ KERNEL_SKINNY_32, KERNEL_SKINNY_16, KERNEL_SKINNY_HALF = 7, 8, 9  # skinny kerne
 KERNEL_SKINNY_32_SPLIT = (10, 11, 12)  # 32 rows of B, K range split between 2 / 4 / 8 workgroups
 KERNEL_SKINNY_16_SPLIT = (13, 14, 15)  # 16 rows of B, likewise
 KERNEL_SKINNY_2WAVES = 16  # 32 rows of B, two waves per workgroup (wide N, short K)
+KERNEL_TILED_128x128 = 17  # tiled kernel with output tiles of 128 x 128
 
 
 def _as_tensor(obj, name: str):

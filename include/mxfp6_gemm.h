@@ -69,16 +69,18 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
                       float *C_f32, int M, int N, int K, int fmt_a, int fmt_b, void *hip_stream);
 
 /*
- * Kernel selection override for measurement and tests: 0 = automatic (default), 1 = generic
- * one-wave-per-tile kernel, 2 = LDS-tiled MFMA kernel (needs N % 8 == 0, K % 128 == 0; 128 or 256 rows of A
- * per output tile, whichever fills the GPU better), 3 = skinny-M streaming kernel (needs M <= 128,
- * K % 512 == 0; its workgroup geometry follows N), 4 = mid-M kernel (needs 32 < M <= 512, K % 1024 == 0,
- * row-major A), 5 / 6 = the tiled kernel with 128- / 256-row tiles, 7 / 8 / 9 = the skinny kernel with 32 rows of B
- * per workgroup / 16 rows / 32 rows and half the waves (none of them splitting K), 10 / 11 / 12 = 32 rows of B with
- * the K range split between 2 / 4 / 8 workgroups, 13 / 14 / 15 = the same with 16 rows of B, 16 = 32 rows of B and two waves per workgroup (the split takes a
- * workspace of 8 MB per stream at first use; without one, e.g. first use under stream capture, the launch runs
- * unsplit).  A forced kernel that cannot run the given
- * shape makes the gemm calls return MXFP6_EINVAL_SHAPE.  Returns the previous value.
+ * Kernel selection override for measurement and tests.  Returns the previous value.  A forced kernel that cannot run the
+ * given shape makes the gemm calls return MXFP6_EINVAL_SHAPE.
+ *    0  automatic (default)
+ *    1  generic one-wave-per-tile kernel (any shape)
+ *    2  LDS-tiled MFMA kernel (needs N % 8 == 0, K % 128 == 0), tile shape by how it fills the GPU;
+ *       5 / 6 / 17: with output tiles of 128 x 256 / 256 x 256 / 128 x 128 (rows of A x rows of B)
+ *    3  skinny-M streaming kernel (needs M <= 128, K % 512 == 0), workgroup geometry by N and K;
+ *       7 / 8 / 9: 32 rows of B per workgroup / 16 rows / 32 rows and half the waves, none of them splitting K;
+ *       10 / 11 / 12: 32 rows of B, the K range split between 2 / 4 / 8 workgroups; 13 / 14 / 15: the same with 16 rows
+ *       (the split takes a workspace of 8 MB per stream at first use; without one, e.g. first use under stream capture,
+ *       the launch runs unsplit); 16: 32 rows of B and two waves per workgroup
+ *    4  mid-M kernel (needs 32 < M <= 512, K % 1024 == 0, row-major A)
  * No counterpart in the reference, whose shapes are compile-time constants per binary
  * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
  */

@@ -403,7 +403,7 @@ def test_automatic_dispatch_agrees_with_generic_kernel_on_ragged_shapes(hk):
 def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, lb, out):
     """More output tiles than compute units: every workgroup of the tiled kernel takes several tiles in turn, the loads of
     the next tile running under the last K-tiles of the current one (K-tile counts 4n, 4n+2, 4n+3; 4n+1 keeps one workgroup
-    per tile), with ragged edge tiles and tile-major operands, for both tile heights (128 and 256 rows of A).  The result
+    per tile), with ragged edge tiles and tile-major operands, for every tile shape (256 x 256, 128 x 256, 128 x 128).  The result
     must equal the one-wave-per-tile kernel's in every
     bit (both round the same fp32 sums once), and nothing may be written outside C (guard rows before and after it)."""
     g = torch.Generator(device="cuda")
@@ -413,7 +413,7 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
     prev_r = hk.tk_kernel.set_relayout(0)
     res = []
     try:
-        for kern in (1, hk.tk_kernel.KERNEL_TILED_128, hk.tk_kernel.KERNEL_TILED_256):
+        for kern in (1, hk.tk_kernel.KERNEL_TILED_128, hk.tk_kernel.KERNEL_TILED_256, hk.tk_kernel.KERNEL_TILED_128x128):
             full = torch.full((M + 2, N), 12345.0, dtype=out, device="cuda")
             prev = hk.tk_kernel.set_kernel(kern)
             try:
@@ -432,7 +432,8 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
 
 # ------------------------------------------------------------------ fused epilogue
 @pytest.mark.parametrize("kernel,M,N,K", [(1, 70, 40, 96), (3, 16, 96, 1024), (3, 32, 100, 512), (4, 64, 72, 1024), (4, 200, 136, 2048),
-                                          (5, 300, 264, 640), (6, 300, 264, 640), (5, 1024, 4104, 512), (6, 2304, 8200, 512)])
+                                          (5, 300, 264, 640), (6, 300, 264, 640), (5, 1024, 4104, 512), (6, 2304, 8200, 512),
+                                          (17, 300, 264, 640), (17, 1024, 4104, 512)])
 @pytest.mark.parametrize("activation", [None, "relu", "gelu", "silu"])
 def test_fused_epilogue_every_kernel(hk, kernel, M, N, K, activation):
     """act(acc * row_scale * col_scale + bias) fused into each kernel's epilogue (the last two shapes have more tiles than
