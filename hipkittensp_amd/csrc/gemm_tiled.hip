@@ -52,24 +52,29 @@ namespace mxfp6 {
 int g_tiled_walk = 1;  // 0: always one workgroup per output tile (development switch)
 
 constexpr int kBK = 128;  // the tile has 256 (TM = 4) or 128 (TM = 2) rows of A and 256 (TN = 2) or 128 (TN = 1) rows of B
-constexpr int kScStage = 256 * 16;   // bytes of one operand's scales for four K-tiles
 constexpr int kGroupM = 4;          // tile rows per raster group
 constexpr int kStages = 3;          // operand ring depth
-constexpr int kScaleBuf = 2 * kScStage;
 constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile (TM * 32) x (TN * 32)
 constexpr int SCL = 1;                       // scale direct loads per wave per slot that carries scales
-// Per tile shape: TM (4 or 2) and TN (2 or 1) 32x32 MFMA tiles per wave in M and N.  An operand tile of 128 rows is
-// 12 loads of 1 KB for 8 waves: every wave issues two, and the last four of the sixteen lie past the end of the
-// operand's buffer resource (they fetch nothing and fill padding behind the tile).
+// Per tile shape: TM (4 or 2) and TN (2 or 1) 32x32 MFMA tiles per wave in M and N.  A's tile of 128 rows against 256
+// of B is 12 loads of 1 KB for 8 waves: every wave issues two, and the last four of the sixteen lie past the end of
+// A's buffer resource (they fetch nothing and fill padding behind the tile).  128 x 128 (SPLIT): both tiles are 12
+// loads, waves 0-3 load A's and waves 4-7 B's, three each; no padding, and the scales take half the room (waves 2, 3,
+// 6, 7 fetch the same 64 rows as waves 0, 1, 4, 5 again, into the same place, so that every wave issues the same number
+// of loads): 80 KB, two workgroups per CU.
 template <int TM, int TN>
 struct Shape {
   static constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  static constexpr int OPA = (BM * 96 / 1024 + NW - 1) / NW;  // direct loads per wave and K-tile for A
-  static constexpr int OPB = (BN * 96 / 1024 + NW - 1) / NW;  // ... and for B
-  static constexpr int NL = OPA + OPB;                        // operand loads per wave and K-tile
+  static constexpr bool SPLIT = TM == 2 && TN == 1;
+  static constexpr int OPA = SPLIT ? 3 : (BM * 96 / 1024 + NW - 1) / NW;  // direct loads per (loading) wave and K-tile for A
+  static constexpr int OPB = SPLIT ? 3 : (BN * 96 / 1024 + NW - 1) / NW;  // ... and for B
+  static constexpr int NL = SPLIT ? 3 : OPA + OPB;                        // operand loads per wave and K-tile
   // of the operand loads per wave and K-tile: issued between MFMAs, one after every second of the 2 TM TN
   static constexpr int kLoadsInCompute = TM * TN < 4 ? TM * TN : 4;
-  static constexpr int kAStage = OPA * NW * 1024, kStage = kAStage + OPB * NW * 1024;  // LDS bytes of A's tile (padded), of a ring slot
+  static constexpr int kAStage = SPLIT ? BM * 96 : OPA * NW * 1024;  // LDS bytes of A's tile (padded)
+  static constexpr int kStage = kAStage + (SPLIT ? BN * 96 : OPB * NW * 1024);  // ... and of a ring slot
+  static constexpr int kScStage = (SPLIT ? 128 : 256) * 16;  // bytes of one operand's scales for four K-tiles
+  static constexpr int kScaleBuf = 2 * kScStage;
   static constexpr int kScaleBase = kStages * kStage, kLdsBytes = kScaleBase + 2 * kScaleBuf;
   static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= NL && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
   static_assert(kLdsBytes <= 163840, "LDS budget");
@@ -115,7 +120,8 @@ template <int FA, int FB, typename Out, int TM, int TN, bool FUSED>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
   typedef Shape<TM, TN> S;
   constexpr int kBM = S::BM, kBN = S::BN, OPA = S::OPA, OPB = S::OPB, NL = S::NL, kLoadsInCompute = S::kLoadsInCompute;
-  constexpr int kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase;
+  constexpr int kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase, kScStage = S::kScStage, kScaleBuf = S::kScaleBuf;
+  constexpr bool SPLIT = S::SPLIT;
   static_assert(TN == 2 || sizeof(typename Out::type) != 1, "the fp6 epilogue pairs a wave's two tiles of a band");
   // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
   __shared__ __attribute__((aligned(1024))) uint8_t smem[S::kLdsBytes];
@@ -156,8 +162,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const auto g = fresh_args();
     const int pm = tile < 0 ? 0 : tile & 0xffff, pn = tile < 0 ? 0 : tile >> 16;
     const int rows_a = tile < 0 ? 0 : min(kBM, g->M - pm * kBM), rows_b = tile < 0 ? 0 : min(kBN, g->N - pn * kBN);
-    rA = make_rsrc(g->A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
-    rB = make_rsrc(g->B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+    if constexpr (SPLIT) {  // a wave loads one operand only: rA is that operand's resource (no branch at the loads)
+      rA = sc_a ? make_rsrc(g->A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes)
+                : make_rsrc(g->B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+    } else {
+      rA = make_rsrc(g->A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
+      rB = make_rsrc(g->B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+    }
   };
   auto scale_rsrc = [&](int tile) __attribute__((always_inline)) {
     const auto g = fresh_args();
@@ -193,12 +204,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     return layout ? vtile : vrow;
   };
 #pragma unroll
-  for (int i = 0; i < OPA; i++) voff_a[i] = load_offset(wave * OPA + i, layout_a);
+  for (int i = 0; i < OPA; i++) voff_a[i] = SPLIT ? load_offset((wave & 3) * OPA + i, sc_a ? layout_a : layout_b) : load_offset(wave * OPA + i, layout_a);
 #pragma unroll
-  for (int i = 0; i < OPB; i++) voff_b[i] = load_offset(wave * OPB + i, layout_b);
-  const int kstep_a = layout_a ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
+  for (int i = 0; i < OPB; i++) voff_b[i] = SPLIT ? 0 : load_offset(wave * OPB + i, layout_b);
+  const int kstep_a = (SPLIT && !sc_a ? layout_b : layout_a) ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
+  const int split_base = (sc_a ? 0 : kAStage) + (wave & 3) * (OPA * 1024);  // SPLIT: where this wave's three loads land in a ring slot
   // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; waves 0-3 load A's, 4-7 B's
-  const int srow = (wave & 3) * 64 + lane, slay = wave < 4 ? layout_a : layout_b;
+  const int swave = SPLIT ? wave & 1 : wave & 3;  // which 64 rows of the operand's tile this wave fetches the scales of
+  const int srow = swave * 64 + lane, slay = wave < 4 ? layout_a : layout_b;
   const int voff_s = slay ? (srow >> 5) * nk4 * 512 + (srow & 31) * 16 : srow * sbytes;
   const int sstep = slay ? 512 : 16;  // bytes between consecutive groups of four K-tiles
 
@@ -226,14 +239,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // tile to empty resources.  INSIDE says that the caller knows kk to lie in the current tile.
   auto issue_scales = [&]<bool INSIDE>(int grp) __attribute__((always_inline)) {
     const int buf = (p0 + grp) & 1;
-    const uint32_t dst = lds0 + kScaleBase + buf * kScaleBuf + (wave & 3) * 1024;
+    const uint32_t dst = lds0 + kScaleBase + buf * kScaleBuf + swave * 1024;
     dma16(rS, sc_a ? dst : dst + kScStage, voff_s, (INSIDE || grp < nk4 ? grp : grp - nk4) * sstep);
   };
   auto issue_one = [&]<bool INSIDE>(int kk, int slot, int n) __attribute__((always_inline)) {
     const int t = INSIDE || kk < nkt ? kk : kk - nkt;
     const uint32_t dst = lds0 + slot * kStage;
-    if (n < OPA) dma16(rA, dst + (wave * OPA + n) * 1024, voff_a[n], t * kstep_a);
-    else dma16(rB, dst + kAStage + (wave * OPB + n - OPA) * 1024, voff_b[n - OPA], t * kstep_b);
+    if constexpr (SPLIT) {
+      dma16(rA, dst + split_base + n * 1024, voff_a[n], t * kstep_a);
+    } else {
+      if (n < OPA) dma16(rA, dst + (wave * OPA + n) * 1024, voff_a[n], t * kstep_a);
+      else dma16(rB, dst + kAStage + (wave * OPB + n - OPA) * 1024, voff_b[n - OPA], t * kstep_b);
+    }
   };
 
   // ---- one K-tile: LDS -> registers (memory cluster) and the MFMAs (compute cluster)
@@ -632,8 +649,8 @@ static int cu_count() {
 // scales of the next output tile are fetched with the last group of four K-tiles of the current one
 // and must have two steps to land: K-tile counts of 4n+1 (and fewer than four K-tiles) keep one
 // workgroup per tile.
-static int grid_size(const GemmArgs& g, int tiles) {
-  const int cus = cu_count() & ~7;  // whole multiples of the 8 XCDs keep the tile -> XCD mapping of the walk
+static int grid_size(const GemmArgs& g, int tiles, int per_cu) {
+  const int cus = (cu_count() & ~7) * per_cu;  // whole multiples of the 8 XCDs keep the tile -> XCD mapping of the walk
   const int nkt = g.K / kBK;
   if (g_tiled_walk == 0 || nkt < 4 || nkt % 4 == 1 || cus < 8) return tiles;
   return tiles < cus ? tiles : cus;
@@ -677,7 +694,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int shape = tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
   const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c};
-  const int grid = grid_size(g, tm * tn);
+  const int grid = grid_size(g, tm * tn, bn == 128 ? 2 : 1);  // 128 x 128: 80 KB of LDS, two workgroups per CU
   if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
     if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
     else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
