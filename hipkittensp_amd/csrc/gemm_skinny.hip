@@ -50,7 +50,7 @@ __device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt
 // AR = rows of A staged (16, 32 or 64: one or two 32-row accumulator tiles per wave); NW = waves per workgroup;
 // BR = rows of B per workgroup (32, or 16 so that a narrow N still gives every CU a workgroup: the MFMA's other 16
 // rows then mirror the first and their outputs are dropped)
-template <int FA, int FB, typename Out, int AR, int NW, int BR>
+template <int FA, int FB, typename Out, int AR, int NW, int BR, int DB>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                               typename Out::type* __restrict__ C, int M, int N, int K, int layout_b,
@@ -60,9 +60,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   constexpr int TA = AR > 32 ? AR / 32 : 1;   // accumulator tiles per wave
   constexpr int KT = AR == 128 ? 2 : 4;       // K-tiles per chunk (128 rows of A: half chunks, so that four waves' buffers fit)
   constexpr int kRow = 96 * KT, kPieces = 6 * KT;  // bytes and 16-byte pieces of a row in a chunk
-  constexpr int kBBuf = BR * kRow, kABuf = AR * kRow, kScOff = kBBuf + kABuf;  // one chunk of B and of A, then the scales:
-  constexpr int kASc = AR <= 64 ? 1024 : AR * 16;                              // 1 KB for B, 16 bytes per row of A
-  constexpr int kBuf = kScOff + 1024 + kASc;
+  // a wave's buffer: DB chunks of B (DB = 2: the chunk after the next is on its way from HBM while the next one's A, which
+  // comes from L2 in a fraction of that time, is fetched one chunk ahead), one chunk of A, then the scales:
+  static_assert(DB == 1 || DB == 2, "chunks of B per wave");
+  constexpr int kBBuf = BR * kRow, kABuf = AR * kRow, kAOff = DB * kBBuf, kScOff = kAOff + kABuf;
+  constexpr int kASc = AR <= 64 ? 1024 : AR * 16;                              // 1 KB per chunk of B, 16 bytes per row of A
+  constexpr int kAScOff = kScOff + DB * 1024;
+  constexpr int kBuf = kAScOff + kASc;
   constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024, NAS = kASc / 1024;  // direct loads per chunk: 12 or 6; 6, 12 or 24; 1 or 2
   static_assert(kBBuf % 1024 == 0 && kABuf % 1024 == 0, "whole direct loads");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kBuf];
@@ -124,7 +128,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     for (int c = 0; c < 3; c++) {
       const int p = u * 6 + 3 * h + c;
       b_rd[u][c] = layout_b ? u * (BR * 96) + rb * 96 + ((3 * h + c) ^ ((rb >> 3) & 1)) * 16 : rb * kRow + swz(p, rb) * 16;
-      a_rd[u][c] = kBBuf + ra * kRow + swz(p, ra) * 16;
+      a_rd[u][c] = kAOff + ra * kRow + swz(p, ra) * 16;
     }
 
   // chunks of this workgroup: [c0, c1); of this wave: c0 + wave, c0 + wave + NW, ...
@@ -132,19 +136,24 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   const int c0 = split * cps, c1 = min(nchunks, c0 + cps);
   const int mine = c0 + wave < c1 ? (c1 - c0 - wave + NW - 1) / NW : 0;
 
-  auto issue_chunk = [&](int chunk) __attribute__((always_inline)) {
+  // B's part of a chunk (NBL + 1 loads) into B buffer `par`, and A's part (NAL + NAS loads)
+  auto issue_b = [&](int chunk, int par) __attribute__((always_inline)) {
     const int sg = KT == 4 ? chunk : chunk >> 1;  // the scales come in groups of four K-tiles
-    const int sos = __builtin_amdgcn_readfirstlane(sg * 16);
     const int sosb = __builtin_amdgcn_readfirstlane(layout_b ? sg * 512 : sg * 16);
-    dma16_sk(rBs, buf + kScOff, voff_bs, sosb);
-#pragma unroll
-    for (int i = 0; i < NAS; i++) dma16_sk(rAs, buf + kScOff + 1024 + i * 1024, voff_as + i * 64 * sbytes, sos);
-    const int so = __builtin_amdgcn_readfirstlane(chunk * kRow);
+    const uint32_t pb = __builtin_amdgcn_readfirstlane(par);
+    dma16_sk(rBs, buf + kScOff + pb * 1024, voff_bs, sosb);
     const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * (KT * 3072) : chunk * kRow);
 #pragma unroll
-    for (int i = 0; i < NBL; i++) dma16_sk(rB, buf + i * 1024, voff_b[i], sob);
+    for (int i = 0; i < NBL; i++) dma16_sk(rB, buf + pb * kBBuf + i * 1024, voff_b[i], sob);
+  };
+  auto issue_a = [&](int chunk) __attribute__((always_inline)) {
+    const int sg = KT == 4 ? chunk : chunk >> 1;
+    const int sos = __builtin_amdgcn_readfirstlane(sg * 16);
 #pragma unroll
-    for (int i = 0; i < NAL; i++) dma16_sk(rA, buf + kBBuf + i * 1024, voff_a[i], so);
+    for (int i = 0; i < NAS; i++) dma16_sk(rAs, buf + kAScOff + i * 1024, voff_as + i * 64 * sbytes, sos);
+    const int so = __builtin_amdgcn_readfirstlane(chunk * kRow);
+#pragma unroll
+    for (int i = 0; i < NAL; i++) dma16_sk(rA, buf + kAOff + i * 1024, voff_a[i], so);
   };
 
   v16f acc[TA];
@@ -154,27 +163,40 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
 
   if (mine > 0) {
-    issue_chunk(c0 + wave);
+    // queue order: B(0), A(0), B(1), A(1), B(2), ...: with DB = 2 chunk j is read once everything up to A(j) has landed,
+    // while B(j+1), the youngest batch, stays in flight
+    issue_b(c0 + wave, 0);
+    issue_a(c0 + wave);
+    if (DB == 2 && mine > 1) issue_b(c0 + wave + NW, 1);
     for (int j = 0; j < mine; j++) {
-      wait_all_loads();
-      const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + rb * 16);
+      if (DB == 2 && j + 1 < mine) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NBL + 1) : "memory");
+      else wait_all_loads();
+      const int par = DB == 2 ? j & 1 : 0;
+      const uint8_t* bufb = bufp + par * kBBuf;
+      const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + par * 1024 + rb * 16);
       v4i sc_a[TA];
       v4i fb[KT][3], fa[TA][KT][3];
       const bool odd = KT == 2 && ((c0 + wave + j * NW) & 1);  // half chunks: which two of the four scale bytes
 #pragma unroll
-      for (int t = 0; t < TA; t++) sc_a[t] = *reinterpret_cast<const v4i*>(bufp + kScOff + 1024 + (t * 32 + ra) * 16);
+      for (int t = 0; t < TA; t++) sc_a[t] = *reinterpret_cast<const v4i*>(bufp + kAScOff + (t * 32 + ra) * 16);
 #pragma unroll
       for (int u = 0; u < KT; u++)
 #pragma unroll
         for (int c = 0; c < 3; c++) {
-          fb[u][c] = *reinterpret_cast<const v4i*>(bufp + b_rd[u][c]);
+          fb[u][c] = *reinterpret_cast<const v4i*>(bufb + b_rd[u][c]);
 #pragma unroll
           for (int t = 0; t < TA; t++) fa[t][u][c] = *reinterpret_cast<const v4i*>(bufp + a_rd[u][c] + t * (32 * kRow));
         }
       // the buffer is about to be refilled: its reads must have left LDS
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
-      if (j + 1 < mine) issue_chunk(c0 + wave + (j + 1) * NW);
+      if (DB == 2) {
+        if (j + 1 < mine) issue_a(c0 + wave + (j + 1) * NW);
+        if (j + 2 < mine) issue_b(c0 + wave + (j + 2) * NW, par);
+      } else if (j + 1 < mine) {
+        issue_b(c0 + wave + (j + 1) * NW, 0);
+        issue_a(c0 + wave + (j + 1) * NW);
+      }
 #pragma unroll
       for (int u = 0; u < KT; u++) {
         const int sb = (uint32_t)(KT == 4 ? sc_b[u] : odd ? sc_b[u + 2] : sc_b[u]) >> (16 * h);
@@ -339,18 +361,22 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     ws = split_workspace(s);
     if (ws.part) nsplit = want;
   }
-#define MXFP6_SK(AR, NW, BR) \
-  gemm_skinny_kernel<FA, FB, Out, AR, NW, BR><<<(g.N + BR - 1) / BR * nsplit, NW * 64, 0, s>>>( \
+#define MXFP6_SK(AR, NW, BR) MXFP6_SKD(AR, NW, BR, 1)
+#define MXFP6_SKD(AR, NW, BR, DB) \
+  gemm_skinny_kernel<FA, FB, Out, AR, NW, BR, DB><<<(g.N + BR - 1) / BR * nsplit, NW * 64, 0, s>>>( \
       g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, g.layout_b, g.ep, nsplit, ws.part, ws.cnt)
+  // two chunks of B per wave (17 - 32 and 65 - 128 rows of A: measured 3 - 15 % and 3 - 6 %); forced geometry 1: one
+  const bool db = g.skinny_geometry != 1;
   if (g.M > 64) {
-    if (geo == 3) MXFP6_SK(128, 2, 32); else MXFP6_SK(128, 4, 32);
+    if (geo == 3) MXFP6_SK(128, 2, 32); else if (db) MXFP6_SKD(128, 4, 32, 2); else MXFP6_SK(128, 4, 32);
   } else if (g.M > 32) {
-    if (geo == 3) MXFP6_SK(64, 2, 32); else MXFP6_SK(64, 4, 32);
+    if (geo == 3) MXFP6_SK(64, 2, 32); else MXFP6_SK(64, 4, 32);  // two chunks of B and three waves: measured level with this
   } else if (g.M <= 16) {
     if (geo == 2) MXFP6_SK(16, 8, 16); else if (geo == 3) MXFP6_SK(16, 4, 32); else if (geo == 5) MXFP6_SK(16, 2, 32); else MXFP6_SK(16, 8, 32);
   } else {
-    if (geo == 2) MXFP6_SK(32, 6, 16); else if (geo == 3) MXFP6_SK(32, 3, 32); else MXFP6_SK(32, 6, 32);
+    if (geo == 2) MXFP6_SK(32, 6, 16); else if (geo == 3) MXFP6_SK(32, 3, 32); else if (db && geo == 1) MXFP6_SKD(32, 4, 32, 2); else MXFP6_SK(32, 6, 32);
   }
+#undef MXFP6_SKD
 #undef MXFP6_SK
   return hipGetLastError();
 }
