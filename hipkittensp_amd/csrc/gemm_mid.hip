@@ -282,16 +282,22 @@ static bool mid_wide(const GemmArgs& g) {
 }
 
 // Estimated time of this kernel in microseconds: rounds of workgroups x K-tiles x time per K-tile and round.
-// Constants measured on MI355X (N = 8192 and 28672, K = 8192): 0.33 / 0.48 us for 64 rows of A with 32 / 64
-// rows of B per workgroup, 0.45 / 0.55 us for 128 rows of A (5 % less with more than one block of rows of A: the blocks
-// share B through one XCD's L2); row-major B costs about 6 % more; 5 us fixed.
+// Constants measured on MI355X.  One block of rows of A (M <= 128; N = 8192 and 28672, K = 8192): 0.33 / 0.48 us for 64
+// rows of A with 32 / 64 rows of B per workgroup, 0.45 / 0.55 us for 128 rows of A, 5 us fixed.  Several blocks (they
+// share B through one XCD's L2; N = 2048 .. 28672, K = 4096 .. 14336): 0.32 / 0.37 us in one round (12 % less when half
+// the CUs have a workgroup), 0.47 us per round in several, 7 / 9.5 us fixed.  Row-major B costs about 6 % more.
 double mid_estimate_us(const GemmArgs& g) {
   const bool wide = mid_wide(g);
   const int bn = wide ? 64 : 32;
   const double wgs = (double)((g.N + bn - 1) / bn) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
   const double rounds = wgs > 256 ? wgs / 256 : 1;
-  const double c = g.M <= 64 ? (wide ? 0.48 : 0.33) : (wide ? 0.55 : 0.45) * (g.M > 128 ? 0.95 : 1.0);
-  return 5.0 + rounds * (g.K / 128) * c * (g.layout_b ? 1.0 : 1.06);
+  const double layout = g.layout_b ? 1.0 : 1.06;
+  if (g.M > 128) {
+    const double c = rounds > 1 ? 0.47 : (wide ? 0.37 : 0.32) * (0.76 + 0.24 * wgs / 256);
+    return (wide ? 9.5 : 7.0) + rounds * (g.K / 128) * c * layout;
+  }
+  const double c = g.M <= 64 ? (wide ? 0.48 : 0.33) : (wide ? 0.55 : 0.45);
+  return 5.0 + rounds * (g.K / 128) * c * layout;
 }
 
 // Automatic choice against the LDS-tiled kernel with either tile height.
