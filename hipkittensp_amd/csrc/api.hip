@@ -1,16 +1,78 @@
 // C ABI of the MXFP6 GEMM library (declared in include/mxfp6_gemm.h): argument validation and
-// kernel selection.  Nothing here synchronises; the only allocation is the stream-ordered workspace of the
-// re-layout pre-pass (relayout_then_tiled), which mxfp6_set_relayout(0) switches off.
+// kernel selection.  Nothing here synchronises the device.  Allocations, all from the stream-ordered allocator on the
+// caller's stream and all kept per (device, stream) until mxfp6_release_workspaces(): the workspace of the re-layout
+// pre-pass (relayout_then_tiled; mxfp6_set_relayout(0) switches it off), the fp32 workspace of mxfp6_gemm_fused_fp6
+// on shapes the tiled kernel does not run, and the K-split workspace of the skinny kernel (gemm_skinny.hip).
 #include "../../include/mxfp6_gemm.h"
 
-#include <atomic>
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <utility>
 
 #include "kernels.hpp"
 
 namespace {
 
-std::atomic<int> g_force{0};
-std::atomic<int> g_relayout{1};
+// Overrides for measurement and tests: per thread, so that a thread that forces a kernel does not change what
+// other threads' calls run.
+thread_local int g_force = 0;
+thread_local int g_relayout = 1;
+
+// Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
+// demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
+struct StreamWs {
+  uint8_t* p = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_sws_mutex;
+std::map<std::tuple<int, hipStream_t, int>, StreamWs> g_sws;
+constexpr size_t kStreamWsMax = 128;
+
+// kind 0: pre-pass copies, kind 1: fp32 result of mxfp6_gemm_fused_fp6.  nullptr: no workspace (capture, limit, out of memory).
+uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(g_sws_mutex);
+  auto it = g_sws.find({dev, s, kind});
+  if (it != g_sws.end() && it->second.bytes >= bytes) return it->second.p;
+  // never allocate into a stream that is being captured: the caller replays the graph with its own memory plan
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (it == g_sws.end() && g_sws.size() >= kStreamWsMax) return nullptr;
+  uint8_t* p = nullptr;
+  const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+  if (hipMallocAsync((void**)&p, want, s) != hipSuccess || !p) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (it != g_sws.end()) {
+    (void)hipFreeAsync(it->second.p, s);
+    it->second = {p, want};
+  } else {
+    g_sws[{dev, s, kind}] = {p, want};
+  }
+  return p;
+}
+
+hipError_t release_stream_workspaces() {
+  std::lock_guard<std::mutex> lock(g_sws_mutex);
+  if (g_sws.empty()) return hipSuccess;
+  int cur = 0;
+  (void)hipGetDevice(&cur);
+  hipError_t first = hipSuccess;
+  for (auto& kv : g_sws) {
+    (void)hipSetDevice(std::get<0>(kv.first));
+    const hipError_t e = hipFreeAsync(kv.second.p, std::get<1>(kv.first));
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  }
+  g_sws.clear();
+  (void)hipSetDevice(cur);
+  return first;
+}
 
 int check_device() {
   // cached per process: the library only carries gfx950 code objects
@@ -29,11 +91,10 @@ int check_device() {
 // 648 with one operand tile-major and 400 with both).  Re-laying an operand out tile-major first costs two passes
 // over it at HBM speed (measured 23 us for 8192 x 8192) and shortens the GEMM by about 15 % (first operand) and
 // 11 % (second): from about 8192^3 on that pays for both, for a tall or wide problem only for the operand with
-// fewer rows.  The workspace comes from the stream-ordered allocator and is returned to it on the same stream
-// right after the GEMM has been enqueued.  Returns false when no pre-pass pays or it cannot run (then the caller
-// launches the row-major path).
+// fewer rows.  The workspace is this stream's (stream_workspace: allocated once, kept).  Returns false when no
+// pre-pass pays or it cannot run (then the caller launches the row-major path).
 bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
-  if (!g_relayout.load(std::memory_order_relaxed) || g.layout_a || g.layout_b || g.K % 128) return false;
+  if (!g_relayout || g.layout_a || g.layout_b || g.K % 128) return false;
   const double tiles = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
   const double t_gemm_us = (tiles > 256 ? tiles / 256 : 1.0) * (g.K / 128) * 1.5;            // row-major tiled kernel
   auto cost_us = [&](int rows) { return (double)rows * g.K * 0.78125 * 2 / 4.9e6; };         // read + write at 4.9 TB/s
@@ -48,17 +109,8 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
   const bool conv_a = a_first ? conv1 : conv2, conv_b = a_first ? conv2 : conv1;
   auto bytes_of = [&](int rows) { return (((size_t)rows * (g.K / 4 * 3) + 255) & ~(size_t)255) + (((size_t)rows * ((g.K + 511) / 512) * 16 + 255) & ~(size_t)255); };
   const size_t bytes_a = conv_a ? bytes_of(g.M) : 0, bytes_b = conv_b ? bytes_of(g.N) : 0;
-  // never allocate into a stream that is being captured: the caller replays the graph with its own memory plan
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return false;
-  }
-  uint8_t* ws = nullptr;
-  if (hipMallocAsync((void**)&ws, bytes_a + bytes_b, s) != hipSuccess || !ws) {
-    (void)hipGetLastError();
-    return false;
-  }
+  uint8_t* ws = stream_workspace(s, 0, bytes_a + bytes_b);
+  if (!ws) return false;
   mxfp6::GemmArgs t = g;
   uint8_t* pa = ws;
   uint8_t* sa = pa + (((size_t)g.M * (g.K / 4 * 3) + 255) & ~(size_t)255);
@@ -74,8 +126,6 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
   if (conv_a) { t.A = pa; t.As = sa; t.layout_a = 1; }
   if (conv_b) { t.B = pb; t.Bs = sb; t.layout_b = 1; }
   if (e == hipSuccess) e = mxfp6::launch_gemm_tiled(t, s);
-  const hipError_t fe = hipFreeAsync(ws, s);
-  if (e == hipSuccess) e = fe;
   return true;
 }
 
@@ -118,7 +168,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   }
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out, layout_a, layout_b};
   g.ep = ep;
-  const int force = g_force.load(std::memory_order_relaxed);
+  const int force = g_force;
   hipError_t e;
   if (K == 0) {
     e = mxfp6::launch_gemm_generic(g, s);  // act(bias) everywhere: the generic kernel's K loop runs zero times
@@ -192,7 +242,7 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
   // the tiled kernel quantises its accumulators itself; where another kernel is the better one (few rows of A: C is
   // small there) the product goes to an fp32 workspace of the stream-ordered allocator and through the quantiser
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C_packed, M, N, K, fmt_a, fmt_b, false, layout_a, layout_b};
-  const int force = g_force.load(std::memory_order_relaxed);
+  const int force = g_force;
   const bool tiled = K > 0 && mxfp6::gemm_tiled_supports(g) &&
                      (force == 2 || force == 5 || force == 6 || force == 17 ||
                       (force == 0 && !mxfp6::gemm_skinny_preferred(g) && !mxfp6::gemm_mid_preferred(g)));
@@ -203,20 +253,21 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
     if (force != 0 || !relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
     return e == hipSuccess ? MXFP6_OK : (int)e;
   }
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return (int)hipErrorStreamCaptureUnsupported;
+  float* tmp = reinterpret_cast<float*>(stream_workspace(s, 1, (size_t)M * N * 4));
+  if (!tmp) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return (int)hipErrorStreamCaptureUnsupported;
+    }
+    return (int)hipErrorOutOfMemory;
   }
-  float* tmp = nullptr;
-  if (hipMallocAsync((void**)&tmp, (size_t)M * N * 4, s) != hipSuccess || !tmp) return (int)hipGetLastError();
   rc = gemm_common(A, B, As, Bs, tmp, M, N, K, fmt_a, fmt_b, true, layout_a, layout_b, stream, ep);
   if (rc == MXFP6_OK) {
     const hipError_t e = mxfp6::launch_quantize(tmp, 0, (uint8_t*)C_packed, (uint8_t*)C_scale, M, N, fmt_c, MXFP6_LAYOUT_ROW, s);
     rc = e == hipSuccess ? MXFP6_OK : (int)e;
   }
-  const hipError_t fe = hipFreeAsync(tmp, s);
-  return rc != MXFP6_OK ? rc : (fe == hipSuccess ? MXFP6_OK : (int)fe);
+  return rc;
 }
 
 int mxfp6_tile_operand(const void* src, void* dst, int rows, int K, int tile, void* stream) {
@@ -241,11 +292,23 @@ int mxfp6_tile_scales(const void* src, void* dst, int rows, int K, int tile, voi
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
-int mxfp6_set_relayout(int on) { return g_relayout.exchange(on ? 1 : 0); }
+int mxfp6_set_relayout(int on) {
+  const int prev = g_relayout;
+  g_relayout = on ? 1 : 0;
+  return prev;
+}
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 17) return g_force.load();
-  return g_force.exchange(which);
+  if (which < 0 || which > 17) return MXFP6_EINVAL_KERNEL;
+  const int prev = g_force;
+  g_force = which;
+  return prev;
+}
+
+int mxfp6_release_workspaces(void) {
+  const hipError_t a = release_stream_workspaces();
+  const hipError_t b = mxfp6::release_split_workspaces();
+  return a != hipSuccess ? (int)a : (b == hipSuccess ? MXFP6_OK : (int)b);
 }
 
 int mxfp6_quantize(const float* X, void* packed, void* scales, int rows, int K, int fmt, void* stream) {
@@ -284,13 +347,14 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_ENODEVICE: return "mxfp6: the current device is not gfx950 (MI355X)";
     case MXFP6_EINVAL_LAYOUT: return "mxfp6: layout must be 0 (row-major) or 1 (tile-major)";
     case MXFP6_EINVAL_EPILOGUE: return "mxfp6: activation must be 0 (none), 1 (relu), 2 (gelu) or 3 (silu)";
+    case MXFP6_EINVAL_KERNEL: return "mxfp6: unknown kernel code";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 112; }
+int mxfp6_abi_version(void) { return 113; }
 
 #pragma GCC visibility pop
 }  // extern "C"

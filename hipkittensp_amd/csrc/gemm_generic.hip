@@ -14,7 +14,9 @@ __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restr
                                                           typename Out::type* __restrict__ C, int M, int N, int K, int layout_a,
                                                           int layout_b, const Epilogue ep) {
   const int lane = threadIdx.x, h = lane >> 5, r = lane & 31;
-  const long m = (long)blockIdx.y * 32 + r, n = (long)blockIdx.x * 32 + r;
+  // tile rows beyond the 65535 a grid dimension holds continue in blockIdx.z
+  const long m = ((long)blockIdx.z * 65535 + blockIdx.y) * 32 + r, n = (long)blockIdx.x * 32 + r;
+  if (m - r >= M) return;
   const int nkb = K / 32;
   const long rowbytes = (long)nkb * 24;
   const bool mv = m < M, nv = n < N;
@@ -55,7 +57,8 @@ __global__ __launch_bounds__(64) void gemm_generic_kernel(const uint8_t* __restr
 
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  dim3 grid((g.N + 31) / 32, (g.M + 31) / 32);
+  const unsigned tm = (g.M + 31) / 32;
+  dim3 grid((g.N + 31) / 32, tm < 65535 ? tm : 65535, (tm + 65534) / 65535);
   gemm_generic_kernel<FA, FB, Out><<<grid, 64, 0, s>>>(g.A, g.B, g.As, g.Bs, (typename Out::type*)g.C, g.M, g.N, g.K, g.layout_a, g.layout_b, g.ep);
   return hipGetLastError();
 }

@@ -269,7 +269,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
 
 bool gemm_mid_supports(const GemmArgs& g) {
   // B slots are 8 K-tiles; A row-major (M need not be a multiple of 32)
-  if (g.layout_a != 0 || g.M <= 32 || g.M > 512 || g.N <= 0 || g.K < 1024 || g.K % 1024 != 0) return false;
+  if (g.layout_a != 0 || g.M <= 32 || g.M > 512 || g.N <= 0 || g.K < 1024 || g.K % 1024 != 0 || !operands_aligned16(g)) return false;
   if ((long)g.M * (g.K / 4 * 3) >= (1L << 31) || (long)32 * (g.K / 4 * 3) >= (1L << 31)) return false;
   return true;
 }

@@ -271,7 +271,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 
 bool gemm_skinny_supports(const GemmArgs& g) {
   // K % 512: chunks of four K-tiles are whole (three 128-byte lines per row, 16 scale bytes per row)
-  return g.layout_a == 0 && g.M >= 1 && g.M <= 128 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31);
+  return g.layout_a == 0 && g.M >= 1 && g.M <= 128 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) && operands_aligned16(g);
 }
 
 // Automatic choice.  Up to 64 rows of A this kernel is the fastest everywhere (measured against the mid-M kernel: 18 us
@@ -284,12 +284,15 @@ bool gemm_skinny_preferred(const GemmArgs& g) {
 }
 
 // Workspace of the K split: 4 KB of partial tile per (tile, split) and a counter per tile that is zero between
-// launches.  One per stream, allocated at first use and kept: launches on one stream are ordered, so they can share it;
-// launches on different streams get different ones.  (Two graphs captured on one stream and replayed at the same time
-// on different streams would share theirs: replay them on one stream, or switch the split off with geometry 7 - 9.)
-// No allocation is possible while the stream is being captured: a capture without a workspace runs unsplit.
+// launches.  One per (device, stream), taken from the stream-ordered allocator on the caller's stream at the first split
+// launch there (no device-wide synchronisation) and kept until release_split_workspaces(): launches on one stream are
+// ordered, so they can share it; launches on different streams get different ones.  (Two graphs captured on one stream
+// and replayed at the same time on different streams would share theirs: replay them on one stream, or switch the split
+// off with geometry 7 - 9.)  No allocation is possible while the stream is being captured: a capture without a workspace
+// runs unsplit.  At most kWsMax workspaces exist at a time; a further stream runs unsplit.
 namespace {
-constexpr int kWsSlots = 2048, kWsTiles = 1024;  // (tile, split) pairs and tiles a workspace holds
+constexpr int kWsSlots = 512, kWsTiles = 512;  // (tile, split) pairs and tiles a workspace holds (the automatic split never needs more than 256)
+constexpr size_t kWsMax = 64;
 struct SplitWs {
   float* part = nullptr;
   int* cnt = nullptr;
@@ -297,31 +300,59 @@ struct SplitWs {
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, SplitWs> g_ws;
 
+__global__ void clear_counters_kernel(int* p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
 SplitWs split_workspace(hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return {};
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   auto it = g_ws.find({dev, s});
   if (it != g_ws.end()) return it->second;
-  if (g_ws.size() >= 64) return {};  // a process with this many streams runs unsplit on the later ones
+  if (g_ws.size() >= kWsMax) return {};
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
     (void)hipGetLastError();
     return {};
   }
   SplitWs w;
-  if (hipMalloc((void**)&w.part, (size_t)kWsSlots * 4096) != hipSuccess) { (void)hipGetLastError(); return {}; }
-  // cleared on the caller's stream (not being captured here): ordered before the launch that follows, whatever that
-  // stream's relation to the null stream is
-  if (hipMalloc((void**)&w.cnt, kWsTiles * sizeof(int)) != hipSuccess || hipMemsetAsync(w.cnt, 0, kWsTiles * sizeof(int), s) != hipSuccess) {
+  uint8_t* base = nullptr;
+  if (hipMallocAsync((void**)&base, (size_t)kWsSlots * 4096 + kWsTiles * sizeof(int), s) != hipSuccess || !base) {
     (void)hipGetLastError();
-    (void)hipFree(w.part);
+    return {};
+  }
+  w.part = reinterpret_cast<float*>(base);
+  w.cnt = reinterpret_cast<int*>(base + (size_t)kWsSlots * 4096);
+  // cleared on the caller's stream: ordered before the launch that follows
+  clear_counters_kernel<<<(kWsTiles + 255) / 256, 256, 0, s>>>(w.cnt, kWsTiles);
+  if (hipGetLastError() != hipSuccess) {
+    (void)hipFreeAsync(base, s);
     return {};
   }
   g_ws[{dev, s}] = w;
   return w;
 }
+
 }  // namespace
+
+hipError_t release_split_workspaces() {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  if (g_ws.empty()) return hipSuccess;
+  int cur = 0;
+  (void)hipGetDevice(&cur);
+  hipError_t first = hipSuccess;
+  for (auto& kv : g_ws) {
+    // stream-ordered: the memory goes back once the work queued on that stream so far has finished with it
+    (void)hipSetDevice(kv.first.first);
+    const hipError_t e = hipFreeAsync(kv.second.part, kv.first.second);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  }
+  g_ws.clear();
+  (void)hipSetDevice(cur);
+  return first;
+}
 
 // Geometry.  Few rows of B (N / 32 workgroups would leave CUs idle): a workgroup takes 16 rows of B, and the K range
 // is split between 2, 4 or 8 workgroups while that still fits the CUs and leaves every wave kMinChunks chunks.  More
@@ -331,9 +362,11 @@ SplitWs split_workspace(hipStream_t s) {
 // streams a longer part of K: measured 5 - 13 % at N = 14336 .. 28672, K = 4096 .. 8192, nothing beyond N = 32768).
 // skinny_geometry: 1 - 3 fix the workgroup shape without a split; 4 + 3 * b + log2(split) - 1 (b = 0: 32 rows of B,
 // b = 1: 16 rows) fixes both; 10 = two waves per workgroup.
-template <int FA, int FB, typename Out>
-static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  typedef typename Out::type T;
+struct SkinnyPlan {
+  int geo, want;   // workgroup shape (1: 32 rows of B, 2: 16 rows, 3: half the waves, 5: two waves) and wanted K split
+  unsigned tiles;  // tiles of C (one arrival counter each when K is split)
+};
+static SkinnyPlan skinny_plan(const GemmArgs& g) {
   const unsigned wgs32 = (g.N + 31) / 32;
   const int nchunks = g.K / 512, nw = g.M <= 16 ? 8 : 6;
   int geo, want = 1;
@@ -354,9 +387,17 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     if (geo != 3)
       while (want < 8 && tiles * want * 2 <= 256 && nchunks / (want * 2) >= kMinChunks * nw) want *= 2;
   }
+  return {geo, want, geo == 2 ? (unsigned)(g.N + 15) / 16 : wgs32};
+}
+
+template <int FA, int FB, typename Out>
+static hipError_t launch(const GemmArgs& g, hipStream_t s) {
+  typedef typename Out::type T;
+  const SkinnyPlan plan = skinny_plan(g);
+  const int geo = plan.geo, want = plan.want;
   int nsplit = 1;
   SplitWs ws;
-  const unsigned tiles = geo == 2 ? (g.N + 15) / 16 : wgs32;
+  const unsigned tiles = plan.tiles;
   if (want > 1 && tiles <= (unsigned)kWsTiles && tiles * want <= (unsigned)kWsSlots) {
     ws = split_workspace(s);
     if (ws.part) nsplit = want;

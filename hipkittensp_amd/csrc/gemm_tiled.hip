@@ -49,7 +49,7 @@
 
 namespace mxfp6 {
 
-int g_tiled_walk = 1;  // 0: always one workgroup per output tile (development switch)
+static constexpr int g_tiled_walk = 1;  // 0 would launch one workgroup per output tile everywhere (no walk)
 
 constexpr int kBK = 128;  // the tile has 256 (TM = 4) or 128 (TM = 2) rows of A and 256 (TN = 2) or 128 (TN = 1) rows of B
 constexpr int kGroupM = 4;          // tile rows per raster group
@@ -629,7 +629,7 @@ bool gemm_tiled_supports(const GemmArgs& g) {
   // any M; N % 8 keeps every run of 8 bf16 outputs whole and aligned; K in whole K-tiles; 32-bit byte
   // offsets inside one tile's operand rows and inside one tile's rows of C
   return g.M > 0 && g.N > 0 && g.K > 0 && g.N % 8 == 0 && g.K % kBK == 0 && (long)256 * (g.K / 4 * 3) < (1L << 31) &&
-         (long)256 * g.N * 4 < (1L << 31) && g.M <= 65535 * 128 && ((uintptr_t)g.C % 16) == 0;
+         (long)256 * g.N * 4 < (1L << 31) && g.M <= 65535 * 128 && ((uintptr_t)g.C % 16) == 0 && operands_aligned16(g);
 }
 
 static int cu_count() {

@@ -21,6 +21,11 @@ struct GemmArgs {
   int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output
 };
 
+// the LDS-staged kernels fetch operands and scales 16 bytes per lane: all four tensors must be 16-byte aligned
+inline bool operands_aligned16(const GemmArgs& g) {
+  return (((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.As | (uintptr_t)g.Bs) & 15) == 0;
+}
+
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
@@ -32,6 +37,7 @@ hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
 bool gemm_skinny_preferred(const GemmArgs& g);  // over the mid-M kernel, by shape
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
+hipError_t release_split_workspaces();             // returns every K-split workspace to the stream-ordered allocator
 hipError_t launch_quantize(const void* X, int x_bf16, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);
 hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);
 hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);

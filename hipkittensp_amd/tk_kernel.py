@@ -263,3 +263,8 @@ def set_relayout(on: bool) -> bool:
 def set_kernel(which: int) -> int:
     """Force a kernel (KERNEL_*) for measurement / tests; returns the previous setting."""
     return _lib.lib().mxfp6_set_kernel(int(which))
+
+
+def release_workspaces() -> None:
+    """Return every workspace the library holds to the stream-ordered allocator."""
+    _lib.check(_lib.lib().mxfp6_release_workspaces(), "release_workspaces")

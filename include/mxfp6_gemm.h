@@ -16,8 +16,31 @@
  *   - tensor -> raw pointer conversion at the boundary   include/pyutils/pyutils.cuh:15-72
  * All pointers are DEVICE pointers.  All functions return 0 on success, a negative MXFP6_E* code
  * for rejected arguments (nothing launched), or a positive hipError_t value if the runtime failed.
- * No function allocates device memory or synchronises; work is queued on `hip_stream`
- * (a hipStream_t; NULL = the null stream).
+ * Work is queued on `hip_stream` (a hipStream_t; NULL = the null stream); no function synchronises the
+ * device or the stream.
+ *
+ * Device memory.  Three entry-point families take a workspace from the stream-ordered allocator
+ * (hipMallocAsync on `hip_stream`), at most once per (device, stream) and size class, and keep it until
+ * mxfp6_release_workspaces():
+ *   - the gemm entry points on large row-major problems (re-layout pre-pass, see mxfp6_set_relayout):
+ *     up to 0.78 (M + N) K bytes;
+ *   - mxfp6_gemm_fused_fp6 on shapes the LDS-tiled kernel does not run: 4 M N bytes;
+ *   - the gemm entry points on decode shapes whose K range is split between workgroups (M <= 32, N <= 2048,
+ *     K >= 24576): 2 MB.
+ * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K split are left out
+ * (same results, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
+ * hipErrorStreamCaptureUnsupported where it would need a new one.
+ *
+ * Alignment.  Pointers are accepted from 4-byte alignment on (C: its element size).  The fast kernels
+ * fetch 16 bytes per lane: they run when A_packed, B_packed, both scale tensors and C are 16-byte aligned
+ * (any tensor PyTorch allocates is); otherwise the call is served by the generic kernel, with the same
+ * results and a fraction of the speed.
+ *
+ * Accuracy.  Products of dequantised values are exact in fp32; with an e2m3 operand on either side the
+ * accumulators agree with an fp64 dequantise-and-matmul to fp32 rounding (relative error < 1e-6 of the
+ * result's range).  e3m2 x e3m2 is weaker: the scaled MFMA's internal sum drops low-order bits of
+ * wide-ranging products, giving an error of up to 1e-4 of sum_k |a_mk| |b_nk| per output, which is above
+ * 2e-3 of the result only where the sum cancels to less than 5 % of its terms.
  */
 #ifndef MXFP6_GEMM_H
 #define MXFP6_GEMM_H
@@ -40,6 +63,7 @@ extern "C" {
 #define MXFP6_ENODEVICE (-5)    /* current device is not gfx950                                */
 #define MXFP6_EINVAL_LAYOUT (-6) /* layout code is not MXFP6_LAYOUT_ROW / MXFP6_LAYOUT_TILE    */
 #define MXFP6_EINVAL_EPILOGUE (-7) /* activation code is not one of MXFP6_ACT_*                */
+#define MXFP6_EINVAL_KERNEL (-9) /* mxfp6_set_kernel: unknown kernel code                        */
 
 /* Activations of mxfp6_gemm_fused. */
 #define MXFP6_ACT_NONE 0
@@ -52,7 +76,8 @@ extern "C" {
  * (analysis/bf16_gemm/mi325x/kernel_8192.cpp:227-231, distributed-kernels/bf16_gemm/kernel.cpp:247-265)
  * for packed-fp6 operands with E8M0 block scales.
  *   A_packed [M, 3K/4] u8, B_packed [N, 3K/4] u8, A_scale [M, K/32] u8, B_scale [N, K/32] u8,
- *   C [M, N] bf16 row-major.  K % 32 == 0.  A_packed/B_packed 4-byte aligned, C 2-byte aligned.
+ *   C [M, N] bf16 row-major.  K % 32 == 0.  A_packed/B_packed 4-byte aligned, C 2-byte aligned (16-byte
+ *   alignment of all five tensors reaches the fast kernels, see "Alignment" above).
  *   M == 0 or N == 0 is a successful no-op; K == 0 writes zeros.
  */
 int mxfp6_gemm(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, void *C_bf16,
@@ -69,8 +94,9 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
                       float *C_f32, int M, int N, int K, int fmt_a, int fmt_b, void *hip_stream);
 
 /*
- * Kernel selection override for measurement and tests.  Returns the previous value.  A forced kernel that cannot run the
- * given shape makes the gemm calls return MXFP6_EINVAL_SHAPE.
+ * Kernel selection override for measurement and tests, per calling thread (it affects the gemm calls this thread
+ * makes afterwards, and nobody else's).  Returns the previous value, or MXFP6_EINVAL_KERNEL for an unknown code.
+ * A forced kernel that cannot run the given shape makes the gemm calls return MXFP6_EINVAL_SHAPE.
  *    0  automatic (default)
  *    1  generic one-wave-per-tile kernel (any shape)
  *    2  LDS-tiled MFMA kernel (needs N % 8 == 0, K % 128 == 0), tile shape by how it fills the GPU;
@@ -78,7 +104,7 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *    3  skinny-M streaming kernel (needs M <= 128, K % 512 == 0), workgroup geometry by N and K;
  *       7 / 8 / 9: 32 rows of B per workgroup / 16 rows / 32 rows and half the waves, none of them splitting K;
  *       10 / 11 / 12: 32 rows of B, the K range split between 2 / 4 / 8 workgroups; 13 / 14 / 15: the same with 16 rows
- *       (the split takes a workspace of 8 MB per stream at first use; without one, e.g. first use under stream capture,
+ *       (the split takes a workspace of 2 MB per stream at first use; without one, e.g. first use under stream capture,
  *       the launch runs unsplit); 16: 32 rows of B and two waves per workgroup
  *    4  mid-M kernel (needs 32 < M <= 512, K % 1024 == 0, row-major A)
  * No counterpart in the reference, whose shapes are compile-time constants per binary
@@ -87,13 +113,12 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
 int mxfp6_set_kernel(int which);
 
 /*
- * Re-layout pre-pass of the automatic path (on by default; returns the previous setting).  For large row-major
- * problems the gemm calls first copy one operand or both (with their scales) into tile-major order in a
- * workspace taken from, and returned to, the stream-ordered allocator (hipMallocAsync / hipFreeAsync on the
- * caller's stream), because the tiled kernel is bound by L2 requests on row-major operands; results are
- * bit-identical.  It is skipped by itself on a stream that is being captured.  Switch it off to measure the
- * row-major kernel itself or where the caller cannot tolerate a stream-ordered allocation.  No counterpart in
- * the reference.
+ * Re-layout pre-pass of the automatic path (on by default; per calling thread; returns the previous setting).
+ * For large row-major problems the gemm calls first copy one operand or both (with their scales) into
+ * tile-major order in this stream's workspace (hipMallocAsync on the caller's stream the first time, kept
+ * until mxfp6_release_workspaces()), because the tiled kernel is bound by L2 requests on row-major operands;
+ * results are bit-identical.  On a stream that is being captured it runs only if the workspace exists already.
+ * Switch it off to measure the row-major kernel itself.  No counterpart in the reference.
  */
 int mxfp6_set_relayout(int on);
 
@@ -186,6 +211,13 @@ int mxfp6_gemm_fused_fp6(const void *A_packed, const void *B_packed, const void 
                          void *C_packed, void *C_scale, int M, int N, int K, int fmt_a, int fmt_b, int layout_a,
                          int layout_b, int fmt_c, const void *bias, int bias_bf16, const float *row_scale,
                          const float *col_scale, int activation, void *hip_stream);
+
+/*
+ * Returns every workspace this library holds (see "Device memory" above) to the stream-ordered allocator, each in
+ * the order of the stream it was taken on; later calls allocate again on demand.  No counterpart in the reference,
+ * which allocates nothing behind its launcher.
+ */
+int mxfp6_release_workspaces(void);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

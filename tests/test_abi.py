@@ -31,7 +31,7 @@ def built_lib():
 def test_header_declares_the_operator():
     names = _declared_functions()
     for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_gemm_fused", "mxfp6_gemm_fused_fp6", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_quantize_bf16", "mxfp6_tile_operand", "mxfp6_tile_scales",
-                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout"):
+                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout", "mxfp6_release_workspaces"):
         assert want in names
 
 
@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 112
+    assert L.mxfp6_abi_version() == 113
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -97,6 +97,21 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     assert L.mxfp6_tile_scales(one, one, 32, 96, 1, None) == -2
     assert L.mxfp6_tile_scales(None, one, 32, 128, 1, None) == -1
     assert L.mxfp6_tile_scales(one, one, 0, 128, 1, None) == 0
+    L.mxfp6_strerror.restype = ctypes.c_char_p
+    L.mxfp6_strerror.argtypes = [ci]
+    # kernel override: per thread, unknown codes are an error
+    L.mxfp6_set_kernel.restype = ci
+    L.mxfp6_set_kernel.argtypes = [ci]
+    assert L.mxfp6_set_kernel(99) == -9 and L.mxfp6_set_kernel(-1) == -9
+    assert L.mxfp6_set_kernel(2) == 0
+    import threading
+    seen = []
+    th = threading.Thread(target=lambda: seen.append(L.mxfp6_set_kernel(0)))
+    th.start(); th.join()
+    assert seen == [0]                      # another thread does not see this thread's override
+    assert L.mxfp6_set_kernel(0) == 2
+    L.mxfp6_release_workspaces.restype = ci
+    assert L.mxfp6_release_workspaces() == 0   # nothing held: no HIP call is made
 
 
 def test_python_operator_rejects_like_the_reference():
