@@ -53,6 +53,8 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_tile_scales.argtypes = [vp, vp, ci, ci, ci, vp]
         L.mxfp6_set_kernel.restype = ci
         L.mxfp6_set_kernel.argtypes = [ci]
+        L.mxfp6_gemm_noalloc.restype = ci
+        L.mxfp6_gemm_noalloc.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.mxfp6_release_workspaces.restype = ci
         L.mxfp6_release_workspaces.argtypes = []
         L.mxfp6_strerror.restype = ctypes.c_char_p

@@ -3,6 +3,7 @@
 // caller's stream and all kept per (device, stream) until mxfp6_release_workspaces(): the workspace of the re-layout
 // pre-pass (relayout_then_tiled; mxfp6_set_relayout(0) switches it off), the fp32 workspace of mxfp6_gemm_fused_fp6
 // on shapes the tiled kernel does not run, and the K-split workspace of the skinny kernel (gemm_skinny.hip).
+// mxfp6_gemm_noalloc allocates nothing.
 #include "../../include/mxfp6_gemm.h"
 
 #include <map>
@@ -94,7 +95,7 @@ int check_device() {
 // fewer rows.  The workspace is this stream's (stream_workspace: allocated once, kept).  Returns false when no
 // pre-pass pays or it cannot run (then the caller launches the row-major path).
 bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
-  if (!g_relayout || g.layout_a || g.layout_b || g.K % 128) return false;
+  if (!g_relayout || g.no_alloc || g.layout_a || g.layout_b || g.K % 128) return false;
   const double tiles = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
   const double t_gemm_us = (tiles > 256 ? tiles / 256 : 1.0) * (g.K / 128) * 1.5;            // row-major tiled kernel
   auto cost_us = [&](int rows) { return (double)rows * g.K * 0.78125 * 2 / 4.9e6; };         // read + write at 4.9 TB/s
@@ -155,7 +156,8 @@ int check_gemm_args(const void* A, const void* B, const void* As, const void* Bs
 }
 
 int gemm_common(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
-                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream, const mxfp6::Epilogue& ep = mxfp6::Epilogue()) {
+                int fmt_b, bool f32out, int layout_a, int layout_b, void* stream, const mxfp6::Epilogue& ep = mxfp6::Epilogue(),
+                int no_alloc = 0, int force_split = 0) {
   bool empty;
   int rc = check_gemm_args(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, f32out ? 3 : 1, layout_a, layout_b, ep, &empty);
   if (rc || empty) return rc;
@@ -168,8 +170,11 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   }
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out, layout_a, layout_b};
   g.ep = ep;
-  const int force = g_force;
+  g.no_alloc = no_alloc, g.force_split = force_split;
+  const int force = no_alloc ? 0 : g_force;  // the entry point that allocates nothing takes no override
   hipError_t e;
+  if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
+  if (no_alloc && (force_split || mxfp6::gemm_skinny_preferred(g)) && mxfp6::gemm_skinny_supports(g) && !mxfp6::gemm_skinny_scratch_fits(g)) return MXFP6_ESCRATCH;
   if (K == 0) {
     e = mxfp6::launch_gemm_generic(g, s);  // act(bias) everywhere: the generic kernel's K loop runs zero times
   } else if (force == 1) {
@@ -185,7 +190,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 4) {
     if (!mxfp6::gemm_mid_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_mid(g, s);
-  } else if (mxfp6::gemm_skinny_preferred(g)) {
+  } else if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) {
     e = mxfp6::launch_gemm_skinny(g, s);
   } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
     e = mxfp6::launch_gemm_mid(g, s);
@@ -305,6 +310,12 @@ int mxfp6_set_kernel(int which) {
   return prev;
 }
 
+int mxfp6_gemm_noalloc(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a,
+                       int fmt_b, int nsplit, void* stream) {
+  if (nsplit != 0 && nsplit != 1 && nsplit != 2 && nsplit != 4 && nsplit != 8) return MXFP6_EINVAL_SHAPE;
+  return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, 0, 0, stream, mxfp6::Epilogue(), 1, nsplit);
+}
+
 int mxfp6_release_workspaces(void) {
   const hipError_t a = release_stream_workspaces();
   const hipError_t b = mxfp6::release_split_workspaces();
@@ -347,6 +358,7 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_ENODEVICE: return "mxfp6: the current device is not gfx950 (MI355X)";
     case MXFP6_EINVAL_LAYOUT: return "mxfp6: layout must be 0 (row-major) or 1 (tile-major)";
     case MXFP6_EINVAL_EPILOGUE: return "mxfp6: activation must be 0 (none), 1 (relu), 2 (gelu) or 3 (silu)";
+    case MXFP6_ESCRATCH: return "mxfp6: the K split of this call needs more than the static scratch memory holds (256 partial tiles: rows of C tiles times nsplit)";
     case MXFP6_EINVAL_KERNEL: return "mxfp6: unknown kernel code";
     default: break;
   }

@@ -33,6 +33,12 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
+// Scratch memory of mxfp6_gemm_noalloc: kScratchSlots partial tiles of 4 KB (one per (tile, split) pair of a K split) followed by
+// kScratchTiles arrival counters.  In host code this name is only a handle for hipGetSymbolAddress; kernels get the device
+// address that call returns.
+constexpr int kScratchSlots = 256, kScratchTiles = 256;
+static __device__ __align__(256) unsigned char scratch[kScratchSlots * 4096 + kScratchTiles * 4];
+
 namespace mxfp6 {
 
 namespace {
@@ -335,6 +341,27 @@ SplitWs split_workspace(hipStream_t s) {
   return w;
 }
 
+// The scratch memory of the entry point that allocates nothing (launch_gemm_skinny with GemmArgs::no_alloc): partial
+// tiles and counters of the K split live in the array `scratch` at the top of this file, of which every GPU holds its
+// own copy at its own address.  The address is looked up once per device, with that device current, and only that
+// pointer is handed to kernels.
+unsigned char* g_scratch_ptr[64] = {};
+hipError_t scratch_of_current_device(unsigned char** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
+}
 }  // namespace
 
 hipError_t release_split_workspaces() {
@@ -380,6 +407,10 @@ static SkinnyPlan skinny_plan(const GemmArgs& g) {
     want = 2 << ((g.skinny_geometry - 4) % 3);
   } else if (g.skinny_geometry) {
     geo = g.skinny_geometry;
+  } else if (g.force_split) {
+    // the caller fixes the split (1, 2, 4 or 8); the workgroup shape follows N as in the automatic choice for split shapes
+    geo = wgs32 <= 128 ? 2 : 1;
+    want = g.force_split;
   } else {
     geo = wgs32 <= 128 ? 2 : wgs32 <= 256 ? 1 : g.M <= 16 && wgs32 <= 1024 && nchunks <= 16 ? 5 : 3;
     constexpr int kMinChunks = 3;  // measured: below this the 2.5 us of the second phase outweigh the wider stream
@@ -390,6 +421,12 @@ static SkinnyPlan skinny_plan(const GemmArgs& g) {
   return {geo, want, geo == 2 ? (unsigned)(g.N + 15) / 16 : wgs32};
 }
 
+// Does the K split this call would use fit the scratch array of the entry point that allocates nothing?
+bool gemm_skinny_scratch_fits(const GemmArgs& g) {
+  const SkinnyPlan p = skinny_plan(g);
+  return p.want <= 1 || (p.tiles <= (unsigned)kScratchTiles && p.tiles * p.want <= (unsigned)kScratchSlots);
+}
+
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   typedef typename Out::type T;
@@ -398,7 +435,22 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   int nsplit = 1;
   SplitWs ws;
   const unsigned tiles = plan.tiles;
-  if (want > 1 && tiles <= (unsigned)kWsTiles && tiles * want <= (unsigned)kWsSlots) {
+  if (g.no_alloc) {
+    // nothing is allocated: the split uses this device's scratch array, whose counters are cleared by a small kernel in
+    // front of the launch (the array keeps whatever the previous call left)
+    if (want > 1) {
+      if (tiles > (unsigned)kScratchTiles || tiles * want > (unsigned)kScratchSlots) return hipErrorInvalidValue;  // the entry point checked this already
+      unsigned char* base = nullptr;
+      const hipError_t e = scratch_of_current_device(&base);
+      if (e != hipSuccess) return e;
+      ws.part = reinterpret_cast<float*>(base);
+      ws.cnt = reinterpret_cast<int*>(base + (size_t)kScratchSlots * 4096);
+      clear_counters_kernel<<<(tiles + 255) / 256, 256, 0, s>>>(ws.cnt, (int)tiles);
+      const hipError_t ce = hipGetLastError();
+      if (ce != hipSuccess) return ce;
+      nsplit = want;
+    }
+  } else if (want > 1 && tiles <= (unsigned)kWsTiles && tiles * want <= (unsigned)kWsSlots) {
     ws = split_workspace(s);
     if (ws.part) nsplit = want;
   }

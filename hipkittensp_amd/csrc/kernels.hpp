@@ -19,6 +19,8 @@ struct GemmArgs {
   Epilogue ep;                     // fused bias / scales / activation (all optional)
   uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
   int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output
+  int no_alloc = 0;                // skinny kernel: the K split keeps its partial tiles in the library's static scratch array instead of an allocated workspace
+  int force_split = 0;             // skinny kernel, M <= 32: split K between this many workgroups (1, 2, 4, 8); 0 = by shape
 };
 
 // the LDS-staged kernels fetch operands and scales 16 bytes per lane: all four tensors must be 16-byte aligned
@@ -37,6 +39,7 @@ hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
 bool gemm_skinny_preferred(const GemmArgs& g);  // over the mid-M kernel, by shape
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
+bool gemm_skinny_scratch_fits(const GemmArgs& g);  // no_alloc: the K split this call would use fits the static scratch array
 hipError_t release_split_workspaces();             // returns every K-split workspace to the stream-ordered allocator
 hipError_t launch_quantize(const void* X, int x_bf16, uint8_t* packed, uint8_t* scales, int rows, int K, int fmt, int layout, hipStream_t s);
 hipError_t launch_tile_operand(const uint8_t* src, uint8_t* dst, int rows, int K, int tile, hipStream_t s);

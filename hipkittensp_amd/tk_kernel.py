@@ -265,6 +265,37 @@ def set_kernel(which: int) -> int:
     return _lib.lib().mxfp6_set_kernel(int(which))
 
 
+def dispatch_micro_noalloc(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, nsplit: int = 0) -> None:
+    """dispatch_micro for callers that cannot allocate device memory (graph capture, tight serving loops): row-major
+    operands, bfloat16 C, no allocation of any kind behind the call.  nsplit = 0 picks kernel and K split like
+    dispatch_micro (bit-identical result); 1, 2, 4 or 8 fixes the K split of the skinny kernel (M <= 32, K % 512 == 0),
+    whose partial tiles live in the library's static scratch memory (256 partial tiles: a RuntimeError says so when a
+    split does not fit)."""
+    import torch
+
+    A, B = _as_tensor(A, "A"), _as_tensor(B, "B")
+    A_scale, B_scale = _as_tensor(A_scale, "A_scale"), _as_tensor(B_scale, "B_scale")
+    C = _as_tensor(C, "C")
+    for t, name in ((A, "A"), (B, "B"), (A_scale, "A_scale"), (B_scale, "B_scale")):
+        if t.dtype != torch.uint8:
+            raise RuntimeError(f"{name}: expected dtype uint8, got {t.dtype}")
+    if C.dtype != torch.bfloat16:
+        raise RuntimeError(f"C: expected dtype bfloat16, got {C.dtype}")
+    M, wa = _rows_cols(A, "A")
+    N, wb = _rows_cols(B, "B")
+    if wa != wb or wa % 24:
+        raise RuntimeError(f"A and B: packed widths {wa} and {wb} must agree and be whole 32-element blocks (24 bytes)")
+    K = wa // 3 * 4
+    if _rows_cols(A_scale, "A_scale") != (M, K // 32) or _rows_cols(B_scale, "B_scale") != (N, K // 32) or _rows_cols(C, "C") != (M, N):
+        raise RuntimeError("A_scale / B_scale / C: shapes must be [M, K/32], [N, K/32] and [M, N]")
+    if len({t.device for t in (A, B, A_scale, B_scale, C)}) != 1:
+        raise RuntimeError("all tensors must be on one device")
+    with _on_device(C.device):
+        rc = _lib.lib().mxfp6_gemm_noalloc(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
+                                           fmt_a, fmt_b, int(nsplit), _stream())
+    _lib.check(rc, "dispatch_micro_noalloc")
+
+
 def release_workspaces() -> None:
     """Return every workspace the library holds to the stream-ordered allocator."""
     _lib.check(_lib.lib().mxfp6_release_workspaces(), "release_workspaces")

@@ -29,7 +29,7 @@
  *     K >= 24576): 2 MB.
  * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K split are left out
  * (same results, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
- * hipErrorStreamCaptureUnsupported where it would need a new one.
+ * hipErrorStreamCaptureUnsupported where it would need a new one.  mxfp6_gemm_noalloc never allocates.
  *
  * Alignment.  Pointers are accepted from 4-byte alignment on (C: its element size).  The fast kernels
  * fetch 16 bytes per lane: they run when A_packed, B_packed, both scale tensors and C are 16-byte aligned
@@ -63,6 +63,7 @@ extern "C" {
 #define MXFP6_ENODEVICE (-5)    /* current device is not gfx950                                */
 #define MXFP6_EINVAL_LAYOUT (-6) /* layout code is not MXFP6_LAYOUT_ROW / MXFP6_LAYOUT_TILE    */
 #define MXFP6_EINVAL_EPILOGUE (-7) /* activation code is not one of MXFP6_ACT_*                */
+#define MXFP6_ESCRATCH (-8)     /* mxfp6_gemm_noalloc: the requested K split does not fit the static scratch memory */
 #define MXFP6_EINVAL_KERNEL (-9) /* mxfp6_set_kernel: unknown kernel code                        */
 
 /* Activations of mxfp6_gemm_fused. */
@@ -218,6 +219,24 @@ int mxfp6_gemm_fused_fp6(const void *A_packed, const void *B_packed, const void 
  * which allocates nothing behind its launcher.
  */
 int mxfp6_release_workspaces(void);
+
+/*
+ * mxfp6_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): same operands, same bf16 result, and no allocation of any kind.  It has no
+ * counterpart in the reference.  The re-layout pre-pass is left out, and the K split of decode shapes keeps its partial
+ * tiles (4 KB per tile of C and split) and arrival counters in a static array of the library's device code: 1 MB + 1 KB
+ * per GPU, held until the process ends, holding 256 partial tiles and 256 counters.
+ *   nsplit = 0: kernel and split chosen as mxfp6_gemm chooses them (never more than 256 partial tiles) -- the result is
+ *               bit-identical to mxfp6_gemm's;
+ *   nsplit = 1, 2, 4, 8: the skinny kernel with K split between that many workgroups per tile of C (needs M <= 32,
+ *               K % 512 == 0; MXFP6_EINVAL_SHAPE otherwise).  A tile of C is 16 columns for N <= 4096 and 32 beyond:
+ *               ceil(N / 16 or 32) * nsplit must not exceed 256, else MXFP6_ESCRATCH and nothing is launched.
+ * Every call on a GPU shares that GPU's array: the counters are cleared by a small kernel in front of each split launch,
+ * and calls that overlap in time on one GPU (two streams, two threads) race on it -- serialise them, or give the
+ * concurrent ones nsplit = 1.
+ */
+int mxfp6_gemm_noalloc(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale,
+                       void *C_bf16, int M, int N, int K, int fmt_a, int fmt_b, int nsplit, void *hip_stream);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

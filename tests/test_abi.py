@@ -31,7 +31,7 @@ def built_lib():
 def test_header_declares_the_operator():
     names = _declared_functions()
     for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_gemm_fused", "mxfp6_gemm_fused_fp6", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_quantize_bf16", "mxfp6_tile_operand", "mxfp6_tile_scales",
-                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout", "mxfp6_release_workspaces"):
+                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout", "mxfp6_gemm_noalloc", "mxfp6_release_workspaces"):
         assert want in names
 
 
@@ -97,8 +97,16 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     assert L.mxfp6_tile_scales(one, one, 32, 96, 1, None) == -2
     assert L.mxfp6_tile_scales(None, one, 32, 128, 1, None) == -1
     assert L.mxfp6_tile_scales(one, one, 0, 128, 1, None) == 0
+    # the entry point that allocates nothing: the same checks, and only the splits the skinny kernel has
+    L.mxfp6_gemm_noalloc.restype = ci
+    L.mxfp6_gemm_noalloc.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+    assert L.mxfp6_gemm_noalloc(one, one, one, one, one, 16, 16, 48, 2, 2, 0, None) == -2
+    assert L.mxfp6_gemm_noalloc(one, one, one, one, one, 16, 16, 512, 2, 2, 3, None) == -2
+    assert L.mxfp6_gemm_noalloc(None, one, one, one, one, 16, 16, 512, 2, 2, 0, None) == -1
+    assert L.mxfp6_gemm_noalloc(one, one, one, one, one, 0, 16, 512, 2, 2, 8, None) == 0
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ci]
+    assert b"scratch" in L.mxfp6_strerror(-8)
     # kernel override: per thread, unknown codes are an error
     L.mxfp6_set_kernel.restype = ci
     L.mxfp6_set_kernel.argtypes = [ci]
