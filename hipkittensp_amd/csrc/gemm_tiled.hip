@@ -31,8 +31,11 @@
 // Any assignment of K-blocks to lane halves is legal as long as both operands use the same one.
 //
 // E8M0 scales ride in LDS too: 16 bytes per row cover four K-tiles, fetched by one dwordx4 direct
-// load per 64 rows per four K-tiles; a lane reads the 2 bytes it needs with ds_read_u16 and the MFMA's
-// op_sel picks byte 0 / byte 1.
+// load per 64 rows per four K-tiles.  A lane needs bytes 2h and 2h+1 (h = lane / 32) of each K-tile's four: every
+// second K-tile it reads the eight bytes of two K-tiles (ds_read_b64) and v_perm_b32 gathers its four into one
+// register, of which the MFMAs' op_sel picks bytes 0, 1 (first K-tile of the pair) and 2, 3 (second).  (A
+// ds_read_u16 per operand tile and K-tile, as before, was 30 % of all LDS cycles in bank conflicts and cost 16 %
+// more shader clocks per GEMM.)
 //
 // Schedule: 8-wave ping-pong (the reference's pattern, analysis/bf16_gemm/mi325x/kernel_8192.cpp:75-153):
 // waves 0-3 and waves 4-7 (one of each per SIMD) run half a K-tile out of phase, so that on every SIMD
@@ -223,8 +226,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     a_rd[c] = (wm * (TM * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
     b_rd[c] = kAStage + (wn * (TN * 32) + r32) * 96 + ((3 * h + c) ^ sw) * 16;
   }
-  const int sa_rd = kScaleBase + (wm * (TM * 32) + r32) * 16 + 2 * h;
-  const int sb_rd = kScaleBase + kScStage + (wn * (TN * 32) + r32) * 16 + 2 * h;
+  const int sa_rd = kScaleBase + (wm * (TM * 32) + r32) * 16;
+  const int sb_rd = kScaleBase + kScStage + (wn * (TN * 32) + r32) * 16;
 
   v16f acc[TM][TN];  // never zeroed: the first K-tile of an output tile multiplies into a zero C operand
 
@@ -257,10 +260,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // a lane's 48 bytes of one 32-row tile live in 12 consecutive VGPRs: dwords 0-5 are the operand of the
   // first MFMA, 6-11 of the second
   v12i fa[TM], fb[TN];
-  int sca[TM], scb[TN];
-  auto read_tile = [&](int stage, int sc_off) __attribute__((always_inline)) {
+  int sca[TM], scb[TN];  // this lane's scale bytes of a pair of K-tiles: bytes 0, 1 the first K-tile's two blocks, 2, 3 the second's
+  // KM: K-tile modulo 4.  sc_off: the scale buffer of the K-tile's group of four.
+  auto read_tile = [&]<int KM>(int stage, int sc_off) __attribute__((always_inline)) {
     const uint8_t* st = smem + stage * kStage;
-    const uint8_t* sc = smem + sc_off;
+    const uint8_t* sc = smem + sc_off + (KM >> 1) * 8;
+    // byte selector of v_perm_b32 for this lane's half, recomputed here instead of living in a register through the loop
+    uint32_t sc_sel = 0;
+    if ((KM & 1) == 0) {
+      int lid = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+      asm volatile("" : "+v"(lid));
+      sc_sel = lid & 32 ? 0x07060302u : 0x05040100u;
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
 #pragma unroll
@@ -269,7 +280,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
         for (int e = 0; e < 4; e++) fb[j][4 * c + e] = p[e];
       }
-      scb[j] = *reinterpret_cast<const uint16_t*>(sc + sb_rd + j * 512);
+      if ((KM & 1) == 0) {
+        const v2i raw = *reinterpret_cast<const v2i*>(sc + sb_rd + j * 512);
+        scb[j] = __builtin_amdgcn_perm(raw[1], raw[0], sc_sel);
+      }
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
@@ -279,14 +293,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
         for (int e = 0; e < 4; e++) fa[i][4 * c + e] = p[e];
       }
-      sca[i] = *reinterpret_cast<const uint16_t*>(sc + sa_rd + i * 512);
+      if ((KM & 1) == 0) {
+        const v2i raw = *reinterpret_cast<const v2i*>(sc + sa_rd + i * 512);
+        sca[i] = __builtin_amdgcn_perm(raw[1], raw[0], sc_sel);
+      }
     }
   };
   // first K-block of every lane for all tiles, then the second: two MFMAs into the same accumulator
   // are TM*TN instructions apart.  First source = B rows (index n), second = A rows (index m): a lane
   // ends up owning 4 consecutive n of row m = lane % 32, four times.  FIRST: the K-tile opens an output tile,
   // so the first MFMA into every accumulator takes zero as its C operand.  between(i) runs after the i-th MFMA.
-  auto mma_tile = [&]<bool FIRST>(auto&& between) __attribute__((always_inline)) {
+  auto mma_tile = [&]<bool FIRST, int KM>(auto&& between) __attribute__((always_inline)) {
+    constexpr int S0 = 2 * (KM & 1), S1 = S0 + 1;  // op_sel: which byte of the scale registers
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < TM; i++) {
@@ -294,7 +312,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const v8i b0 = __builtin_shufflevector(fb[j], fb[j], 0, 1, 2, 3, 4, 5, -1, -1);
-        acc[i][j] = mfma_fp6<FB, FA, 0, 0>(b0, a0, FIRST ? zero : acc[i][j], scb[j], sca[i]);
+        acc[i][j] = mfma_fp6<FB, FA, S0, S0>(b0, a0, FIRST ? zero : acc[i][j], scb[j], sca[i]);
         between(i * TN + j);
       }
     }
@@ -304,7 +322,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const v8i b1 = __builtin_shufflevector(fb[j], fb[j], 6, 7, 8, 9, 10, 11, -1, -1);
-        acc[i][j] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[i][j], scb[j], sca[i]);
+        acc[i][j] = mfma_fp6<FB, FA, S1, S1>(b1, a1, acc[i][j], scb[j], sca[i]);
         between(TM * TN + i * TN + j);
       }
     }
@@ -335,7 +353,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     // other across the steps of a trip they become a few dozen induction variables in scalar registers
     if (!STEADY) asm volatile("" : "+s"(kt));
     const int slotx = GRP == 0 ? stage2 : stage;
-    read_tile(stage, ((p0 + (kt >> 2)) & 1) * kScaleBuf + KM * 4);
+    read_tile.template operator()<KM>(stage, ((p0 + (kt >> 2)) & 1) * kScaleBuf);
     __builtin_amdgcn_sched_barrier(0);
     // the loads reach the next output tile: group 0's with K-tile kt+2 at the start of a step, group 1's
     // with K-tile kt+3 in its compute cluster; the scales with group nk4
@@ -359,7 +377,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     if (GRP == 1) wait_vmcnt<NL + (KM == 0 ? SCL : 0)>();
     barrier();
     __builtin_amdgcn_s_setprio(1);
-    mma_tile.template operator()<FIRST>([&](int i) __attribute__((always_inline)) {
+    mma_tile.template operator()<FIRST, KM>([&](int i) __attribute__((always_inline)) {
       if ((i & 1) && i / 2 < kLoadsInCompute) {
         __builtin_amdgcn_sched_barrier(0);
         issue_one.template operator()<STEADY>(kt + AHEAD, slotx, i / 2);
