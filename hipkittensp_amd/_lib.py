@@ -55,6 +55,12 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_set_kernel.argtypes = [ci]
         L.mxfp6_gemm_noalloc.restype = ci
         L.mxfp6_gemm_noalloc.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        L.mxfp6_probe_mfma.restype = ci
+        L.mxfp6_probe_mfma.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, vp, vp]
+        L.mxfp6_probe_stream.restype = ci
+        L.mxfp6_probe_stream.argtypes = [vp, ctypes.c_size_t, ci, ci, vp, vp]
+        L.mxfp6_probe_tiled_clock.restype = ci
+        L.mxfp6_probe_tiled_clock.argtypes = [vp]
         L.mxfp6_release_workspaces.restype = ci
         L.mxfp6_release_workspaces.argtypes = []
         L.mxfp6_strerror.restype = ctypes.c_char_p

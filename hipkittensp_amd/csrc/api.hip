@@ -19,6 +19,7 @@ namespace {
 // other threads' calls run.
 thread_local int g_force = 0;
 thread_local int g_relayout = 1;
+thread_local uint32_t* g_clock_stamps = nullptr;  // mxfp6_probe_tiled_clock
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
 // demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
@@ -171,6 +172,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out, layout_a, layout_b};
   g.ep = ep;
   g.no_alloc = no_alloc, g.force_split = force_split;
+  g.clock_stamps = g_clock_stamps;
   const int force = no_alloc ? 0 : g_force;  // the entry point that allocates nothing takes no override
   hipError_t e;
   if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
@@ -314,6 +316,37 @@ int mxfp6_gemm_noalloc(const void* A, const void* B, const void* As, const void*
                        int fmt_b, int nsplit, void* stream) {
   if (nsplit != 0 && nsplit != 1 && nsplit != 2 && nsplit != 4 && nsplit != 8) return MXFP6_EINVAL_SHAPE;
   return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, 0, 0, stream, mxfp6::Epilogue(), 1, nsplit);
+}
+
+int mxfp6_probe_tiled_clock(uint32_t* stamps) {
+  g_clock_stamps = stamps;
+  return MXFP6_OK;
+}
+
+int mxfp6_probe_mfma(const void* A, const void* B, const void* As, const void* Bs, int rows_a, int rows_b, int K, int fmt_a, int fmt_b, int iters,
+                     float* sink, uint32_t* stats, void* stream) {
+  if (rows_a < 32 || rows_b < 32 || K < 64 || K % 32 || iters < 1) return MXFP6_EINVAL_SHAPE;
+  if ((fmt_a != MXFP6_FMT_E2M3 && fmt_a != MXFP6_FMT_E3M2) || (fmt_b != MXFP6_FMT_E2M3 && fmt_b != MXFP6_FMT_E3M2)) return MXFP6_EINVAL_FMT;
+  if (!A || !B || !As || !Bs || !sink || !stats) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)sink | (uintptr_t)stats) & 3) return MXFP6_EINVAL_ALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  // two workgroups of four waves per compute unit: two waves per SIMD, as in the tiled kernel
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return MXFP6_ENODEVICE;
+  const hipError_t e = mxfp6::launch_mfma_probe((const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, rows_a, rows_b, K, fmt_a, fmt_b,
+                                                iters, 2 * cus, sink, stats, (hipStream_t)stream);
+  return e == hipSuccess ? 2 * cus * 4 : -(int)e - 1000;  // waves launched (each issues 4 * iters MFMAs of 131072 flop)
+}
+
+int mxfp6_probe_stream(const void* buf, size_t bytes, int workgroups, int waves, uint32_t* stats, void* stream) {
+  if (!buf || !stats) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)buf & 15) || ((uintptr_t)stats & 3)) return MXFP6_EINVAL_ALIGN;
+  if (workgroups < 1 || (waves != 4 && waves != 8) || bytes == 0 || bytes % ((size_t)workgroups * waves * 8192) != 0) return MXFP6_EINVAL_SHAPE;
+  int rc = check_device();
+  if (rc) return rc;
+  const hipError_t e = mxfp6::launch_stream_probe((const uint8_t*)buf, bytes, workgroups, waves, stats, (hipStream_t)stream);
+  return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
 int mxfp6_release_workspaces(void) {

@@ -114,6 +114,7 @@ struct TiledArgs {
   Epilogue ep;
   uint8_t* C_scale;  // fp6 output only
   int fmt_c;
+  uint32_t* stamps;  // measurement only (else null): workgroup 0 leaves its shader-clock and real-time counters here at start and end
 };
 
 // FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
@@ -618,6 +619,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     }
   };
 
+  auto clock_stamp = [&](int where) __attribute__((always_inline)) {
+    const auto g = fresh_args();
+    uint32_t* st = g->stamps;
+    if (st && blockIdx.x == 0 && threadIdx.x == 0) {
+      uint64_t t, r;
+      asm volatile("s_memtime %0\n\ts_memrealtime %1\n\ts_waitcnt lgkmcnt(0)" : "=s"(t), "=s"(r)::"memory");
+      st[2 * where] = (uint32_t)t, st[2 * where + 1] = (uint32_t)r;
+    }
+  };
+  clock_stamp(0);
   // prologue: scales of the first four K-tiles, K-tiles 0 and 1 and, for group 1, the loads of tile 2
   // that its compute cluster of "step -1" would have issued; tile 0 must have landed everywhere
   issue_scales.template operator()<true>(0);
@@ -641,6 +652,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     run.template operator()<1>();
   }
   wait_vmcnt<0>();  // no direct load may still be on its way into LDS when the workgroup gives the memory back
+  clock_stamp(1);
 }
 
 bool gemm_tiled_supports(const GemmArgs& g) {
@@ -711,7 +723,7 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int shape = tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c};
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.clock_stamps};
   const int grid = grid_size(g, tm * tn, bn == 128 ? 2 : 1);  // 128 x 128: 80 KB of LDS, two workgroups per CU
   if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
     if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);

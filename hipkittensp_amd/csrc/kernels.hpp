@@ -19,6 +19,7 @@ struct GemmArgs {
   Epilogue ep;                     // fused bias / scales / activation (all optional)
   uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
   int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output
+  uint32_t* clock_stamps = nullptr;  // tiled kernel, measurement only: four words for workgroup 0's clock / real-time counters at start and end
   int no_alloc = 0;                // skinny kernel: the K split keeps its partial tiles in the library's static scratch array instead of an allocated workspace
   int force_split = 0;             // skinny kernel, M <= 32: split K between this many workgroups (1, 2, 4, 8); 0 = by shape
 };
@@ -47,5 +48,8 @@ hipError_t launch_tile_scales(const uint8_t* src, uint8_t* dst, int rows, int K,
 hipError_t launch_tile_both(const uint8_t* src0, uint8_t* dst0, const uint8_t* ssrc0, uint8_t* sdst0, int rows0, const uint8_t* src1,
                             uint8_t* dst1, const uint8_t* ssrc1, uint8_t* sdst1, int rows1, int K, hipStream_t s);
 hipError_t launch_fill_zero(void* p, size_t bytes, hipStream_t s);
+hipError_t launch_mfma_probe(const uint8_t* A, const uint8_t* B, const uint8_t* As, const uint8_t* Bs, int rows_a, int rows_b, int K, int fmt_a,
+                             int fmt_b, int iters, int workgroups, float* sink, uint32_t* stats, hipStream_t s);
+hipError_t launch_stream_probe(const uint8_t* buf, size_t bytes, int workgroups, int waves, uint32_t* stats, hipStream_t s);
 
 }  // namespace mxfp6

@@ -45,6 +45,7 @@
 #ifndef MXFP6_GEMM_H
 #define MXFP6_GEMM_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -237,6 +238,28 @@ int mxfp6_release_workspaces(void);
  */
 int mxfp6_gemm_noalloc(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale,
                        void *C_bf16, int M, int N, int K, int fmt_a, int fmt_b, int nsplit, void *hip_stream);
+
+/*
+ * Measurement probes (no counterpart in the reference; bench.py reports them next to the roofline fractions).
+ *
+ * mxfp6_probe_mfma: a kernel that only issues v_mfma_scale_f32_32x32x64_f8f6f4 -- two waves per SIMD, each with two
+ * fragments of A and two of B taken once from the given packed operands and scales (rows >= 32, K >= 64) and four
+ * independent accumulators, `iters` rounds of four MFMAs.  Returns the number of waves launched (> 0; each issues
+ * 4 * iters MFMAs of 131072 flop), or a negative MXFP6_E* code, or -(1000 + hipError_t).  stats[0..3] receive the shader
+ * clock counter and the 100 MHz real-time counter of one workgroup at its start and end: clocks / time is the clock the
+ * chip sustains under this load.  sink: one float of device memory (never written in practice).
+ *
+ * mxfp6_probe_stream: `workgroups` workgroups of `waves` (4 or 8) waves read `bytes` bytes (a multiple of
+ * workgroups * waves * 8192) once, each wave a private contiguous range, through direct-to-LDS loads with 16 KB in flight
+ * per wave, and do nothing else.  stats as above.
+ *
+ * mxfp6_probe_tiled_clock: per calling thread; while `stamps` is not NULL the LDS-tiled GEMM kernel's workgroup 0 writes
+ * the same four counters (start, end) there on every launch.
+ */
+int mxfp6_probe_mfma(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, int rows_a,
+                     int rows_b, int K, int fmt_a, int fmt_b, int iters, float *sink, uint32_t *stats, void *hip_stream);
+int mxfp6_probe_stream(const void *buf, size_t bytes, int workgroups, int waves, uint32_t *stats, void *hip_stream);
+int mxfp6_probe_tiled_clock(uint32_t *stamps);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);
