@@ -224,6 +224,8 @@ def main():
     p.add_argument("--warmup", type=int, default=100)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-rows", type=int, default=8192)
+    p.add_argument("--raster-sweep", action="store_true", help="only time the tiled kernel at 8192^3 (tile-major operands) over raster settings and print one JSON line")
+    p.add_argument("--kernel", type=int, default=0, help="with --raster-sweep: kernel code to time as well (18 = the 4-wave schedule)")
     p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the decode run with tile-major weights (used for profiling one layout of the skinny kernel)")
     args = p.parse_args()
     if args.gpus != 1:
@@ -242,6 +244,26 @@ def main():
     M = N = K = 8192
     inputs = make_inputs(hk, torch, M, N, K, 2, 2, seed=1, sets=3)
     C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    if args.raster_sweep:
+        # the tiled kernel alone on tile-major operands, per raster setting (the kernel's own: 4 tile rows per group, XCD remap on)
+        L = _lib.lib()
+        hk.tk_kernel.set_relayout(False)
+        kin = [(hk.tile_operand(ap), hk.tile_operand(bp), hk.tile_scales(asc, K), hk.tile_scales(bsc, K)) for ap, bp, asc, bsc in inputs]
+        res = {}
+        for rnd in range(2):  # two rounds over all settings: the second is reported (the first also warms the chip up)
+            for xcd in (1, 0):
+                for gm in (1, 2, 4, 8, 16, 32):
+                    assert L.mxfp6_probe_raster(gm, xcd) == 0
+                    _, ms = timed_loop(hk, torch, kin, C, args.steps, args.warmup, 1, 1)
+                    res[f"xcd_remap={xcd},group_m={gm}"] = {"launch_ms_mean": ms, "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12}
+            L.mxfp6_probe_raster(0, 1)
+            if args.kernel:
+                prevk = hk.tk_kernel.set_kernel(args.kernel)
+                _, ms = timed_loop(hk, torch, kin, C, args.steps, args.warmup, 1, 1)
+                hk.tk_kernel.set_kernel(prevk)
+                res[f"kernel={args.kernel}"] = {"launch_ms_mean": ms, "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12}
+        print(json.dumps({"what": "gemm_tiled_kernel, 8192^3 e2m3, operands and scales tile-major, per raster setting", "steps": args.steps, "warmup": args.warmup, "settings": res}))
+        return
     # the operator as a caller gets it: for this size the library re-lays both operands out tile-major in a
     # pre-pass (one small kernel each) and runs the tiled kernel on them; `value` is the whole step
     wall, step_ms = timed_loop(hk, torch, inputs, C, args.steps, args.warmup)

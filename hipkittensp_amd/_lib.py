@@ -61,6 +61,10 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_probe_stream.argtypes = [vp, ctypes.c_size_t, ci, ci, vp, vp]
         L.mxfp6_probe_tiled_clock.restype = ci
         L.mxfp6_probe_tiled_clock.argtypes = [vp]
+        L.mxfp6_tile_order.restype = ci
+        L.mxfp6_tile_order.argtypes = [ci, ci, ci, ci, vp]
+        L.mxfp6_probe_raster.restype = ci
+        L.mxfp6_probe_raster.argtypes = [ci, ci]
         L.mxfp6_release_workspaces.restype = ci
         L.mxfp6_release_workspaces.argtypes = []
         L.mxfp6_strerror.restype = ctypes.c_char_p

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmxfp6_gemm.so")
-SOURCES = ["api.hip", "gemm_generic.hip", "gemm_tiled.hip", "gemm_mid.hip", "gemm_skinny.hip", "quantize.hip", "probes.hip"]
+SOURCES = ["api.hip", "gemm_generic.hip", "gemm_tiled.hip", "gemm_tiled4.hip", "gemm_mid.hip", "gemm_skinny.hip", "quantize.hip", "probes.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-std=c++20", "-O3", "-fPIC", "-fvisibility=hidden",

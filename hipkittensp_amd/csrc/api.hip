@@ -20,6 +20,7 @@ namespace {
 thread_local int g_force = 0;
 thread_local int g_relayout = 1;
 thread_local uint32_t* g_clock_stamps = nullptr;  // mxfp6_probe_tiled_clock
+thread_local int g_raster_group_m = 0, g_raster_no_xcd = 0;  // mxfp6_probe_raster
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
 // demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
@@ -173,6 +174,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   g.ep = ep;
   g.no_alloc = no_alloc, g.force_split = force_split;
   g.clock_stamps = g_clock_stamps;
+  g.raster_group_m = g_raster_group_m, g.raster_no_xcd_remap = g_raster_no_xcd;
   const int force = no_alloc ? 0 : g_force;  // the entry point that allocates nothing takes no override
   hipError_t e;
   if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
@@ -192,6 +194,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 4) {
     if (!mxfp6::gemm_mid_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_mid(g, s);
+  } else if (force == 18) {
+    if (!mxfp6::gemm_tiled4_supports(g)) return MXFP6_EINVAL_SHAPE;
+    e = mxfp6::launch_gemm_tiled4(g, s);
   } else if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) {
     e = mxfp6::launch_gemm_skinny(g, s);
   } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
@@ -306,7 +311,7 @@ int mxfp6_set_relayout(int on) {
 }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 17) return MXFP6_EINVAL_KERNEL;
+  if (which < 0 || which > 18) return MXFP6_EINVAL_KERNEL;
   const int prev = g_force;
   g_force = which;
   return prev;
@@ -316,6 +321,20 @@ int mxfp6_gemm_noalloc(const void* A, const void* B, const void* As, const void*
                        int fmt_b, int nsplit, void* stream) {
   if (nsplit != 0 && nsplit != 1 && nsplit != 2 && nsplit != 4 && nsplit != 8) return MXFP6_EINVAL_SHAPE;
   return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, 0, 0, stream, mxfp6::Epilogue(), 1, nsplit);
+}
+
+int mxfp6_probe_raster(int group_m, int xcd_remap) {
+  if (group_m < 0 || group_m > 4096) return MXFP6_EINVAL_SHAPE;
+  g_raster_group_m = group_m, g_raster_no_xcd = xcd_remap ? 0 : 1;
+  return MXFP6_OK;
+}
+
+int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int* order) {
+  if (tiles_m < 1 || tiles_n < 1 || tiles_m > 65535 || tiles_n > 32767 || group_m < 1 || (long)tiles_m * tiles_n >= (1L << 31)) return MXFP6_EINVAL_SHAPE;
+  if (!order) return MXFP6_EINVAL_PTR;
+  const int nb = tiles_m * tiles_n;
+  for (int b = 0; b < nb; b++) order[b] = mxfp6::tile_order(b, tiles_m, tiles_n, group_m, xcd_remap);
+  return mxfp6::tile_order(nb, tiles_m, tiles_n, group_m, xcd_remap) == -1 ? MXFP6_OK : MXFP6_EINVAL_SHAPE;
 }
 
 int mxfp6_probe_tiled_clock(uint32_t* stamps) {

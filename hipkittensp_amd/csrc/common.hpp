@@ -105,6 +105,26 @@ __device__ __forceinline__ v16f mfma_fp6(v8i sa, v8i sb, v16f acc, int scale_sa,
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(sa, sb, acc, FMT_SA, FMT_SB, OPA, scale_sa, OPB, scale_sb);
 }
 
+// Workgroup -> output tile of the LDS-tiled kernels.  Workgroup `bid` of a launch works on tiles bid, bid + grid, ... of a
+// logical order in which the round-robin placement of workgroups on the 8 XCDs (workgroup b runs on XCD b % 8) is
+// undone, so that each XCD gets a contiguous run of logical tiles (xcd_remap; the idea of chiplet_transform_chunked,
+// include/common/util.cuh:78-101, as an exact bijection for any tile count), and the raster walks group_m tile rows at a
+// time down the columns (analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61): the tiles an XCD works on at once share
+// operand rows in its L2.  Returns pm | pn << 16, or -1 past the last tile.
+__host__ __device__ __forceinline__ int tile_order(int bid, int tiles_m, int tiles_n, int group_m, int xcd_remap) {
+  const int nb = tiles_m * tiles_n;
+  if (bid >= nb) return -1;
+  int L = bid;
+  if (xcd_remap) {
+    const int xcd = bid & 7, idx = bid >> 3;
+    const int per = nb >> 3, rem = nb & 7;
+    L = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+  }
+  const int width = group_m * tiles_n, group = L / width, first = group * group_m;
+  const int gsz = tiles_m - first < group_m ? tiles_m - first : group_m, in = L - group * width;
+  return (first + in % gsz) | (in / gsz) << 16;
+}
+
 // Byte offset, inside a tile-major operand, of byte `b` (0 .. 3K/4) of row `row`; nkt = K / 128.
 // Tiles are 32 rows x 96 bytes in the kernels' LDS image order (16-byte pieces, pairs swapped in
 // rows with bit 3 set).

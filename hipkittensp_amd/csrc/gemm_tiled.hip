@@ -114,6 +114,7 @@ struct TiledArgs {
   Epilogue ep;
   uint8_t* C_scale;  // fp6 output only
   int fmt_c;
+  int group_m, xcd_remap;  // raster: tile rows per group (kGroupM unless a measurement overrides it), XCD remap on / off
   uint32_t* stamps;  // measurement only (else null): workgroup 0 leaves its shader-clock and real-time counters here at start and end
 };
 
@@ -142,21 +143,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     return p;
   };
 
-  // ---- workgroup -> output tiles.  Workgroup b works on tiles b, b + gridDim.x, ... of a logical order in
-  // which the round-robin XCD placement is undone and the raster is grouped.  Hardware places workgroup b on
-  // XCD b % 8; the remapping gives each XCD a contiguous run of logical tiles so that the 32 tiles an XCD
-  // works on at once share operand rows in its L2 (the idea of chiplet_transform_chunked,
-  // include/common/util.cuh:78-101, as an exact bijection).  Returns pm | pn << 16, or -1 past the last tile.
+  // ---- workgroup -> output tiles: workgroup b works on tiles b, b + gridDim.x, ... of tile_order() (common.hpp)
   auto tile_of = [&](int bid) __attribute__((always_inline)) {
     const auto g = fresh_args();
-    const int tiles_m = g->tiles_m, tiles_n = g->tiles_n, nb = tiles_m * tiles_n;
-    if (bid >= nb) return -1;
-    const int xcd = bid & 7, idx = bid >> 3;
-    const int per = nb >> 3, rem = nb & 7;
-    const int L = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
-    const int width = kGroupM * tiles_n, group = L / width, first = group * kGroupM;
-    const int gsz = min(tiles_m - first, kGroupM), in = L - group * width;
-    return (first + in % gsz) | (in / gsz) << 16;
+    return tile_order(bid, g->tiles_m, g->tiles_n, g->group_m, g->xcd_remap);
   };
   // Buffer resources of one output tile's operand rows (A and B) and of the scale rows this wave loads.  Edge
   // tiles: rows past M (or N) lie beyond the end of the resource and read as zeros.  tile < 0: resources of
@@ -723,7 +713,7 @@ template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const int shape = tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.clock_stamps};
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, g.clock_stamps};
   const int grid = grid_size(g, tm * tn, bn == 128 ? 2 : 1);  // 128 x 128: 80 KB of LDS, two workgroups per CU
   if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
     if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);

@@ -19,6 +19,7 @@ struct GemmArgs {
   Epilogue ep;                     // fused bias / scales / activation (all optional)
   uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
   int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output
+  int raster_group_m = 0, raster_no_xcd_remap = 0;  // tiled kernel, measurement only: tile rows per raster group (0 = the default, 4), XCD remap off
   uint32_t* clock_stamps = nullptr;  // tiled kernel, measurement only: four words for workgroup 0's clock / real-time counters at start and end
   int no_alloc = 0;                // skinny kernel: the K split keeps its partial tiles in the library's static scratch array instead of an allocated workspace
   int force_split = 0;             // skinny kernel, M <= 32: split K between this many workgroups (1, 2, 4, 8); 0 = by shape
@@ -32,6 +33,8 @@ inline bool operands_aligned16(const GemmArgs& g) {
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
+bool gemm_tiled4_supports(const GemmArgs& g);  // the 4-wave variant of the tiled kernel (selectable, never chosen automatically)
+hipError_t launch_gemm_tiled4(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
 bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
 double tiled_estimate_us(const GemmArgs& g, int rows, int cols = 256);  // estimated time of the tiled kernel with tiles of rows x cols

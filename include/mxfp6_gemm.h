@@ -109,6 +109,8 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *       (the split takes a workspace of 2 MB per stream at first use; without one, e.g. first use under stream capture,
  *       the launch runs unsplit); 16: 32 rows of B and two waves per workgroup
  *    4  mid-M kernel (needs 32 < M <= 512, K % 1024 == 0, row-major A)
+ *   18  the 4-wave interleaved schedule of the LDS-tiled kernel (one wave per SIMD with a 128 x 128 wave tile; shapes
+ *       of kernel 2, no fused epilogue); never chosen automatically, kept to compare the two schedules
  * No counterpart in the reference, whose shapes are compile-time constants per binary
  * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
  */
@@ -260,6 +262,17 @@ int mxfp6_probe_mfma(const void *A_packed, const void *B_packed, const void *A_s
                      int rows_b, int K, int fmt_a, int fmt_b, int iters, float *sink, uint32_t *stats, void *hip_stream);
 int mxfp6_probe_stream(const void *buf, size_t bytes, int workgroups, int waves, uint32_t *stats, void *hip_stream);
 int mxfp6_probe_tiled_clock(uint32_t *stamps);
+
+/*
+ * The workgroup -> output tile map of the LDS-tiled kernel, evaluated on the host with the kernel's own function:
+ * order[b] = pm | pn << 16 is the tile (row pm, column pn of a tiles_m x tiles_n grid) that logical workgroup b works on.
+ * The kernel uses group_m = 4 and xcd_remap = 1; mxfp6_probe_raster (per calling thread, measurement only; group_m = 0
+ * restores the default) makes later launches use other values, for sweeps of the raster like the reference's
+ * (analysis/paper_experiments/grid_micro/data_to_log.json; remap include/common/util.cuh:78-101).  A host-side pointer:
+ * `order` holds tiles_m * tiles_n ints.
+ */
+int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int *order);
+int mxfp6_probe_raster(int group_m, int xcd_remap);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

@@ -199,3 +199,40 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "ONE GPU" in (r.stdout + r.stderr)
+
+
+@pytest.mark.parametrize("tiles_m,tiles_n", [(1, 1), (1, 7), (7, 1), (3, 5), (4, 8), (32, 32), (16, 112), (5, 13), (33, 31), (9, 9), (2, 3), (61, 7)])
+@pytest.mark.parametrize("group_m,xcd", [(4, 1), (4, 0), (1, 1), (8, 1), (16, 1), (3, 1)])
+def test_tile_order_is_a_bijection(built_lib, tiles_m, tiles_n, group_m, xcd):
+    """The tiled kernel's workgroup -> tile map (XCD remap + grouped raster), evaluated by the library's own function on
+    the host: every tile exactly once for ragged tile counts too (the reference's remap leaves tail ids unmapped,
+    include/common/util.cuh:92), and with the remap on, the tiles one XCD works on form a contiguous run of the raster."""
+    import numpy as np
+
+    L = ctypes.CDLL(built_lib)
+    L.mxfp6_tile_order.restype = ctypes.c_int
+    L.mxfp6_tile_order.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    nb = tiles_m * tiles_n
+    order = np.full(nb, -7, np.int32)
+    assert L.mxfp6_tile_order(tiles_m, tiles_n, group_m, xcd, order.ctypes.data) == 0
+    pm, pn = order & 0xFFFF, order >> 16
+    assert pm.min() >= 0 and pm.max() < tiles_m and pn.min() >= 0 and pn.max() < tiles_n
+    assert len(set(zip(pm.tolist(), pn.tolist()))) == nb                      # a bijection onto the tile grid
+    # the raster without the remap: groups of group_m tile rows, columns inside a group, rows fastest
+    ident = np.full(nb, -7, np.int32)
+    assert L.mxfp6_tile_order(tiles_m, tiles_n, group_m, 0, ident.ctypes.data) == 0
+    k = 0
+    for first in range(0, tiles_m, group_m):
+        gsz = min(group_m, tiles_m - first)
+        for col in range(tiles_n):
+            for r in range(gsz):
+                assert ident[k] == (first + r) | col << 16
+                k += 1
+    if xcd:
+        # workgroups b, b + 8, b + 16, ... (one XCD) get consecutive positions of that raster
+        pos = {int(v): i for i, v in enumerate(ident)}
+        for x in range(min(8, nb)):
+            run = [pos[int(order[b])] for b in range(x, nb, 8)]
+            assert run == list(range(run[0], run[0] + len(run)))
+        starts = sorted(pos[int(order[x])] for x in range(min(8, nb)))
+        assert starts[0] == 0

@@ -131,12 +131,13 @@ def test_generic_kernel_any_shape(hk, M, N, K, fa, fb):
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (256, 512, 384), (512, 256, 1664), (768, 1024, 1024),
                                    (300, 264, 256), (257, 8, 128), (100, 1000, 384), (33, 520, 640), (1, 256, 128)])  # edge tiles too
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
-def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb):
+@pytest.mark.parametrize("kernel", [2, 18])  # 8-wave ping-pong (the one the automatic choice uses) and the 4-wave interleaved schedule
+def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M * 3 + N + K, kind_a="laplace" if fa == 3 else "normal", kind_b="weights")
     ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
-    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=2)
+    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel)
     check(got, ref, fa, fb, ap, asc, bp, bsc)
-    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=2)
+    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=kernel)
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
@@ -305,7 +306,7 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
 
 
 @pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
-                                          (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128)])
+                                          (18, 256, 512, 640), (18, 320, 544, 1152), (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
     if kernel in (3, 4) and la == 1:
@@ -639,13 +640,20 @@ def test_gpu_quantiser_bit_exact(hk, fmt, kind):
 
 
 # ------------------------------------------------------------------ full-size configurations
-def _sampled_check(hk, ap, asc, bp, bsc, fa, fb, kernel, rng, ns=48):
+def _sampled_check(hk, ap, asc, bp, bsc, fa, fb, kernel, rng, ns=48, band=256):
+    """Full-size check of one configuration: a whole band of `band` consecutive rows of the fp32 result (all N columns, so
+    every tile column, straddling a tile-row boundary) against the C oracle's dequantise-and-matmul; sampled rows and
+    columns against the fp64 oracle; exact scale linearity; bf16 = RNE of the accumulators."""
     M, N = ap.shape[0], bp.shape[0]
     C = torch.empty(M, N, dtype=torch.float32, device="cuda")
     dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
     prev = hk.tk_kernel.set_kernel(kernel)
     try:
         hk.dispatch_micro(dA, dB, dAs, dBs, C, fa, fb)
+        if band and M > band:
+            r0 = (M // 2 - band // 2) // 32 * 32 + 32  # not aligned to the 128- or 256-row tiles: the band crosses a tile-row boundary
+            full = co.gemm_f32(ap[r0:r0 + band], bp, asc[r0:r0 + band], bsc, fa, fb)
+            check(C[r0:r0 + band].cpu().numpy(), full, fa, fb)
         rows = np.sort(rng.choice(M, size=min(ns, M), replace=False))
         cols = np.sort(rng.choice(N, size=min(ns, N), replace=False))
         ref = o.gemm_ref(ap[rows], bp[cols], asc[rows], bsc[cols], fa, fb, acc=np.float64)
