@@ -61,6 +61,16 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_probe_stream.argtypes = [vp, ctypes.c_size_t, ci, ci, vp, vp]
         L.mxfp6_probe_tiled_clock.restype = ci
         L.mxfp6_probe_tiled_clock.argtypes = [vp]
+        L.mxfp6_blob_bytes.restype = ctypes.c_size_t
+        L.mxfp6_blob_bytes.argtypes = [ci, ci]
+        L.mxfp6_blob_header_write.restype = ci
+        L.mxfp6_blob_header_write.argtypes = [vp, ci, ci, ci]
+        L.mxfp6_blob_header_read.restype = ci
+        L.mxfp6_blob_header_read.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        L.mxfp6_blob_pack.restype = ci
+        L.mxfp6_blob_pack.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+        L.mxfp6_blob_unpack.restype = ci
+        L.mxfp6_blob_unpack.argtypes = [vp, vp, vp, ci, ci, vp]
         L.mxfp6_tile_order.restype = ci
         L.mxfp6_tile_order.argtypes = [ci, ci, ci, ci, vp]
         L.mxfp6_probe_raster.restype = ci

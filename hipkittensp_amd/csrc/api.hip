@@ -323,6 +323,84 @@ int mxfp6_gemm_noalloc(const void* A, const void* B, const void* As, const void*
   return gemm_common(A, B, As, Bs, C, M, N, K, fmt_a, fmt_b, false, 0, 0, stream, mxfp6::Epilogue(), 1, nsplit);
 }
 
+// ---- serialised tile-major operand ("blob"): 16-byte header, tile-major packed bytes, tile-major scales
+namespace {
+constexpr uint32_t kBlobMagic = 0x5436584du;  // "MX6T"
+constexpr uint8_t kBlobVersion = 1;
+__global__ void blob_header_kernel(uint32_t* dst, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+  dst[0] = w0, dst[1] = w1, dst[2] = w2, dst[3] = w3;
+}
+bool blob_shape_ok(int rows, int K) { return rows > 0 && K > 0 && rows % 32 == 0 && K % 128 == 0 && (size_t)rows * (K / 4 * 3) < ((size_t)1 << 40); }
+void blob_words(int rows, int K, int fmt, uint32_t w[4]) {
+  w[0] = kBlobMagic;
+  w[1] = (uint32_t)kBlobVersion | (uint32_t)fmt << 8 | (uint32_t)MXFP6_LAYOUT_TILE << 16;  // byte 7 reserved (0)
+  w[2] = (uint32_t)rows;
+  w[3] = (uint32_t)K;
+}
+}  // namespace
+
+size_t mxfp6_blob_bytes(int rows, int K) {
+  if (!blob_shape_ok(rows, K)) return 0;
+  return 16 + (size_t)rows * (K / 4 * 3) + (size_t)rows * ((K + 511) / 512) * 16;
+}
+
+int mxfp6_blob_header_write(void* header16, int rows, int K, int fmt) {
+  if (!header16) return MXFP6_EINVAL_PTR;
+  if (!blob_shape_ok(rows, K)) return MXFP6_EINVAL_SHAPE;
+  if (fmt != MXFP6_FMT_E2M3 && fmt != MXFP6_FMT_E3M2) return MXFP6_EINVAL_FMT;
+  uint32_t w[4];
+  blob_words(rows, K, fmt, w);
+  uint8_t* h = static_cast<uint8_t*>(header16);
+  for (int i = 0; i < 4; i++)
+    for (int b = 0; b < 4; b++) h[4 * i + b] = (uint8_t)(w[i] >> (8 * b));  // little endian whatever the host is
+  return MXFP6_OK;
+}
+
+int mxfp6_blob_header_read(const void* header16, int* rows, int* K, int* fmt) {
+  if (!header16 || !rows || !K || !fmt) return MXFP6_EINVAL_PTR;
+  const uint8_t* h = static_cast<const uint8_t*>(header16);
+  uint32_t w[4];
+  for (int i = 0; i < 4; i++) w[i] = (uint32_t)h[4 * i] | (uint32_t)h[4 * i + 1] << 8 | (uint32_t)h[4 * i + 2] << 16 | (uint32_t)h[4 * i + 3] << 24;
+  if (w[0] != kBlobMagic) return MXFP6_EBLOB;
+  if ((w[1] & 0xff) != kBlobVersion || ((w[1] >> 16) & 0xff) != MXFP6_LAYOUT_TILE || (w[1] >> 24) != 0) return MXFP6_EBLOB;
+  const int f = (int)((w[1] >> 8) & 0xff);
+  if (f != MXFP6_FMT_E2M3 && f != MXFP6_FMT_E3M2) return MXFP6_EBLOB;
+  if (w[2] > 0x7fffffffu || w[3] > 0x7fffffffu || !blob_shape_ok((int)w[2], (int)w[3])) return MXFP6_EBLOB;
+  *rows = (int)w[2], *K = (int)w[3], *fmt = f;
+  return MXFP6_OK;
+}
+
+int mxfp6_blob_pack(const void* packed, const void* scales, void* blob, int rows, int K, int fmt, void* stream) {
+  if (!blob_shape_ok(rows, K)) return MXFP6_EINVAL_SHAPE;
+  if (fmt != MXFP6_FMT_E2M3 && fmt != MXFP6_FMT_E3M2) return MXFP6_EINVAL_FMT;
+  if (!packed || !scales || !blob) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)packed & 15) || ((uintptr_t)blob & 15) || ((uintptr_t)scales & 3)) return MXFP6_EINVAL_ALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t w[4];
+  blob_words(rows, K, fmt, w);
+  blob_header_kernel<<<1, 1, 0, s>>>(static_cast<uint32_t*>(blob), w[0], w[1], w[2], w[3]);
+  hipError_t e = hipGetLastError();
+  uint8_t* body = static_cast<uint8_t*>(blob) + 16;
+  if (e == hipSuccess) e = mxfp6::launch_tile_operand((const uint8_t*)packed, body, rows, K, 1, s);
+  if (e == hipSuccess) e = mxfp6::launch_tile_scales((const uint8_t*)scales, body + (size_t)rows * (K / 4 * 3), rows, K, 1, s);
+  return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
+int mxfp6_blob_unpack(const void* blob, void* packed, void* scales, int rows, int K, void* stream) {
+  if (!blob_shape_ok(rows, K)) return MXFP6_EINVAL_SHAPE;
+  if (!packed || !scales || !blob) return MXFP6_EINVAL_PTR;
+  if (((uintptr_t)packed & 15) || ((uintptr_t)blob & 15) || ((uintptr_t)scales & 3)) return MXFP6_EINVAL_ALIGN;
+  int rc = check_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* body = static_cast<const uint8_t*>(blob) + 16;
+  hipError_t e = mxfp6::launch_tile_operand(body, (uint8_t*)packed, rows, K, 0, s);
+  if (e == hipSuccess) e = mxfp6::launch_tile_scales(body + (size_t)rows * (K / 4 * 3), (uint8_t*)scales, rows, K, 0, s);
+  return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
 int mxfp6_probe_raster(int group_m, int xcd_remap) {
   if (group_m < 0 || group_m > 4096) return MXFP6_EINVAL_SHAPE;
   g_raster_group_m = group_m, g_raster_no_xcd = xcd_remap ? 0 : 1;
@@ -412,13 +490,14 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_EINVAL_EPILOGUE: return "mxfp6: activation must be 0 (none), 1 (relu), 2 (gelu) or 3 (silu)";
     case MXFP6_ESCRATCH: return "mxfp6: the K split of this call needs more than the static scratch memory holds (256 partial tiles: rows of C tiles times nsplit)";
     case MXFP6_EINVAL_KERNEL: return "mxfp6: unknown kernel code";
+    case MXFP6_EBLOB: return "mxfp6: not a tile-major operand blob this library reads (magic, version, format, layout or shape)";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 113; }
+int mxfp6_abi_version(void) { return 114; }
 
 #pragma GCC visibility pop
 }  // extern "C"

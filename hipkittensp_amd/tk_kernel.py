@@ -300,3 +300,49 @@ def dispatch_micro_noalloc(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: 
 def release_workspaces() -> None:
     """Return every workspace the library holds to the stream-ordered allocator."""
     _lib.check(_lib.lib().mxfp6_release_workspaces(), "release_workspaces")
+
+
+def pack_weights(packed, scales, fmt: int = E2M3):
+    """Row-major packed operand [rows, 3K/4] + scales [rows, K/32] (GPU tensors) -> one uint8 blob on the GPU: 16-byte
+    header (magic "MX6T", version, format, layout, rows, K), tile-major operand, tile-major scales.  The blob can be
+    copied to the host and stored; unpack_weights() of a blob in GPU memory gives views that dispatch_micro takes as a
+    tile-major operand without any conversion."""
+    import torch
+
+    packed, scales = _as_tensor(packed, "packed"), _as_tensor(scales, "scales")
+    if packed.dtype != torch.uint8 or scales.dtype != torch.uint8:
+        raise RuntimeError("packed / scales: expected dtype uint8")
+    rows, w = _rows_cols(packed, "packed")
+    if w % 96 or rows % 32:
+        raise RuntimeError("a tile-major blob needs rows % 32 == 0 and K % 128 == 0")
+    K = w // 3 * 4
+    if _rows_cols(scales, "scales") != (rows, K // 32):
+        raise RuntimeError(f"scales: expected shape [{rows}, {K // 32}], got {tuple(scales.shape)}")
+    L = _lib.lib()
+    blob = torch.empty(L.mxfp6_blob_bytes(rows, K), dtype=torch.uint8, device=packed.device)
+    with _on_device(packed.device):
+        rc = L.mxfp6_blob_pack(packed.data_ptr(), scales.data_ptr(), blob.data_ptr(), rows, K, fmt, _stream())
+    _lib.check(rc, "pack_weights")
+    return blob
+
+
+def unpack_weights(blob):
+    """A blob of pack_weights() (uint8, GPU) -> (operand [rows, 3K/4], scales [rows, ceil(K/512) * 16], fmt): views into the
+    blob in tile-major layout, for dispatch_micro(..., layout_b=LAYOUT_TILE).  Raises RuntimeError for anything that is not
+    a blob of a version this library reads."""
+    import ctypes
+
+    import torch
+
+    blob = _as_tensor(blob, "blob")
+    if blob.dtype != torch.uint8 or blob.dim() != 1 or blob.numel() < 16:
+        raise RuntimeError("blob: expected a 1-D uint8 tensor of at least 16 bytes")
+    L = _lib.lib()
+    head = bytes(blob[:16].cpu().tolist())
+    rows, K, fmt = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _lib.check(L.mxfp6_blob_header_read(head, ctypes.byref(rows), ctypes.byref(K), ctypes.byref(fmt)), "unpack_weights")
+    rows, K, fmt = rows.value, K.value, fmt.value
+    if blob.numel() != L.mxfp6_blob_bytes(rows, K):
+        raise RuntimeError(f"blob: header says {L.mxfp6_blob_bytes(rows, K)} bytes, tensor has {blob.numel()}")
+    nop = rows * (K // 4 * 3)
+    return blob[16:16 + nop].view(rows, K // 4 * 3), blob[16 + nop:].view(rows, scale_width(K, LAYOUT_TILE)), fmt

@@ -66,6 +66,7 @@ extern "C" {
 #define MXFP6_EINVAL_EPILOGUE (-7) /* activation code is not one of MXFP6_ACT_*                */
 #define MXFP6_ESCRATCH (-8)     /* mxfp6_gemm_noalloc: the requested K split does not fit the static scratch memory */
 #define MXFP6_EINVAL_KERNEL (-9) /* mxfp6_set_kernel: unknown kernel code                        */
+#define MXFP6_EBLOB (-10)       /* not a tile-major operand blob of a version this library reads */
 
 /* Activations of mxfp6_gemm_fused. */
 #define MXFP6_ACT_NONE 0
@@ -162,6 +163,33 @@ int mxfp6_tile_operand(const void *src, void *dst, int rows, int K, int tile, vo
  * reference (its operands carry no scales); part of the tile-major operand format above.
  */
 int mxfp6_tile_scales(const void *src, void *dst, int rows, int K, int tile, void *hip_stream);
+
+/*
+ * Serialised tile-major operand (a weight converted once, stored or shipped, and used without conversion): a blob of
+ *   bytes  0 ..  3  magic "MX6T"
+ *   byte   4        format version (1)
+ *   byte   5        operand format (MXFP6_FMT_E2M3 / MXFP6_FMT_E3M2)
+ *   byte   6        layout (MXFP6_LAYOUT_TILE)
+ *   byte   7        reserved, 0
+ *   bytes  8 .. 11  rows, bytes 12 .. 15  K   (little endian)
+ *   then the tile-major packed bytes (rows * 3K/4) and the tile-major scales (rows * ceil(K/512) * 16), as defined above.
+ * rows % 32 == 0, K % 128 == 0.  Both parts start 16-byte aligned inside a 16-byte aligned blob, so a blob in device
+ * memory is used in place: blob + 16 and blob + 16 + rows * 3K/4 are the operand and scale pointers of mxfp6_gemm_ex with
+ * MXFP6_LAYOUT_TILE.  mxfp6_blob_bytes: size of the blob (0 for a shape it cannot hold).  mxfp6_blob_header_write /
+ * _read work on 16 bytes of HOST memory; _read returns MXFP6_EBLOB for a wrong magic, an unknown version, format or
+ * layout, a non-zero reserved byte or an impossible shape.  mxfp6_blob_pack writes the whole blob, header included, in
+ * DEVICE memory from a row-major operand and its row-major scales; mxfp6_blob_unpack converts a device blob's body back
+ * (the caller has read rows and K from a host copy of the header).  No counterpart in the reference, which has no
+ * stored operand format; the layout itself is the swizzle of include/ops/warp/memory/tile/global_to_shared.cuh:46-59
+ * applied to the data.
+ */
+size_t mxfp6_blob_bytes(int rows, int K);
+int mxfp6_blob_header_write(void *header16_host, int rows, int K, int fmt);
+int mxfp6_blob_header_read(const void *header16_host, int *rows, int *K, int *fmt);
+int mxfp6_blob_pack(const void *packed_row_major, const void *scales_row_major, void *blob, int rows, int K, int fmt,
+                    void *hip_stream);
+int mxfp6_blob_unpack(const void *blob, void *packed_row_major, void *scales_row_major, int rows, int K,
+                      void *hip_stream);
 
 /*
  * mxfp6_gemm / mxfp6_gemm_f32out with a layout per operand (MXFP6_LAYOUT_*) and out_f32 != 0 for

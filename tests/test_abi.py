@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 113
+    assert L.mxfp6_abi_version() == 114
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -236,3 +236,33 @@ def test_tile_order_is_a_bijection(built_lib, tiles_m, tiles_n, group_m, xcd):
             assert run == list(range(run[0], run[0] + len(run)))
         starts = sorted(pos[int(order[x])] for x in range(min(8, nb)))
         assert starts[0] == 0
+
+
+def test_blob_header_round_trip_and_rejections(built_lib):
+    """The 16-byte header of the serialised tile-major operand: written and read on the host, byte for byte as documented."""
+    L = ctypes.CDLL(built_lib)
+    ci, vp = ctypes.c_int, ctypes.c_void_p
+    L.mxfp6_blob_bytes.restype = ctypes.c_size_t
+    L.mxfp6_blob_bytes.argtypes = [ci, ci]
+    L.mxfp6_blob_header_write.restype = ci
+    L.mxfp6_blob_header_write.argtypes = [vp, ci, ci, ci]
+    L.mxfp6_blob_header_read.restype = ci
+    L.mxfp6_blob_header_read.argtypes = [vp, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+    assert L.mxfp6_blob_bytes(64, 640) == 16 + 64 * 480 + 64 * 2 * 16      # K = 640: two groups of four K-tiles of scales
+    assert L.mxfp6_blob_bytes(8192, 8192) == 16 + 8192 * 6144 + 8192 * 256
+    assert L.mxfp6_blob_bytes(33, 128) == 0 and L.mxfp6_blob_bytes(32, 96) == 0
+    buf = ctypes.create_string_buffer(16)
+    assert L.mxfp6_blob_header_write(buf, 96, 1152, 3) == 0
+    assert buf.raw == b"MX6T" + bytes([1, 3, 1, 0]) + (96).to_bytes(4, "little") + (1152).to_bytes(4, "little")
+    rows, K, fmt = ci(), ci(), ci()
+    assert L.mxfp6_blob_header_read(buf, ctypes.byref(rows), ctypes.byref(K), ctypes.byref(fmt)) == 0
+    assert (rows.value, K.value, fmt.value) == (96, 1152, 3)
+    assert L.mxfp6_blob_header_write(buf, 96, 100, 2) == -2 and L.mxfp6_blob_header_write(buf, 96, 128, 4) == -3
+    good = bytearray(buf.raw)
+    for pos, val in ((0, ord("X")), (4, 2), (5, 1), (6, 0), (7, 9), (8, 1), (12, 7)):   # magic, version, fmt, layout, reserved, rows % 32, K % 128
+        bad = bytearray(good)
+        bad[pos] = val
+        assert L.mxfp6_blob_header_read(bytes(bad), ctypes.byref(rows), ctypes.byref(K), ctypes.byref(fmt)) == -10, pos
+    L.mxfp6_strerror.restype = ctypes.c_char_p
+    L.mxfp6_strerror.argtypes = [ci]
+    assert b"blob" in L.mxfp6_strerror(-10)

@@ -331,6 +331,49 @@ def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb)
     check(ref, o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64), fa, fb)
 
 
+@pytest.mark.parametrize("rows,K,fmt", [(32, 128, 2), (96, 1152, 3), (256, 640, 2), (64, 8192, 2)])
+def test_weight_blob_round_trip(hk, rows, K, fmt):
+    """The serialised tile-major operand: header as documented, body = the CPU definition of the tile-major layouts
+    (oracle.tile_operand / tile_scales) of CPU-generated bytes, unpack = the original, and the views of a blob are usable
+    as a tile-major B without conversion."""
+    rng = np.random.default_rng(rows + K)
+    packed = rng.integers(0, 256, (rows, K // 4 * 3), dtype=np.uint8)
+    scales = rng.integers(100, 150, (rows, K // 32), dtype=np.uint8)
+    blob = hk.pack_weights(dev(packed), dev(scales), fmt)
+    raw = blob.cpu().numpy()
+    assert raw[:16].tobytes() == b"MX6T" + bytes([1, fmt, 1, 0]) + rows.to_bytes(4, "little") + K.to_bytes(4, "little")
+    nop = rows * (K // 4 * 3)
+    assert np.array_equal(raw[16:16 + nop].reshape(rows, -1), o.tile_operand(packed))
+    st = o.tile_scales(scales)
+    got_s = raw[16 + nop:].reshape(rows, -1)
+    assert got_s.shape == st.shape
+    valid = o.tile_scales(np.ones_like(scales)) == 1      # the bytes of K-blocks past K are padding (written as 0)
+    assert np.array_equal(got_s[valid], st[valid]) and not got_s[~valid].any()
+    op, sc, f = hk.unpack_weights(blob)
+    assert f == fmt and np.array_equal(hk.tile_operand(op.contiguous(), untile=True).cpu().numpy(), packed)
+    assert np.array_equal(hk.tile_scales(sc.contiguous(), K, untile=True).cpu().numpy(), scales)
+    # through the C ABI's own unpack as well
+    from hipkittensp_amd import _lib
+    p2, s2 = torch.empty(rows, K // 4 * 3, dtype=torch.uint8, device="cuda"), torch.empty(rows, K // 32, dtype=torch.uint8, device="cuda")
+    assert _lib.lib().mxfp6_blob_unpack(blob.data_ptr(), p2.data_ptr(), s2.data_ptr(), rows, K, None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(p2.cpu().numpy(), packed) and np.array_equal(s2.cpu().numpy(), scales)
+    # the views are a tile-major B as they are (same result as the row-major operand, bit for bit)
+    ap, asc, bp, bsc = operands(48, rows, K, 2, fmt, seed=rows, kind_b="weights")
+    blob2 = hk.pack_weights(dev(bp), dev(bsc), fmt)
+    B, Bs, _ = hk.unpack_weights(blob2)
+    C1 = torch.empty(48, rows, dtype=torch.float32, device="cuda")
+    C2 = torch.empty_like(C1)
+    hk.dispatch_micro(dev(ap), dev(bp), dev(asc), dev(bsc), C1, 2, fmt)
+    hk.dispatch_micro(dev(ap), B, dev(asc), Bs, C2, 2, fmt, layout_b=hk.LAYOUT_TILE)
+    torch.cuda.synchronize()
+    assert torch.equal(C1, C2)
+    corrupt = blob.clone()
+    corrupt[4] = 9
+    with pytest.raises(RuntimeError, match="blob"):
+        hk.unpack_weights(corrupt)
+
+
 def test_tile_major_rejects_bad_shapes(hk):
     ap, asc, bp, bsc = operands(48, 32, 128, 2, 2, seed=3)
     C = torch.empty(48, 32, dtype=torch.float32, device="cuda")
