@@ -159,9 +159,26 @@ def probes(hk, torch, L, inputs, kinputs, C, M, N, K):
             ghz, clk = _clock_ghz(stats.cpu().numpy())
             out["tiled_kernel_" + name] = {"launch_ms_mean": ms, "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12, "shader_clock_ghz": ghz,
                                            "clocks_per_k_tile": clk / ((M // 256) * (N // 256) / 256.0 * (K // 128))}
+        # what each part of the kernel costs: builds of the same kernel without its LDS reads (1), its loads (2), its MFMAs (4)
+        abl = {}
+        names = {0: "full", 1: "no_lds_reads", 2: "no_loads", 3: "mfma_only", 4: "no_mfma", 5: "loads_only", 6: "lds_reads_only", 7: "barriers_and_epilogue_only"}
+        for mask in (0, 1, 2, 3, 4, 5, 6, 7, 0):
+            assert L.mxfp6_probe_tiled_ablation(mask) == 0
+            _, ms = timed_loop(hk, torch, [kinputs[0]], C, 20, 10, 1, 1)
+            ghz, clk = _clock_ghz(stats.cpu().numpy())
+            abl[names[mask]] = {"launch_ms_mean": ms, "shader_clock_ghz": ghz, "kclocks": clk / 1e3}
+        out["tiled_kernel_ablations"] = abl
+        # the builds with MFMAs run at a power-managed clock: what adding a part costs there, in time
+        t = {k: v["launch_ms_mean"] * 1e3 for k, v in abl.items()}
+        out["power_limited_time_split_us"] = {
+            "mfma_only": t["mfma_only"], "lds_reads_added": t["no_loads"] - t["mfma_only"], "loads_added": t["no_lds_reads"] - t["mfma_only"],
+            "rest": t["full"] - t["no_loads"] - t["no_lds_reads"] + t["mfma_only"], "full": t["full"],
+            "what": "launch time (us) of the MFMA-only build, what the LDS reads and what the direct loads add to it when added alone, and what is left of the full kernel's time",
+        }
     finally:
         hk.tk_kernel.set_relayout(prev)
         L.mxfp6_probe_tiled_clock(None)
+        L.mxfp6_probe_tiled_ablation(0)
     return out
 
 

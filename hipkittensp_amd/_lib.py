@@ -73,6 +73,8 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_blob_unpack.argtypes = [vp, vp, vp, ci, ci, vp]
         L.mxfp6_tile_order.restype = ci
         L.mxfp6_tile_order.argtypes = [ci, ci, ci, ci, vp]
+        L.mxfp6_probe_tiled_ablation.restype = ci
+        L.mxfp6_probe_tiled_ablation.argtypes = [ci]
         L.mxfp6_probe_raster.restype = ci
         L.mxfp6_probe_raster.argtypes = [ci, ci]
         L.mxfp6_release_workspaces.restype = ci

@@ -21,6 +21,7 @@ thread_local int g_force = 0;
 thread_local int g_relayout = 1;
 thread_local uint32_t* g_clock_stamps = nullptr;  // mxfp6_probe_tiled_clock
 thread_local int g_raster_group_m = 0, g_raster_no_xcd = 0;  // mxfp6_probe_raster
+thread_local int g_ablation = 0;                              // mxfp6_probe_tiled_ablation
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
 // demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
@@ -175,6 +176,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   g.no_alloc = no_alloc, g.force_split = force_split;
   g.clock_stamps = g_clock_stamps;
   g.raster_group_m = g_raster_group_m, g.raster_no_xcd_remap = g_raster_no_xcd;
+  g.ablation = g_ablation;
   const int force = no_alloc ? 0 : g_force;  // the entry point that allocates nothing takes no override
   hipError_t e;
   if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
@@ -399,6 +401,12 @@ int mxfp6_blob_unpack(const void* blob, void* packed, void* scales, int rows, in
   hipError_t e = mxfp6::launch_tile_operand(body, (uint8_t*)packed, rows, K, 0, s);
   if (e == hipSuccess) e = mxfp6::launch_tile_scales(body + (size_t)rows * (K / 4 * 3), (uint8_t*)scales, rows, K, 0, s);
   return e == hipSuccess ? MXFP6_OK : (int)e;
+}
+
+int mxfp6_probe_tiled_ablation(int mask) {
+  if (mask < 0 || mask > 7) return MXFP6_EINVAL_SHAPE;
+  g_ablation = mask;
+  return MXFP6_OK;
 }
 
 int mxfp6_probe_raster(int group_m, int xcd_remap) {

@@ -121,7 +121,11 @@ struct TiledArgs {
 // FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
 // around updates of all accumulators make the compiler copy them at every output tile, taken or not (3-4 % of an
 // unfused 8192^3 GEMM).
-template <int FA, int FB, typename Out, int TM, int TN, bool FUSED>
+// ABL (measurement only, results are then meaningless): bit 0 leaves out the LDS reads of the operands after the first
+// K-tile of an output tile, bit 1 the direct loads after the prologue, bit 2 the MFMAs after the first K-tile of an output
+// tile.  What the remaining parts of the kernel take, in time and in shader clocks, is how bench.py splits the kernel's
+// time between the matrix cores, the LDS reads and the loads.
+template <int FA, int FB, typename Out, int TM, int TN, bool FUSED, int ABL = 0>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
   typedef Shape<TM, TN> S;
   constexpr int kBM = S::BM, kBN = S::BN, OPA = S::OPA, OPB = S::OPB, NL = S::NL, kLoadsInCompute = S::kLoadsInCompute;
@@ -231,12 +235,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // The resources rA, rB (and rS) are those of the output tile the loads have reached: they move on to the
   // next output tile just before the first load that belongs to it, and past the workgroup's last output
   // tile to empty resources.  INSIDE says that the caller knows kk to lie in the current tile.
+  [[maybe_unused]] bool abl_started = false;  // ABL & 2: the prologue is over
   auto issue_scales = [&]<bool INSIDE>(int grp) __attribute__((always_inline)) {
+    if constexpr ((ABL & 2) != 0) {
+      if (abl_started) return;
+    }
     const int buf = (p0 + grp) & 1;
     const uint32_t dst = lds0 + kScaleBase + buf * kScaleBuf + swave * 1024;
     dma16(rS, sc_a ? dst : dst + kScStage, voff_s, (INSIDE || grp < nk4 ? grp : grp - nk4) * sstep);
   };
   auto issue_one = [&]<bool INSIDE>(int kk, int slot, int n) __attribute__((always_inline)) {
+    if constexpr ((ABL & 2) != 0) {
+      if (abl_started) return;
+    }
     const int t = INSIDE || kk < nkt ? kk : kk - nkt;
     const uint32_t dst = lds0 + slot * kStage;
     if constexpr (SPLIT) {
@@ -296,6 +307,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // so the first MFMA into every accumulator takes zero as its C operand.  between(i) runs after the i-th MFMA.
   auto mma_tile = [&]<bool FIRST, int KM>(auto&& between) __attribute__((always_inline)) {
     constexpr int S0 = 2 * (KM & 1), S1 = S0 + 1;  // op_sel: which byte of the scale registers
+    if ((ABL & 4) && !FIRST) {
+#pragma unroll
+      for (int q = 0; q < 2 * TM * TN; q++) between(q);
+      return;
+    }
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < TM; i++) {
@@ -344,7 +360,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     // other across the steps of a trip they become a few dozen induction variables in scalar registers
     if (!STEADY) asm volatile("" : "+s"(kt));
     const int slotx = GRP == 0 ? stage2 : stage;
-    read_tile.template operator()<KM>(stage, ((p0 + (kt >> 2)) & 1) * kScaleBuf);
+    if (!(ABL & 1) || FIRST) read_tile.template operator()<KM>(stage, ((p0 + (kt >> 2)) & 1) * kScaleBuf);
     __builtin_amdgcn_sched_barrier(0);
     // the loads reach the next output tile: group 0's with K-tile kt+2 at the start of a step, group 1's
     // with K-tile kt+3 in its compute cluster; the scales with group nk4
@@ -634,6 +650,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     wait_vmcnt<NL>();
   }
   barrier();
+  abl_started = true;
   if (wm == 0) {
     run.template operator()<0>();
     barrier();  // every wave executes the same number of barriers
@@ -722,6 +739,22 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     if (bn == 128) gemm_tiled_kernel<FA, FB, Out, 2, 1, true><<<grid, NW * 64, 0, s>>>(ta);
     else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
     else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
+  } else if (g.ablation > 0 && g.ablation < 8) {
+    // measurement instantiations: e2m3 x e2m3, bf16 output, 256 x 256 tiles only
+    if constexpr (FA == 2 && FB == 2 && sizeof(typename Out::type) == 2) {
+      if (bm != 256 || bn != 256) return hipErrorInvalidValue;
+      switch (g.ablation) {
+        case 1: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 1><<<grid, NW * 64, 0, s>>>(ta); break;
+        case 2: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 2><<<grid, NW * 64, 0, s>>>(ta); break;
+        case 3: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 3><<<grid, NW * 64, 0, s>>>(ta); break;
+        case 4: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 4><<<grid, NW * 64, 0, s>>>(ta); break;
+        case 5: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 5><<<grid, NW * 64, 0, s>>>(ta); break;
+        case 6: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 6><<<grid, NW * 64, 0, s>>>(ta); break;
+        default: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 7><<<grid, NW * 64, 0, s>>>(ta); break;
+      }
+    } else {
+      return hipErrorInvalidValue;
+    }
   } else {
     if (bn == 128) gemm_tiled_kernel<FA, FB, Out, 2, 1, false><<<grid, NW * 64, 0, s>>>(ta);
     else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, false><<<grid, NW * 64, 0, s>>>(ta);

@@ -13,7 +13,7 @@
  *   seeded host init + timing shape  kernels/gemm/fp8fp32/profile_utils.cpp:5-45
  *
  * This file is written independently of oracle/mxfp6_oracle.py (bit manipulation here, frexp /
- * ldexp arithmetic there); tests/test_oracle_cross.py requires the two to agree bit for bit, and
+ * ldexp arithmetic there); tests/test_oracle.py requires the two to agree bit for bit, and
  * each is separately pinned against closed forms, brute force and the golden vectors under
  * tests/golden/.
  */

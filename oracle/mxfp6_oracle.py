@@ -14,7 +14,7 @@ mirrors the reference's CPU oracles for its other GEMMs:
   * operand convention (both K-contiguous)    kernels/gemm/bf16fp32/utils.py:28-37
   * output pre-allocated, bf16                analysis/bf16_gemm/mi325x/kernel_8192.cpp:223-224
 
-How each function is pinned (tests/test_oracle_*.py):
+How each function is pinned (tests/test_oracle.py):
   decode_table      closed form, exhaustive 64 codes, vs golden table produced by ROCm's own
                     host fp6 conversion (amd_hip_fp6.h; tests/golden/fp6_tables.json)
   e8m0_to_f32       exhaustive 255 values vs ldexp

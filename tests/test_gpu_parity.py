@@ -682,6 +682,43 @@ def test_gpu_quantiser_bit_exact(hk, fmt, kind):
         assert np.array_equal(scales.cpu().numpy(), es) and np.array_equal(packed.cpu().numpy(), ep)
 
 
+def test_measurement_probes_run_and_leave_results_alone(hk):
+    """The probe kernels bench.py reports (MFMA-only loop on real operand bytes, read-only stream, the tiled kernel's
+    clock stamps, raster override): they run, return plausible counters, and a GEMM with the stamps and a raster override on
+    gives the same bits as without."""
+    from hipkittensp_amd import _lib
+
+    L = _lib.lib()
+    M = N = 512
+    K = 1024
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=77)
+    a, b, sa, sb = dev(ap), dev(bp), dev(asc), dev(bsc)
+    stats = torch.zeros(4, dtype=torch.int32, device="cuda")
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    waves = L.mxfp6_probe_mfma(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), M, N, K, 2, 2, 64, sink.data_ptr(), stats.data_ptr(), None)
+    torch.cuda.synchronize()
+    assert waves > 0 and waves % 8 == 0
+    st = stats.cpu().numpy().astype(np.int64)
+    assert (st[2] - st[0]) % 2**32 > 64 * 4 * 16 and (st[3] - st[1]) % 2**32 > 0      # at least the MFMA issue time, and real time moved
+    assert L.mxfp6_probe_mfma(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), 16, N, K, 2, 2, 64, sink.data_ptr(), stats.data_ptr(), None) == -2
+    buf = torch.zeros(64 << 20, dtype=torch.uint8, device="cuda")
+    assert L.mxfp6_probe_stream(buf.data_ptr(), buf.numel(), 256, 8, stats.data_ptr(), None) == 0
+    assert L.mxfp6_probe_stream(buf.data_ptr(), buf.numel(), 512, 4, stats.data_ptr(), None) == 0
+    assert L.mxfp6_probe_stream(buf.data_ptr(), buf.numel() - 8192, 256, 8, stats.data_ptr(), None) == -2
+    torch.cuda.synchronize()
+    ref = gemm(hk, ap, bp, asc, bsc, kernel=2)
+    assert L.mxfp6_probe_tiled_clock(stats.data_ptr()) == 0 and L.mxfp6_probe_raster(2, 0) == 0
+    try:
+        stats.zero_()
+        got = gemm(hk, ap, bp, asc, bsc, kernel=2)
+        st = stats.cpu().numpy().astype(np.int64)
+        assert (st[2] - st[0]) % 2**32 > 8 * 1024 and (st[3] - st[1]) % 2**32 > 0  # eight K-tiles of MFMA work at least
+    finally:
+        L.mxfp6_probe_tiled_clock(None)
+        L.mxfp6_probe_raster(0, 1)
+    assert np.array_equal(got, ref)
+
+
 # ------------------------------------------------------------------ full-size configurations
 def _sampled_check(hk, ap, asc, bp, bsc, fa, fb, kernel, rng, ns=48, band=256):
     """Full-size check of one configuration: a whole band of `band` consecutive rows of the fp32 result (all N columns, so
