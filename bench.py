@@ -63,11 +63,27 @@ def make_inputs(hk, torch, M, N, K, fmt_a, fmt_b, seed, sets, std_b=1.0):
     return out
 
 
-def timed_loop(hk, torch, inputs, C, steps, warmup, layout_a=0, layout_b=0):
+PREWARM_MS = 40.0  # see timed_loop
+
+
+def timed_loop(hk, torch, inputs, C, steps, warmup, layout_a=0, layout_b=0, prewarm_ms=0.0):
     """W untimed + K timed launches.  Returns (wall seconds for the K steps between two device
     synchronisations, mean per-launch milliseconds from one pair of device events recorded on the
-    launch stream around the K back-to-back launches)."""
+    launch stream around the K back-to-back launches).
+    prewarm_ms > 0: before the W warm-up steps the same launches run untimed for that long.  The chip's power
+    management takes tens of milliseconds to settle under this load (launch durations by rocprofv3 kernel-trace at
+    8192^3: ~290 us for the first ~8 launches after idle, 340-370 us from the 10th to the 25th, back to ~295 us from about
+    the 45th on), so a short W + K would time the transient instead of the kernel."""
     n = len(inputs)
+    if prewarm_ms > 0:
+        t_end = time.perf_counter() + prewarm_ms * 1e-3
+        i = 0
+        while time.perf_counter() < t_end:
+            for _ in range(8):
+                ap, bp, asc, bsc = inputs[i % n]
+                hk.dispatch_micro(ap, bp, asc, bsc, C, layout_a=layout_a, layout_b=layout_b)
+                i += 1
+            torch.cuda.synchronize()
     for i in range(warmup):
         ap, bp, asc, bsc = inputs[i % n]
         hk.dispatch_micro(ap, bp, asc, bsc, C, layout_a=layout_a, layout_b=layout_b)
@@ -284,7 +300,7 @@ def main():
         return
     # the operator as a caller gets it: for this size the library re-lays both operands out tile-major in a
     # pre-pass (one small kernel each) and runs the tiled kernel on them; `value` is the whole step
-    wall, step_ms = timed_loop(hk, torch, inputs, C, args.steps, args.warmup)
+    wall, step_ms = timed_loop(hk, torch, inputs, C, args.steps, args.warmup, prewarm_ms=PREWARM_MS)
     flops = 2.0 * M * N * K
     ms_per_step = wall / args.steps * 1e3
     value = flops / (wall / args.steps) / 1e12
@@ -292,9 +308,9 @@ def main():
     # the same inputs re-laid out beforehand, pre-pass off
     prev = hk.tk_kernel.set_relayout(False)
     kinputs = [(hk.tile_operand(ap), hk.tile_operand(bp), hk.tile_scales(asc, K), hk.tile_scales(bsc, K)) for ap, bp, asc, bsc in inputs]
-    _, ev_ms = timed_loop(hk, torch, kinputs, C, args.steps, args.warmup, 1, 1)
+    _, ev_ms = timed_loop(hk, torch, kinputs, C, args.steps, args.warmup, 1, 1, prewarm_ms=PREWARM_MS)
     # and the tiled kernel on the row-major operands themselves (what the pre-pass avoids)
-    _, row_ms = timed_loop(hk, torch, inputs, C, args.steps, args.warmup)
+    _, row_ms = timed_loop(hk, torch, inputs, C, args.steps, args.warmup, prewarm_ms=PREWARM_MS)
     hk.tk_kernel.set_relayout(prev)
     sustained = probes(hk, torch, _lib.lib(), inputs, kinputs, C, M, N, K)
     del kinputs
@@ -442,6 +458,7 @@ def main():
         "config": {
             "workload": "BASELINE configs[1]: square MXFP6 e2m3 GEMM C=A.B^T, M=N=K=8192, N(0,1) sources quantised per 32-block, bf16 output",
             "M": M, "N": N, "K": K, "fmt_a": "e2m3", "fmt_b": "e2m3", "input_sets": 3,
+            "prewarm": f"{PREWARM_MS:.0f} ms of the same launches, untimed, in front of the warm-up steps of the three 8192^3 loops (the power management's transient after idle)",
         },
         "pct_of_mfma_peak": 100.0 * value / MFMA_PEAK_TFLOPS,
         "roofline": roofline,
