@@ -261,6 +261,7 @@ def main():
     p.add_argument("--cpu-rows", type=int, default=8192)
     p.add_argument("--raster-sweep", action="store_true", help="only time the tiled kernel at 8192^3 (tile-major operands) over raster settings and print one JSON line")
     p.add_argument("--kernel", type=int, default=0, help="with --raster-sweep: kernel code to time as well (18 = the 4-wave schedule)")
+    p.add_argument("--shape", type=int, nargs=3, metavar=("M", "N", "K"), default=None, help="with --raster-sweep: the problem shape (default 8192 8192 8192)")
     p.add_argument("--sweep-settings", choices=["all", "default"], default="all", help="with --raster-sweep: all raster settings, or only the kernel's own (to compare schedules under a profiler)")
     p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the decode run with tile-major weights (used for profiling one layout of the skinny kernel)")
     args = p.parse_args()
@@ -278,7 +279,9 @@ def main():
 
     # ---- headline: configs[1], 8192^3 e2m3 x e2m3 -> bf16
     M = N = K = 8192
-    inputs = make_inputs(hk, torch, M, N, K, 2, 2, seed=1, sets=3)
+    if args.raster_sweep and args.shape:
+        M, N, K = args.shape
+    inputs = make_inputs(hk, torch, M, N, K, 2, 2, seed=1, sets=3 if not (args.raster_sweep and args.shape) else 2)
     C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
     if args.raster_sweep:
         # the tiled kernel alone on tile-major operands, per raster setting (the kernel's own: 4 tile rows per group, XCD remap on)
@@ -298,7 +301,7 @@ def main():
                 _, ms = timed_loop(hk, torch, kin, C, args.steps, args.warmup, 1, 1)
                 hk.tk_kernel.set_kernel(prevk)
                 res[f"kernel={args.kernel}"] = {"launch_ms_mean": ms, "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12}
-        print(json.dumps({"what": "gemm_tiled_kernel, 8192^3 e2m3, operands and scales tile-major, per raster setting", "steps": args.steps, "warmup": args.warmup, "settings": res}))
+        print(json.dumps({"what": f"gemm_tiled_kernel, {M} x {N} x {K} e2m3, operands and scales tile-major, per raster setting", "steps": args.steps, "warmup": args.warmup, "settings": res}))
         return
     # the operator as a caller gets it: for this size the library re-lays both operands out tile-major in a
     # pre-pass (one small kernel each) and runs the tiled kernel on them; `value` is the whole step
