@@ -490,9 +490,9 @@ const char* mxfp6_strerror(int code) {
   switch (code) {
     case MXFP6_OK: return "success";
     case MXFP6_EINVAL_PTR: return "mxfp6: a required pointer is NULL";
-    case MXFP6_EINVAL_SHAPE: return "mxfp6: bad shape (M, N, K >= 0 and K % 32 == 0 required; a forced kernel may need more)";
+    case MXFP6_EINVAL_SHAPE: return "mxfp6: bad shape (M, N, K >= 0 and K % 32 == 0 required; a forced kernel may need more, and 16-byte aligned operands and scales)";
     case MXFP6_EINVAL_FMT: return "mxfp6: format must be 2 (e2m3) or 3 (e3m2)";
-    case MXFP6_EINVAL_ALIGN: return "mxfp6: pointer alignment (packed operands 4 bytes, fp32 input 16 bytes)";
+    case MXFP6_EINVAL_ALIGN: return "mxfp6: pointer alignment (packed operands 4 bytes, C its element size, fp32 / bf16 input and vectors of the fused epilogue 16 bytes)";
     case MXFP6_ENODEVICE: return "mxfp6: the current device is not gfx950 (MI355X)";
     case MXFP6_EINVAL_LAYOUT: return "mxfp6: layout must be 0 (row-major) or 1 (tile-major)";
     case MXFP6_EINVAL_EPILOGUE: return "mxfp6: activation must be 0 (none), 1 (relu), 2 (gelu) or 3 (silu)";

@@ -682,6 +682,42 @@ def test_gpu_quantiser_bit_exact(hk, fmt, kind):
         assert np.array_equal(scales.cpu().numpy(), es) and np.array_equal(packed.cpu().numpy(), ep)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 512), (16, 64, 1024), (64, 96, 1024)])
+def test_operands_not_16_byte_aligned_run_on_the_generic_kernel(hk, M, N, K):
+    """The fast kernels fetch 16 bytes per lane and need 16-byte aligned operands and scales; pointers that are only
+    4-byte aligned are accepted and served by the generic kernel with the same result, and a forced fast kernel refuses
+    them instead of issuing misaligned loads."""
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=M + N)
+    ref = gemm(hk, ap, bp, asc, bsc, kernel=1)
+
+    def shifted(a, off):
+        buf = torch.zeros(a.size + 64, dtype=torch.uint8, device="cuda")
+        buf[off:off + a.size] = torch.from_numpy(a.reshape(-1)).cuda()
+        v = buf[off:off + a.size].view(a.shape)
+        assert v.data_ptr() % 16 == off % 16
+        return v
+
+    for which, off in (("A", 4), ("B", 8), ("As", 4), ("Bs", 12)):
+        A = shifted(ap, off) if which == "A" else dev(ap)
+        B = shifted(bp, off) if which == "B" else dev(bp)
+        As = shifted(asc, off) if which == "As" else dev(asc)
+        Bs = shifted(bsc, off) if which == "Bs" else dev(bsc)
+        C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        hk.dispatch_micro(A, B, As, Bs, C)
+        torch.cuda.synchronize()
+        assert np.array_equal(C.cpu().numpy(), ref), which
+        for forced in ((2,) if K % 128 == 0 and N % 8 == 0 else ()) + ((3,) if M <= 128 and K % 512 == 0 else ()):
+            prev = hk.tk_kernel.set_kernel(forced)
+            try:
+                with pytest.raises(RuntimeError, match="bad shape"):
+                    hk.dispatch_micro(A, B, As, Bs, C)
+            finally:
+                hk.tk_kernel.set_kernel(prev)
+    # operands off by 2 bytes are rejected outright
+    with pytest.raises(RuntimeError, match="alignment"):
+        hk.dispatch_micro(shifted(ap, 2), dev(bp), dev(asc), dev(bsc), torch.empty(M, N, dtype=torch.float32, device="cuda"))
+
+
 def test_measurement_probes_run_and_leave_results_alone(hk):
     """The probe kernels bench.py reports (MFMA-only loop on real operand bytes, read-only stream, the tiled kernel's
     clock stamps, raster override): they run, return plausible counters, and a GEMM with the stamps and a raster override on
