@@ -30,6 +30,9 @@ struct StreamWs {
   size_t bytes = 0;
 };
 std::mutex g_sws_mutex;
+// Held while a call enqueues the kernels that write and then read a stream's workspace (pre-pass + GEMM, GEMM + quantiser):
+// two threads that launch into the same stream must not interleave those, or one's GEMM would read the other's copies.
+std::recursive_mutex g_sws_launch_mutex;
 std::map<std::tuple<int, hipStream_t, int>, StreamWs> g_sws;
 constexpr size_t kStreamWsMax = 128;
 
@@ -63,6 +66,7 @@ uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes) {
 }
 
 hipError_t release_stream_workspaces() {
+  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);
   std::lock_guard<std::mutex> lock(g_sws_mutex);
   if (g_sws.empty()) return hipSuccess;
   int cur = 0;
@@ -113,6 +117,7 @@ bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e)
   const bool conv_a = a_first ? conv1 : conv2, conv_b = a_first ? conv2 : conv1;
   auto bytes_of = [&](int rows) { return (((size_t)rows * (g.K / 4 * 3) + 255) & ~(size_t)255) + (((size_t)rows * ((g.K + 511) / 512) * 16 + 255) & ~(size_t)255); };
   const size_t bytes_a = conv_a ? bytes_of(g.M) : 0, bytes_b = conv_b ? bytes_of(g.N) : 0;
+  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);
   uint8_t* ws = stream_workspace(s, 0, bytes_a + bytes_b);
   if (!ws) return false;
   mxfp6::GemmArgs t = g;
@@ -267,6 +272,7 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
     if (force != 0 || !relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
     return e == hipSuccess ? MXFP6_OK : (int)e;
   }
+  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);
   float* tmp = reinterpret_cast<float*>(stream_workspace(s, 1, (size_t)M * N * 4));
   if (!tmp) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;

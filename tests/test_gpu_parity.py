@@ -718,6 +718,50 @@ def test_operands_not_16_byte_aligned_run_on_the_generic_kernel(hk, M, N, K):
         hk.dispatch_micro(shifted(ap, 2), dev(bp), dev(asc), dev(bsc), torch.empty(M, N, dtype=torch.float32, device="cuda"))
 
 
+def test_two_threads_launching_into_one_stream_share_the_prepass_workspace_safely(hk):
+    """The re-layout pre-pass writes tile-major copies into the stream's workspace and the GEMM behind it reads them: two
+    threads that call the operator on the same stream with different operands must each get their own product (the library
+    enqueues pre-pass and GEMM of one call without letting another call's pre-pass in between)."""
+    import threading
+
+    M = N = 8192
+    K = 4096            # large enough for the pre-pass on both operands
+    g = torch.Generator(device="cuda")
+    g.manual_seed(91)
+    sets = []
+    for _ in range(2):
+        a, sa = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+        b, sb = hk.quantize(torch.randn(N, K, device="cuda", generator=g), 2)
+        sets.append((a, b, sa, sb))
+    want = []
+    for ops in sets:
+        C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        hk.dispatch_micro(*ops, C)
+        want.append(C)
+    torch.cuda.synchronize()
+    assert not torch.equal(want[0], want[1])
+    outs = [[torch.empty(M, N, dtype=torch.bfloat16, device="cuda") for _ in range(6)] for _ in range(2)]
+    errs = []
+
+    def work(t):
+        try:
+            for C in outs[t]:
+                hk.dispatch_micro(*sets[t], C)
+        except Exception as e:  # noqa: BLE001
+            errs.append(e)
+
+    th = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    for x in th:
+        x.start()
+    for x in th:
+        x.join()
+    torch.cuda.synchronize()
+    assert not errs, errs
+    for t in range(2):
+        for C in outs[t]:
+            assert torch.equal(C, want[t])
+
+
 def test_measurement_probes_run_and_leave_results_alone(hk):
     """The probe kernels bench.py reports (MFMA-only loop on real operand bytes, read-only stream, the tiled kernel's
     clock stamps, raster override): they run, return plausible counters, and a GEMM with the stamps and a raster override on
