@@ -194,9 +194,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
     e = mxfp6::launch_gemm_tiled(g, s);
-  } else if (force == 3 || (force >= 7 && force <= 16)) {
+  } else if (force == 3 || (force >= 7 && force <= 16) || (force >= 19 && force <= 21)) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
-    g.skinny_geometry = force == 3 ? 0 : force - 6;
+    g.skinny_geometry = force == 3 ? 0 : force >= 19 ? force - 8 : force - 6;
     e = mxfp6::launch_gemm_skinny(g, s);
   } else if (force == 4) {
     if (!mxfp6::gemm_mid_supports(g)) return MXFP6_EINVAL_SHAPE;
@@ -319,7 +319,7 @@ int mxfp6_set_relayout(int on) {
 }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 18) return MXFP6_EINVAL_KERNEL;
+  if (which < 0 || which > 21) return MXFP6_EINVAL_KERNEL;
   const int prev = g_force;
   g_force = which;
   return prev;

@@ -54,16 +54,19 @@ __device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt
 }  // namespace
 
 // AR = rows of A staged (16, 32 or 64: one or two 32-row accumulator tiles per wave); NW = waves per workgroup;
-// BR = rows of B per workgroup (32, or 16 so that a narrow N still gives every CU a workgroup: the MFMA's other 16
-// rows then mirror the first and their outputs are dropped)
+// BR = rows of B per workgroup (32; 16 so that a narrow N still gives every CU a workgroup: the MFMA's other 16
+// rows then mirror the first and their outputs are dropped; 64 = two 32-row tiles of B against every fragment of A,
+// which halves the bytes of A a workgroup pulls from L2 per byte of B)
 template <int FA, int FB, typename Out, int AR, int NW, int BR, int DB>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                               const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bs,
                                                               typename Out::type* __restrict__ C, int M, int N, int K, int layout_b,
                                                               const Epilogue ep, int nsplit, float* ws_part, int* ws_cnt) {
-  static_assert(BR == 32 || BR == 16, "rows of B per workgroup");
+  static_assert(BR == 64 || BR == 32 || BR == 16, "rows of B per workgroup");
   static_assert(AR == 16 || AR == 32 || AR == 64 || AR == 128, "rows of A");
-  constexpr int TA = AR > 32 ? AR / 32 : 1;   // accumulator tiles per wave
+  constexpr int TA = AR > 32 ? AR / 32 : 1;   // 32-row tiles of A per wave
+  constexpr int TB = BR == 64 ? 2 : 1;        // 32-row tiles of B per wave
+  constexpr int TT = TA * TB;                 // accumulator tiles per wave (tile t of A, tb of B: t * TB + tb)
   constexpr int KT = AR == 128 ? 2 : 4;       // K-tiles per chunk (128 rows of A: half chunks, so that four waves' buffers fit)
   constexpr int kRow = 96 * KT, kPieces = 6 * KT;  // bytes and 16-byte pieces of a row in a chunk
   // a wave's buffer: DB chunks of B (DB = 2: the chunk after the next is on its way from HBM while the next one's A, which
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   constexpr int NBL = kBBuf / 1024, NAL = kABuf / 1024, NAS = kASc / 1024;  // direct loads per chunk: 12 or 6; 6, 12 or 24; 1 or 2
   static_assert(kBBuf % 1024 == 0 && kABuf % 1024 == 0, "whole direct loads");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NW * kBuf];
-  static_assert(NW * kBuf <= 163840 && NW * kBuf >= NW * TA * 16 * 64 * 4 + 64, "LDS budget (the buffers double as the reduction buffer)");
+  static_assert(NW * kBuf <= 163840 && NW * kBuf >= NW * TT * 16 * 64 * 4 + 64, "LDS budget (the buffers double as the reduction buffer)");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -87,15 +90,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
   const int tile = blockIdx.x % ntiles, split = blockIdx.x / ntiles;
   const int n0 = tile * BR;
   const int nrows = min(BR, N - n0);
-  const int rt = BR == 32 ? tile : tile >> 1, half = BR == 32 ? 0 : tile & 1;  // tile-major B: row-tile, and which 16 rows of it
+  // tile-major B: first row-tile of this workgroup, how many it has, and (BR = 16) which 16 rows of it
+  const int rt = BR == 64 ? tile * 2 : BR == 32 ? tile : tile >> 1, half = BR == 16 ? tile & 1 : 0;
+  const int nrt = BR == 64 ? min(2, (N + 31) / 32 - rt) : 1;
 
   // rows that do not exist (n >= N, m >= M) lie past the end of the resource and read as zeros
-  const __amdgpu_buffer_rsrc_t rB = layout_b ? make_rsrc(B + (size_t)rt * 32 * rowbytes, (uint32_t)32 * rowbytes)
+  const __amdgpu_buffer_rsrc_t rB = layout_b ? make_rsrc(B + (size_t)rt * 32 * rowbytes, (uint32_t)nrt * 32 * rowbytes)
                                              : make_rsrc(B + (size_t)n0 * rowbytes, (uint32_t)nrows * rowbytes);
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(A, (uint32_t)M * rowbytes);
   // tile-major B: this workgroup's 32 rows are one row-tile, whose scales are nk4 chunks of 512 bytes (row r at r * 16)
   const int nk4 = nkt / 4;
-  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)rt * nk4 * 512, (uint32_t)nk4 * 512)
+  const __amdgpu_buffer_rsrc_t rBs = layout_b ? make_rsrc(Bs + (size_t)rt * nk4 * 512, (uint32_t)nrt * nk4 * 512)
                                               : make_rsrc(Bs + (size_t)n0 * sbytes, (uint32_t)nrows * sbytes);
   const __amdgpu_buffer_rsrc_t rAs = make_rsrc(As, (uint32_t)M * sbytes);
 
@@ -109,8 +114,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 #pragma unroll
   for (int i = 0; i < NBL; i++) {
     const int o = i * 64 + lane, r = o / kPieces, p = swz(o - r * kPieces, r);
-    constexpr int kPer = BR * 6;  // 16-byte pieces per K-tile of this workgroup's rows
-    voff_b[i] = layout_b ? (o / kPer) * 3072 + half * 1536 + (o % kPer) * 16 : r * rowbytes + p * 16;
+    constexpr int kPer = (BR == 16 ? 16 : 32) * 6;  // 16-byte pieces per K-tile of one row-tile (BR = 16: of this workgroup's half of it)
+    constexpr int kPerRt = KT * kPer;                // ... per chunk
+    voff_b[i] = layout_b ? (o / kPerRt) * (32 * rowbytes) + (o % kPerRt / kPer) * 3072 + half * 1536 + (o % kPer) * 16 : r * rowbytes + p * 16;
   }
 #pragma unroll
   for (int i = 0; i < NAL; i++) {
@@ -118,10 +124,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     voff_a[i] = r * rowbytes + p * 16;
   }
   // scale loads: lane l fetches the 16 bytes (four K-tiles) of row l % 32 (both halves of the wave fetch the same rows;
-  // 64 or more rows of A: of row l, l + 64)
+  // 64 or more rows of A: of row l, l + 64; 64 rows of B: of row l)
   const int ra = AR == 16 ? (r32 & 15) : r32;  // AR = 16: lanes 16-31 mirror rows 0-15 (their outputs are never stored)
   const int rb = BR == 16 ? (r32 & 15) : r32;  // BR = 16: likewise for B
-  const int voff_bs = layout_b ? (half * 16 + rb) * 16 : rb * sbytes;
+  const int voff_bs = BR == 64 ? (layout_b ? h * (nk4 * 512) + r32 * 16 : lane * sbytes) : layout_b ? (half * 16 + rb) * 16 : rb * sbytes;
   const int voff_as = (AR >= 64 ? lane : r32) * sbytes;
 
   const uint32_t buf = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem + wave * kBuf;
@@ -133,7 +139,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const int p = u * 6 + 3 * h + c;
-      b_rd[u][c] = layout_b ? u * (BR * 96) + rb * 96 + ((3 * h + c) ^ ((rb >> 3) & 1)) * 16 : rb * kRow + swz(p, rb) * 16;
+      b_rd[u][c] = layout_b ? u * ((BR == 16 ? 16 : 32) * 96) + rb * 96 + ((3 * h + c) ^ ((rb >> 3) & 1)) * 16 : rb * kRow + swz(p, rb) * 16;
       a_rd[u][c] = kAOff + ra * kRow + swz(p, ra) * 16;
     }
 
@@ -162,9 +168,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     for (int i = 0; i < NAL; i++) dma16_sk(rA, buf + kAOff + i * 1024, voff_a[i], so);
   };
 
-  v16f acc[TA];
+  v16f acc[TT];
 #pragma unroll
-  for (int t = 0; t < TA; t++)
+  for (int t = 0; t < TT; t++)
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[t][e] = 0.f;
 
@@ -179,9 +185,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
       else wait_all_loads();
       const int par = DB == 2 ? j & 1 : 0;
       const uint8_t* bufb = bufp + par * kBBuf;
-      const v4i sc_b = *reinterpret_cast<const v4i*>(bufp + kScOff + par * 1024 + rb * 16);
-      v4i sc_a[TA];
-      v4i fb[KT][3], fa[TA][KT][3];
+      v4i sc_b[TB], sc_a[TA];
+      v4i fb[TB][KT][3], fa[TA][KT][3];
+#pragma unroll
+      for (int tb = 0; tb < TB; tb++) sc_b[tb] = *reinterpret_cast<const v4i*>(bufp + kScOff + par * 1024 + (tb * 32 + rb) * 16);
       const bool odd = KT == 2 && ((c0 + wave + j * NW) & 1);  // half chunks: which two of the four scale bytes
 #pragma unroll
       for (int t = 0; t < TA; t++) sc_a[t] = *reinterpret_cast<const v4i*>(bufp + kAScOff + (t * 32 + ra) * 16);
@@ -189,7 +196,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
       for (int u = 0; u < KT; u++)
 #pragma unroll
         for (int c = 0; c < 3; c++) {
-          fb[u][c] = *reinterpret_cast<const v4i*>(bufb + b_rd[u][c]);
+#pragma unroll
+          for (int tb = 0; tb < TB; tb++) fb[tb][u][c] = *reinterpret_cast<const v4i*>(bufb + b_rd[u][c] + tb * (kBBuf / 2));
 #pragma unroll
           for (int t = 0; t < TA; t++) fa[t][u][c] = *reinterpret_cast<const v4i*>(bufp + a_rd[u][c] + t * (32 * kRow));
         }
@@ -204,72 +212,74 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
         issue_a(c0 + wave + (j + 1) * NW);
       }
 #pragma unroll
-      for (int u = 0; u < KT; u++) {
-        const int sb = (uint32_t)(KT == 4 ? sc_b[u] : odd ? sc_b[u + 2] : sc_b[u]) >> (16 * h);
-        const v8i b0 = __builtin_shufflevector(fb[u][0], fb[u][1], 0, 1, 2, 3, 4, 5, -1, -1);
-        const v8i b1 = __builtin_shufflevector(fb[u][1], fb[u][2], 2, 3, 4, 5, 6, 7, -1, -1);
+      for (int u = 0; u < KT; u++)
 #pragma unroll
-        for (int t = 0; t < TA; t++) {
-          const int sa = (uint32_t)(KT == 4 ? sc_a[t][u] : odd ? sc_a[t][u + 2] : sc_a[t][u]) >> (16 * h);
-          const v8i a0 = __builtin_shufflevector(fa[t][u][0], fa[t][u][1], 0, 1, 2, 3, 4, 5, -1, -1);
-          const v8i a1 = __builtin_shufflevector(fa[t][u][1], fa[t][u][2], 2, 3, 4, 5, 6, 7, -1, -1);
-          acc[t] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[t], sb, sa);
-          acc[t] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[t], sb, sa);
+        for (int tb = 0; tb < TB; tb++) {
+          const int sb = (uint32_t)(KT == 4 ? sc_b[tb][u] : odd ? sc_b[tb][u + 2] : sc_b[tb][u]) >> (16 * h);
+          const v8i b0 = __builtin_shufflevector(fb[tb][u][0], fb[tb][u][1], 0, 1, 2, 3, 4, 5, -1, -1);
+          const v8i b1 = __builtin_shufflevector(fb[tb][u][1], fb[tb][u][2], 2, 3, 4, 5, 6, 7, -1, -1);
+#pragma unroll
+          for (int t = 0; t < TA; t++) {
+            const int sa = (uint32_t)(KT == 4 ? sc_a[t][u] : odd ? sc_a[t][u + 2] : sc_a[t][u]) >> (16 * h);
+            const v8i a0 = __builtin_shufflevector(fa[t][u][0], fa[t][u][1], 0, 1, 2, 3, 4, 5, -1, -1);
+            const v8i a1 = __builtin_shufflevector(fa[t][u][1], fa[t][u][2], 2, 3, 4, 5, 6, 7, -1, -1);
+            acc[t * TB + tb] = mfma_fp6<FB, FA, 0, 0>(b0, a0, acc[t * TB + tb], sb, sa);
+            acc[t * TB + tb] = mfma_fp6<FB, FA, 1, 1>(b1, a1, acc[t * TB + tb], sb, sa);
+          }
         }
-      }
     }
   }
 
-  // sum the K-slices: register e of lane l is C[m = 32 t + l % 32][n = 8*(e/4) + 4*(l/32) + e%4] of accumulator tile t.
+  // sum the K-slices: register e of lane l is C[m = 32 t + l % 32][n = 32 tb + 8*(e/4) + 4*(l/32) + e%4] of accumulator tile t * TB + tb.
   // The buffers double as the reduction buffer once every wave has drained its loads.
   __syncthreads();
   float* part = reinterpret_cast<float*>(smem);
 #pragma unroll
-  for (int t = 0; t < TA; t++)
+  for (int t = 0; t < TT; t++)
 #pragma unroll
-    for (int e = 0; e < 16; e++) part[((wave * TA + t) * 16 + e) * 64 + lane] = acc[t][e];
+    for (int e = 0; e < 16; e++) part[((wave * TT + t) * 16 + e) * 64 + lane] = acc[t][e];
   __syncthreads();
   const bool has_ep = epilogue_any(ep);
-  if (TA == 1 && nsplit > 1) {
+  if (nsplit > 1) {
     // K split between workgroups: every workgroup leaves its partial tile in the workspace; the one that arrives last
     // (a counter per tile) adds them up in split order, so the result does not depend on who that is.  The other
     // workgroups may run on XCDs with L2s of their own: partial tiles and counter are written and read with
     // device-scope atomic accesses, which go past those caches, instead of device-scope fences, which write back and
     // invalidate a whole L2 per wave (measured: 0.2 us per workgroup, one after the other).
-    float* mine_ws = ws_part + ((size_t)tile * nsplit + split) * 1024;
-    for (int idx = tid; idx < 1024; idx += NW * 64) {
-      const int e = idx >> 6, l = idx & 63;
+    // (a workgroup's partial result is TT tiles of 4 KB: idx = (tile of the wave * 16 + register) * 64 + lane)
+    float* mine_ws = ws_part + ((size_t)tile * nsplit + split) * (TT * 1024);
+    for (int idx = tid; idx < TT * 1024; idx += NW * 64) {
       float t = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; w++) t += part[(w * 16 + e) * 64 + l];
+      for (int w = 0; w < NW; w++) t += part[w * (TT * 1024) + idx];
       __hip_atomic_store(mine_ws + idx, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     wait_all_loads();  // stores count there too: the partial tile has arrived before the counter moves
     __syncthreads();
-    int* flag = reinterpret_cast<int*>(smem + NW * 16 * 64 * 4);  // behind the partial tiles
+    int* flag = reinterpret_cast<int*>(smem + NW * TT * 16 * 64 * 4);  // behind the partial tiles
     if (tid == 0) *flag = __hip_atomic_fetch_add(ws_cnt + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1;
     __syncthreads();
     if (!*flag) return;
-    const float* all = ws_part + (size_t)tile * nsplit * 1024;
-    for (int idx = tid; idx < 1024; idx += NW * 64) {
-      const int e = idx >> 6, l = idx & 63;
+    const float* all = ws_part + (size_t)tile * nsplit * (TT * 1024);
+    for (int idx = tid; idx < TT * 1024; idx += NW * 64) {
+      const int tt = idx >> 10, e = (idx >> 6) & 15, l = idx & 63;
       float t = 0.f;
-      for (int q = 0; q < nsplit; q++) t += __hip_atomic_load(all + q * 1024 + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int m = l & 31;
-      const int nl = 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
+      for (int q = 0; q < nsplit; q++) t += __hip_atomic_load(all + q * (TT * 1024) + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int m = (tt / TB) * 32 + (l & 31);
+      const int nl = (tt % TB) * 32 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
       const long nn = (long)n0 + nl;
       if (m < M && nl < BR && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, t, m, nn) : t);
     }
     if (tid == 0) __hip_atomic_store(ws_cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     return;
   }
-  for (int idx = tid; idx < TA * 1024; idx += NW * 64) {
-    const int t = idx >> 10, e = (idx >> 6) & 15, l = idx & 63;
+  for (int idx = tid; idx < TT * 1024; idx += NW * 64) {
+    const int tt = idx >> 10, e = (idx >> 6) & 15, l = idx & 63;
     float s = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; w++) s += part[((w * TA + t) * 16 + e) * 64 + l];
-    const int m = t * 32 + (l & 31);
-    const int nl = 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
+    for (int w = 0; w < NW; w++) s += part[w * (TT * 1024) + idx];
+    const int m = (tt / TB) * 32 + (l & 31);
+    const int nl = (tt % TB) * 32 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3);
     const long nn = (long)n0 + nl;
     if (m < M && nl < BR && nn < N) store1(C + (long)m * N + nn, has_ep ? epilogue_apply(ep, s, m, nn) : s);
   }
@@ -297,7 +307,7 @@ bool gemm_skinny_preferred(const GemmArgs& g) {
 // off with geometry 7 - 9.)  No allocation is possible while the stream is being captured: a capture without a workspace
 // runs unsplit.  At most kWsMax workspaces exist at a time; a further stream runs unsplit.
 namespace {
-constexpr int kWsSlots = 512, kWsTiles = 512;  // (tile, split) pairs and tiles a workspace holds (the automatic split never needs more than 256)
+constexpr int kWsSlots = 512, kWsTiles = 512;  // partial tiles of 4 KB and tiles of C a workspace holds (the automatic choice never needs more)
 constexpr size_t kWsMax = 64;
 struct SplitWs {
   float* part = nullptr;
@@ -387,17 +397,26 @@ hipError_t release_split_workspaces() {
 // a CU and one's first loads run under the other's stream (a workgroup with a short K range is mostly load latency);
 // with at most 16 chunks of K and up to 16 rows of A, two waves per workgroup (eight workgroups share a CU, each wave
 // streams a longer part of K: measured 5 - 13 % at N = 14336 .. 28672, K = 4096 .. 8192, nothing beyond N = 32768).
+// 64 rows of B per workgroup (17 - 128 rows of A): every fragment of A meets two tiles of B, so a workgroup pulls half
+// the bytes of A from L2 per byte of B; the K range is split in two (or four) where N / 64 alone would leave CUs idle.
 // skinny_geometry: 1 - 3 fix the workgroup shape without a split; 4 + 3 * b + log2(split) - 1 (b = 0: 32 rows of B,
-// b = 1: 16 rows) fixes both; 10 = two waves per workgroup.
+// b = 1: 16 rows) fixes both; 10 = two waves per workgroup; 11 - 13 = 64 rows of B with K unsplit / split in 2 / in 4.
 struct SkinnyPlan {
-  int geo, want;   // workgroup shape (1: 32 rows of B, 2: 16 rows, 3: half the waves, 5: two waves) and wanted K split
+  int geo, want;   // workgroup shape (1: 32 rows of B, 2: 16 rows, 3: half the waves, 5: two waves, 6: 64 rows of B) and wanted K split
   unsigned tiles;  // tiles of C (one arrival counter each when K is split)
+  unsigned slots;  // 4 KB partial tiles the split leaves in the workspace
 };
 static SkinnyPlan skinny_plan(const GemmArgs& g) {
   const unsigned wgs32 = (g.N + 31) / 32;
   const int nchunks = g.K / 512, nw = g.M <= 16 ? 8 : 6;
   int geo, want = 1;
-  if (g.M > 32) {
+  if (g.skinny_geometry >= 11 && g.skinny_geometry <= 13) {
+    geo = 6, want = 1 << (g.skinny_geometry - 11);
+  } else if (g.skinny_geometry == 0 && !g.force_split && g.M > 16 && g.M <= 64 && (g.N + 63) / 64 >= 256 && g.K >= 8192) {
+    // wide N, long K, 17 - 64 rows of A: 64 rows of B per workgroup (measured 5 - 13 % at N = 16384 .. 57344, K >= 8192;
+    // 3 - 9 % slower at K = 4096, where a workgroup's K range is too short for its fewer, larger chunks)
+    geo = 6;
+  } else if (g.M > 32) {
     // 33 - 128 rows of A: two or four accumulator tiles per wave, four waves or two (two workgroups per CU), no K split
     geo = g.skinny_geometry == 3 || (g.skinny_geometry == 0 && wgs32 > 256) ? 3 : 1;
   } else if (g.skinny_geometry == 10) {
@@ -418,13 +437,15 @@ static SkinnyPlan skinny_plan(const GemmArgs& g) {
     if (geo != 3)
       while (want < 8 && tiles * want * 2 <= 256 && nchunks / (want * 2) >= kMinChunks * nw) want *= 2;
   }
-  return {geo, want, geo == 2 ? (unsigned)(g.N + 15) / 16 : wgs32};
+  const unsigned tiles = geo == 2 ? (unsigned)(g.N + 15) / 16 : geo == 6 ? (unsigned)(g.N + 63) / 64 : wgs32;
+  const unsigned tt = geo == 6 ? 2 * (g.M > 64 ? 4 : g.M > 32 ? 2 : 1) : 1;  // accumulator tiles per workgroup
+  return {geo, want, tiles, tiles * want * tt};
 }
 
 // Does the K split this call would use fit the scratch array of the entry point that allocates nothing?
 bool gemm_skinny_scratch_fits(const GemmArgs& g) {
   const SkinnyPlan p = skinny_plan(g);
-  return p.want <= 1 || (p.tiles <= (unsigned)kScratchTiles && p.tiles * p.want <= (unsigned)kScratchSlots);
+  return p.want <= 1 || (p.tiles <= (unsigned)kScratchTiles && p.slots <= (unsigned)kScratchSlots);
 }
 
 template <int FA, int FB, typename Out>
@@ -439,7 +460,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     // nothing is allocated: the split uses this device's scratch array, whose counters are cleared by a small kernel in
     // front of the launch (the array keeps whatever the previous call left)
     if (want > 1) {
-      if (tiles > (unsigned)kScratchTiles || tiles * want > (unsigned)kScratchSlots) return hipErrorInvalidValue;  // the entry point checked this already
+      if (tiles > (unsigned)kScratchTiles || plan.slots > (unsigned)kScratchSlots) return hipErrorInvalidValue;  // the entry point checked this already
       unsigned char* base = nullptr;
       const hipError_t e = scratch_of_current_device(&base);
       if (e != hipSuccess) return e;
@@ -450,7 +471,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
       if (ce != hipSuccess) return ce;
       nsplit = want;
     }
-  } else if (want > 1 && tiles <= (unsigned)kWsTiles && tiles * want <= (unsigned)kWsSlots) {
+  } else if (want > 1 && tiles <= (unsigned)kWsTiles && plan.slots <= (unsigned)kWsSlots) {
     ws = split_workspace(s);
     if (ws.part) nsplit = want;
   }
@@ -460,7 +481,9 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
       g.A, g.B, g.As, g.Bs, (T*)g.C, g.M, g.N, g.K, g.layout_b, g.ep, nsplit, ws.part, ws.cnt)
   // two chunks of B per wave (17 - 32 and 65 - 128 rows of A: measured 3 - 15 % and 3 - 6 %); forced geometry 1: one
   const bool db = g.skinny_geometry != 1;
-  if (g.M > 64) {
+  if (geo == 6) {
+    if (g.M > 64) MXFP6_SK(128, 4, 64); else if (g.M > 32) MXFP6_SK(64, 3, 64); else MXFP6_SK(32, 4, 64);
+  } else if (g.M > 64) {
     if (geo == 3) MXFP6_SK(128, 2, 32); else if (db) MXFP6_SKD(128, 4, 32, 2); else MXFP6_SK(128, 4, 32);
   } else if (g.M > 32) {
     if (geo == 3) MXFP6_SK(64, 2, 32); else MXFP6_SK(64, 4, 32);  // two chunks of B and three waves: measured level with this

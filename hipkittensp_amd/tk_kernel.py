@@ -41,6 +41,8 @@ KERNEL_SKINNY_32_SPLIT = (10, 11, 12)  # 32 rows of B, K range split between 2 /
 KERNEL_SKINNY_16_SPLIT = (13, 14, 15)  # 16 rows of B, likewise
 KERNEL_SKINNY_2WAVES = 16  # 32 rows of B, two waves per workgroup (wide N, short K)
 KERNEL_TILED_128x128 = 17  # tiled kernel with output tiles of 128 x 128
+KERNEL_SKINNY_64 = 19  # skinny kernel with 64 rows of B per workgroup (two tiles of B against every fragment of A), K unsplit
+KERNEL_SKINNY_64_SPLIT = (20, 21)  # the same with the K range split between 2 / 4 workgroups
 KERNEL_TILED_4WAVE = 18  # the 4-wave interleaved schedule of the tiled kernel (measurement: never chosen automatically)
 
 

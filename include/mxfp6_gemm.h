@@ -108,7 +108,10 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *       7 / 8 / 9: 32 rows of B per workgroup / 16 rows / 32 rows and half the waves, none of them splitting K;
  *       10 / 11 / 12: 32 rows of B, the K range split between 2 / 4 / 8 workgroups; 13 / 14 / 15: the same with 16 rows
  *       (the split takes a workspace of 2 MB per stream at first use; without one, e.g. first use under stream capture,
- *       the launch runs unsplit); 16: 32 rows of B and two waves per workgroup
+ *       the launch runs unsplit); 16: 32 rows of B and two waves per workgroup;
+ *       19 / 20 / 21: 64 rows of B per workgroup (two tiles of B against every fragment of A: half the bytes of A come
+ *       from L2 per byte of B), the K range unsplit / split between 2 / 4 workgroups (the same workspace; a split whose partial
+ *       tiles do not fit it runs unsplit)
  *    4  mid-M kernel (needs 32 < M <= 512, K % 1024 == 0, row-major A)
  *   18  the 4-wave interleaved schedule of the LDS-tiled kernel (one wave per SIMD with a 128 x 128 wave tile; shapes
  *       of kernel 2, no fused epilogue); never chosen automatically, kept to compare the two schedules

@@ -177,13 +177,14 @@ def test_skinny_kernel_vs_oracle(hk, M, N, K, fa, fb):
     # the K range split between 2 / 4 / 8 workgroups per tile of C (more splits than chunks leaves some without work);
     # twice each: the tile counters must be back at zero after a launch
     check(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=hk.tk_kernel.KERNEL_SKINNY_2WAVES), ref, fa, fb, ap, asc, bp, bsc)
-    for kern in hk.tk_kernel.KERNEL_SKINNY_32_SPLIT + hk.tk_kernel.KERNEL_SKINNY_16_SPLIT:
+    check(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=hk.tk_kernel.KERNEL_SKINNY_64), ref, fa, fb, ap, asc, bp, bsc)  # 64 rows of B per workgroup
+    for kern in hk.tk_kernel.KERNEL_SKINNY_32_SPLIT + hk.tk_kernel.KERNEL_SKINNY_16_SPLIT + hk.tk_kernel.KERNEL_SKINNY_64_SPLIT:
         for _ in range(2):
             check(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kern), ref, fa, fb, ap, asc, bp, bsc)
 
 
-@pytest.mark.parametrize("kernel", [7, 8, 9, 11, 13, 16])
-@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 2080, 1536), (5, 17408, 1024), (64, 4096, 2048), (100, 2080, 1536), (128, 17408, 1024)])
+@pytest.mark.parametrize("kernel", [3, 7, 8, 9, 11, 13, 16, 19, 20])
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 4096), (32, 2080, 1536), (5, 17408, 1024), (64, 4096, 2048), (100, 2080, 1536), (128, 17408, 1024), (40, 16416, 8192)])
 def test_skinny_geometries_tile_major_weights(hk, kernel, M, N, K):
     """Each geometry with tile-major weights and scales (16 rows per workgroup read half of every 3 KB tile) against the
     generic kernel on the row-major operands; ragged N only row-major."""
