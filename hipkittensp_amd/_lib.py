@@ -77,6 +77,10 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_probe_tiled_ablation.argtypes = [ci]
         L.mxfp6_probe_raster.restype = ci
         L.mxfp6_probe_raster.argtypes = [ci, ci]
+        L.mxfp6_probe_ksplit.restype = ci
+        L.mxfp6_probe_ksplit.argtypes = [ci]
+        L.mxfp6_probe_ksplit_plan.restype = ci
+        L.mxfp6_probe_ksplit_plan.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
         L.mxfp6_release_workspaces.restype = ci
         L.mxfp6_release_workspaces.argtypes = []
         L.mxfp6_strerror.restype = ctypes.c_char_p

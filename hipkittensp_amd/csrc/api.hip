@@ -22,6 +22,7 @@ thread_local int g_relayout = 1;
 thread_local uint32_t* g_clock_stamps = nullptr;  // mxfp6_probe_tiled_clock
 thread_local int g_raster_group_m = 0, g_raster_no_xcd = 0;  // mxfp6_probe_raster
 thread_local int g_ablation = 0;                              // mxfp6_probe_tiled_ablation
+thread_local int g_ksplit = 0;                                // mxfp6_probe_ksplit: 0 = where it pays, -1 = wherever possible, 1 = never, n = n shares per output tile
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
 // demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
@@ -36,7 +37,8 @@ std::recursive_mutex g_sws_launch_mutex;
 std::map<std::tuple<int, hipStream_t, int>, StreamWs> g_sws;
 constexpr size_t kStreamWsMax = 128;
 
-// kind 0: pre-pass copies, kind 1: fp32 result of mxfp6_gemm_fused_fp6.  nullptr: no workspace (capture, limit, out of memory).
+// kind 0: pre-pass copies, kind 1: fp32 result of mxfp6_gemm_fused_fp6, kind 2: partial sums of the tiled kernel's K split.
+// nullptr: no workspace (capture, limit, out of memory).
 uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
@@ -63,6 +65,29 @@ uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes) {
     g_sws[{dev, s, kind}] = {p, want};
   }
   return p;
+}
+
+// The tiled kernel's K split for this call, if its shape wants one and this stream has (or can get) the workspace:
+// fills in g.ksplit, g.tile_rows and the workspace pointer.
+void plan_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
+  int rows = 0;
+  size_t part = 0;
+  const int shares = mxfp6::tiled_ksplit_plan(g, g_ksplit, &rows, &part);
+  if (shares <= 1) return;
+  uint8_t* pp = stream_workspace(s, 2, part);
+  if (!pp) return;
+  g.ksplit = shares, g.tile_rows = rows, g.tile_cols = 256;
+  g.ks_part = reinterpret_cast<float*>(pp);
+}
+
+// Automatic path: launches the tiled kernel with its K split if the shape calls for one (and the workspace is there).
+bool launch_tiled_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
+  if (g.no_alloc || g.K == 0 || !mxfp6::gemm_tiled_supports(g)) return false;
+  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
+  plan_ksplit(g, s);
+  if (g.ksplit <= 1) return false;
+  e = mxfp6::launch_gemm_tiled(g, s);
+  return true;
 }
 
 hipError_t release_stream_workspaces() {
@@ -193,6 +218,8 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 2 || force == 5 || force == 6 || force == 17) {
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
+    std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
+    plan_ksplit(g, s);
     e = mxfp6::launch_gemm_tiled(g, s);
   } else if (force == 3 || (force >= 7 && force <= 16) || (force >= 19 && force <= 21)) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
@@ -204,6 +231,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 18) {
     if (!mxfp6::gemm_tiled4_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_tiled4(g, s);
+  } else if (!force_split && (M > 64 || layout_a) && launch_tiled_ksplit(g, s, e)) {
+    // few output tiles, long K: the tiled kernel with K split between workgroups (before the skinny and mid-M kernels,
+    // which it beats there; up to 64 rows of a row-major A stay with the skinny kernel)
   } else if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) {
     e = mxfp6::launch_gemm_skinny(g, s);
   } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
@@ -415,6 +445,25 @@ int mxfp6_probe_tiled_ablation(int mask) {
   return MXFP6_OK;
 }
 
+int mxfp6_probe_ksplit(int shares) {
+  if (shares < -1 || shares > 64) return MXFP6_EINVAL_SHAPE;
+  const int prev = g_ksplit;
+  g_ksplit = shares;
+  return prev;
+}
+
+int mxfp6_probe_ksplit_plan(int M, int N, int K, int layout_a, int shares, int* tile_rows) {
+  if (M <= 0 || N <= 0 || K <= 0 || shares < -1 || shares > 64) return MXFP6_EINVAL_SHAPE;
+  const int rc = check_device();
+  if (rc) return rc;
+  mxfp6::GemmArgs g{nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, 2, 2, false, layout_a, 0};
+  int rows = 0;
+  size_t part = 0;
+  const int n = N % 8 == 0 && K % 128 == 0 ? mxfp6::tiled_ksplit_plan(g, shares, &rows, &part) : 1;
+  if (tile_rows) *tile_rows = n > 1 ? rows : 0;
+  return n;
+}
+
 int mxfp6_probe_raster(int group_m, int xcd_remap) {
   if (group_m < 0 || group_m > 4096) return MXFP6_EINVAL_SHAPE;
   g_raster_group_m = group_m, g_raster_no_xcd = xcd_remap ? 0 : 1;
@@ -511,7 +560,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 114; }
+int mxfp6_abi_version(void) { return 115; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -116,6 +116,7 @@ struct TiledArgs {
   int fmt_c;
   int group_m, xcd_remap;  // raster: tile rows per group (kGroupM unless a measurement overrides it), XCD remap on / off
   uint32_t* stamps;  // measurement only (else null): workgroup 0 leaves its shader-clock and real-time counters here at start and end
+  int nsplit;        // KSPLIT: workgroups that share an output tile, each over K / nsplit (1 otherwise)
 };
 
 // FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
@@ -125,7 +126,12 @@ struct TiledArgs {
 // K-tile of an output tile, bit 1 the direct loads after the prologue, bit 2 the MFMAs after the first K-tile of an output
 // tile.  What the remaining parts of the kernel take, in time and in shader clocks, is how bench.py splits the kernel's
 // time between the matrix cores, the LDS reads and the loads.
-template <int FA, int FB, typename Out, int TM, int TN, bool FUSED, int ABL = 0>
+// KSPLIT: the K range of an output tile is split between args.nsplit workgroups (few output tiles, long K: M of a few
+// hundred rows).  Share s of a tile multiplies K-tiles [s, s + 1) * nkt / nsplit and stores its fp32 sums into matrix s of
+// args.C, which is then a workspace of nsplit matrices [M, N]; ksplit_reduce_kernel adds them in share order and applies
+// the epilogue.  (Summed inside this kernel instead -- partial tiles and arrival counters at device scope, the last
+// wave to arrive adds -- the few waves that end up adding read nsplit tiles each past the L2s: 30 us for 32 MB.)
+template <int FA, int FB, typename Out, int TM, int TN, bool FUSED, int ABL = 0, bool KSPLIT = false>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
   typedef Shape<TM, TN> S;
   constexpr int kBM = S::BM, kBN = S::BN, OPA = S::OPA, OPB = S::OPB, NL = S::NL, kLoadsInCompute = S::kLoadsInCompute;
@@ -136,8 +142,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   __shared__ __attribute__((aligned(1024))) uint8_t smem[S::kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
   const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
-  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK;
-  const int nk4 = (nkt + 3) / 4;  // groups of four K-tiles; tile-major scales hold one 512-byte chunk per 32 rows and group
+  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt_all = K / kBK;
+  const int nk4_all = (nkt_all + 3) / 4;  // groups of four K-tiles; tile-major scales hold one 512-byte chunk per 32 rows and group
+  // K-tiles (and groups of four) of one workgroup's share of an output tile: all of them, or (KSPLIT) a whole number of groups
+  const int nkt = KSPLIT ? nkt_all / args.nsplit : nkt_all, nk4 = KSPLIT ? nkt / 4 : nk4_all;
+  static_assert(!KSPLIT || (!Shape<TM, TN>::SPLIT && sizeof(typename Out::type) == 4 && ABL == 0 && !FUSED), "K split: 256 rows of B, plain fp32 partial sums");
   const bool sc_a = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) < 4;  // this wave loads A's scales (else B's)
 
   // the arguments, read afresh (the empty asm hides from the compiler that the pointer is always the same)
@@ -148,40 +157,60 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   };
 
   // ---- workgroup -> output tiles: workgroup b works on tiles b, b + gridDim.x, ... of tile_order() (common.hpp)
+  // KSPLIT: workgroup b takes share b / tiles of tile b % tiles (shares of one tile start on the same XCD)
   auto tile_of = [&](int bid) __attribute__((always_inline)) {
     const auto g = fresh_args();
+    if constexpr (KSPLIT) {
+      const int tiles = g->tiles_m * g->tiles_n;
+      return bid < tiles * g->nsplit ? tile_order(bid % tiles, g->tiles_m, g->tiles_n, g->group_m, g->xcd_remap) : -1;
+    }
     return tile_order(bid, g->tiles_m, g->tiles_n, g->group_m, g->xcd_remap);
+  };
+  // first K-tile of workgroup-share bid (0 without the split)
+  auto ktile0_of = [&](int bid) __attribute__((always_inline)) {
+    if constexpr (KSPLIT) {
+      const auto g = fresh_args();
+      return bid / (g->tiles_m * g->tiles_n) * nkt;
+    }
+    return 0;
   };
   // Buffer resources of one output tile's operand rows (A and B) and of the scale rows this wave loads.  Edge
   // tiles: rows past M (or N) lie beyond the end of the resource and read as zeros.  tile < 0: resources of
   // length zero, loads through them fetch nothing.
   __amdgpu_buffer_rsrc_t rA, rB, rS;
-  auto operand_rsrc = [&](int tile) __attribute__((always_inline)) {
+  // kt0 (KSPLIT): the share's first K-tile; the resources start there (K-tile kt0 of a row or row-tile is 96 or 3072 bytes
+  // times kt0 into it) and end that much earlier, so that rows past the tile's last still lie beyond the end.
+  auto operand_rsrc = [&](int tile, int kt0) __attribute__((always_inline)) {
     const auto g = fresh_args();
     const int pm = tile < 0 ? 0 : tile & 0xffff, pn = tile < 0 ? 0 : tile >> 16;
     const int rows_a = tile < 0 ? 0 : min(kBM, g->M - pm * kBM), rows_b = tile < 0 ? 0 : min(kBN, g->N - pn * kBN);
     if constexpr (SPLIT) {  // a wave loads one operand only: rA is that operand's resource (no branch at the loads)
       rA = sc_a ? make_rsrc(g->A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes)
                 : make_rsrc(g->B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+    } else if constexpr (KSPLIT) {
+      const uint32_t oa = tile < 0 ? 0 : (uint32_t)kt0 * (layout_a ? 3072 : 96), ob = tile < 0 ? 0 : (uint32_t)kt0 * (layout_b ? 3072 : 96);
+      rA = make_rsrc(g->A + (size_t)pm * kBM * rowbytes + oa, (uint32_t)rows_a * rowbytes - oa);
+      rB = make_rsrc(g->B + (size_t)pn * kBN * rowbytes + ob, (uint32_t)rows_b * rowbytes - ob);
     } else {
       rA = make_rsrc(g->A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
       rB = make_rsrc(g->B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
     }
   };
-  auto scale_rsrc = [&](int tile) __attribute__((always_inline)) {
+  auto scale_rsrc = [&](int tile, int kt0) __attribute__((always_inline)) {
     const auto g = fresh_args();
     const int pm = tile < 0 ? 0 : tile & 0xffff, pn = tile < 0 ? 0 : tile >> 16;
     const int rows_a = tile < 0 ? 0 : min(kBM, g->M - pm * kBM), rows_b = tile < 0 ? 0 : min(kBN, g->N - pn * kBN);
     const uint8_t* sp = sc_a ? g->As : g->Bs;
     const int slay = sc_a ? layout_a : layout_b, srows = sc_a ? rows_a : rows_b, stile = sc_a ? pm : pn;
     const int sheight = sc_a ? kBM : kBN;  // rows per tile of the operand whose scales these are
-    rS = slay ? make_rsrc(sp + (size_t)stile * (sheight / 32) * nk4 * 512, (uint32_t)((srows + 31) / 32) * nk4 * 512)
-              : make_rsrc(sp + (size_t)stile * sheight * sbytes, (uint32_t)srows * sbytes);
+    const uint32_t off = KSPLIT && tile >= 0 ? (uint32_t)(kt0 >> 2) * (slay ? 512 : 16) : 0;  // the share's first group of four K-tiles
+    rS = slay ? make_rsrc(sp + (size_t)stile * (sheight / 32) * nk4_all * 512 + off, (uint32_t)((srows + 31) / 32) * nk4_all * 512 - off)
+              : make_rsrc(sp + (size_t)stile * sheight * sbytes + off, (uint32_t)srows * sbytes - off);
   };
-  int bid_next = blockIdx.x + gridDim.x;
-  int tile_cur = tile_of(blockIdx.x), tile_next = tile_of(bid_next);
-  operand_rsrc(tile_cur);
-  scale_rsrc(tile_cur);
+  int bid_cur = blockIdx.x, bid_next = blockIdx.x + gridDim.x;
+  int tile_cur = tile_of(bid_cur), tile_next = tile_of(bid_next);
+  operand_rsrc(tile_cur, ktile0_of(bid_cur));
+  scale_rsrc(tile_cur, ktile0_of(bid_cur));
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -198,7 +227,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const int o = q * 64 + lane;  // linear 16-byte slot inside the LDS image
     const int r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
     const int vrow = r * rowbytes + c * 16;
-    const int vtile = (q / 3) * (nkt * 3072) + (q % 3) * 1024 + lane * 16;
+    const int vtile = (q / 3) * (nkt_all * 3072) + (q % 3) * 1024 + lane * 16;
     return layout ? vtile : vrow;
   };
 #pragma unroll
@@ -210,7 +239,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // scales: a lane fetches the 16 scale bytes (four K-tiles) of one row; waves 0-3 load A's, 4-7 B's
   const int swave = SPLIT ? wave & 1 : wave & 3;  // which 64 rows of the operand's tile this wave fetches the scales of
   const int srow = swave * 64 + lane, slay = wave < 4 ? layout_a : layout_b;
-  const int voff_s = slay ? (srow >> 5) * nk4 * 512 + (srow & 31) * 16 : srow * sbytes;
+  const int voff_s = slay ? (srow >> 5) * nk4_all * 512 + (srow & 31) * 16 : srow * sbytes;
   const int sstep = slay ? 512 : 16;  // bytes between consecutive groups of four K-tiles
 
   // per-lane LDS read offsets (bytes from the start of a stage): the lane's three pieces 3h..3h+2
@@ -364,14 +393,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     __builtin_amdgcn_sched_barrier(0);
     // the loads reach the next output tile: group 0's with K-tile kt+2 at the start of a step, group 1's
     // with K-tile kt+3 in its compute cluster; the scales with group nk4
-    if (!STEADY && GRP == 0 && kt + 2 == nkt) operand_rsrc(tile_next);
+    if (!STEADY && GRP == 0 && kt + 2 == nkt) operand_rsrc(tile_next, ktile0_of(bid_next));
 #pragma unroll
     for (int n = kLoadsInCompute; n < NL; n++) issue_one.template operator()<STEADY>(kt + 2, stage2, n);
     if (KM == 0) {
-      if (!STEADY && (kt + 4) >> 2 == nk4) scale_rsrc(tile_next);
+      if (!STEADY && (kt + 4) >> 2 == nk4) scale_rsrc(tile_next, ktile0_of(bid_next));
       issue_scales.template operator()<STEADY>((kt + 4) >> 2);
     }
-    if (!STEADY && GRP == 1 && kt + 3 == nkt) operand_rsrc(tile_next);
+    if (!STEADY && GRP == 1 && kt + 3 == nkt) operand_rsrc(tile_next, ktile0_of(bid_next));
     wait_lds_reads();  // this tile's LDS reads are done before anyone may refill its slot
     // the middle 16-byte piece straddles the two operands; naming each fragment as one 384-bit value here
     // makes the register allocator keep it in one tuple, and the MFMAs read sub-tuples of it instead of
@@ -554,7 +583,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     }
     const int N = g->N, N2 = N * (int)sizeof(OutT);  // N2: bytes per row of C
     // the resource ends with the tile's last valid element
-    const __amdgpu_buffer_rsrc_t rC = make_rsrc((OutT*)g->C + (size_t)(tile_cur & 0xffff) * kBM * N + (size_t)(tile_cur >> 16) * kBN,
+    OutT* cbase = (OutT*)g->C;
+    if constexpr (KSPLIT) cbase += (size_t)(bid_cur / (g->tiles_m * g->tiles_n)) * g->M * N;  // this share's matrix
+    const __amdgpu_buffer_rsrc_t rC = make_rsrc(cbase + (size_t)(tile_cur & 0xffff) * kBM * N + (size_t)(tile_cur >> 16) * kBN,
                                                 (uint32_t)((rows_a - 1) * N + rows_b) * (uint32_t)sizeof(OutT));
     const int row_l = wm * (TM * 32) + r32;
     if constexpr (sizeof(OutT) == 2) {
@@ -620,6 +651,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
       if (tile_next < 0) break;
       p0 = (p0 + nk4) & 1;
       tile_cur = tile_next;
+      bid_cur = bid_next;
       bid_next += gridDim.x;
       tile_next = tile_of(bid_next);
     }
@@ -726,11 +758,98 @@ static int tile_shape(const GemmArgs& g) {
   return (t128 < t256 ? 128 : 256) | 256 << 16;
 }
 
+// Sum of the K split's partial matrices, in share order, with the epilogue: 4 consecutive outputs per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restrict__ part, int nsplit, T* __restrict__ C, int M, int N, const Epilogue ep) {
+  const size_t mn = (size_t)M * N, i4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i4 >= mn) return;
+  v4f acc = *reinterpret_cast<const v4f*>(part + i4);
+  for (int s = 1; s < nsplit; s++) {
+    const v4f p = *reinterpret_cast<const v4f*>(part + s * mn + i4);
+    acc += p;
+  }
+  const long m = (long)(i4 / N), n = (long)(i4 % N);
+  if (epilogue_any(ep)) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[e] = epilogue_apply(ep, acc[e], m, n + e);
+  }
+  if constexpr (sizeof(T) == 2) {
+    *reinterpret_cast<u32x2*>(C + i4) = u32x2{pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3])};
+  } else {
+    *reinterpret_cast<v4f*>(C + i4) = acc;
+  }
+}
+
+// K split (KSPLIT instantiations): for problems of few output tiles and long K, typically 100 - 1000 rows of A against a
+// wide weight matrix, where one workgroup per output tile would leave most CUs idle and the kernel would stream B at a
+// fraction of HBM speed.  Shares per tile = CUs / tiles, rounded down to a divisor of the groups of four K-tiles that
+// leaves every share at least kMinShareTiles K-tiles; the tile height is the one whose shares finish first.
+// want: 0 = where it pays (below), -1 = wherever the shape allows it, 1 = never, n > 1 = n shares if the shape allows it
+// (the last three for measurement).  Returns the shares per tile (1: no split) and the tile height and workspace size
+// that go with them.
+// Where it pays (measured on MI355X against the best unsplit kernel, tile-major and row-major operands, N = 2048 .. 28672):
+// with K >= 14336 for up to 512 rows of A (768 from K = 24576 on): 0.45 - 0.85 of the unsplit time, e.g.
+// 256 x 8192 x 28672 108 -> 69 us, 128 x 4096 x 14336 46 -> 24 us; with 8192 <= K < 14336 only while 128-row tiles
+// number 32 or fewer and the skinny kernel is not an option (more than 128 rows of A, or a tile-major A):
+// 256 x 2048 x 8192 28.5 -> 21 us.  Shorter K loses (the partial sums cost 12 - 25 us to write, read and add):
+// 256 x 8192 x 4096 19 -> 24 us.
+constexpr int kMinShareTiles = 8;
+int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes) {
+  if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps || g.K % (4 * kBK) != 0) return 1;
+  const int cus = cu_count() & ~7, groups = g.K / (4 * kBK), nkt = g.K / kBK;
+  if (cus < 8) return 1;
+  if (want == 0) {
+    const long tiles128 = (long)((g.M + 127) / 128) * ((g.N + 255) / 256);
+    const bool pays = nkt >= 112 ? (g.M <= 512 || (nkt >= 192 && g.M <= 768)) : (nkt >= 64 && tiles128 <= 32 && (g.M > 128 || g.layout_a));
+    if (!pays) return 1;
+  }
+  int best = 1, best_rows = 0;
+  double best_us = 0;
+  for (int bm = 256; bm >= 128; bm -= 128) {
+    if ((g.tile_rows && g.tile_rows != bm) || g.tile_cols == 128) continue;
+    const long tiles = (long)((g.M + bm - 1) / bm) * ((g.N + 255) / 256);
+    if (tiles * 2 > cus) continue;
+    for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
+      if (groups % sh != 0 || nkt / sh < kMinShareTiles) {
+        if (want > 1) break;
+        continue;
+      }
+      // a share's K-tiles at this tile height's pace with every CU busy, plus writing and reading the partial matrices
+      const double us = (double)nkt / sh * (bm == 256 ? 1.35 : 0.84) + 2.0 * sh * g.M * g.N * 4.0 / 4e6;
+      if (best_rows == 0 || us < best_us) best = sh, best_rows = bm, best_us = us;
+      if (want > 1) break;
+    }
+  }
+  if (best <= 1) return 1;
+  *rows = best_rows;
+  *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
+  return best;
+}
+
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
-  const int shape = tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
+  const bool ksplit = g.ksplit > 1 && g.ks_part;
+  const int shape = ksplit ? g.tile_rows | 256 << 16 : tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, g.clock_stamps};
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, g.clock_stamps,
+                        ksplit ? g.ksplit : 1};
+  if (ksplit) {
+    if constexpr (sizeof(typename Out::type) != 1) {
+      if ((bm != 128 && bm != 256) || g.K % (4 * kBK * g.ksplit) != 0 || g.K / kBK / g.ksplit < kMinShareTiles || (size_t)g.M * g.N % 4) return hipErrorInvalidValue;
+      TiledArgs tp = ta;  // the shares write fp32 partial matrices into the workspace, without the epilogue
+      tp.C = g.ks_part, tp.ep = Epilogue{};
+      const int grid = grid_size(g, tm * tn * g.ksplit, 1);
+      if (bm == 128) gemm_tiled_kernel<FA, FB, OutF32, 2, 2, false, 0, true><<<grid, NW * 64, 0, s>>>(tp);
+      else gemm_tiled_kernel<FA, FB, OutF32, 4, 2, false, 0, true><<<grid, NW * 64, 0, s>>>(tp);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return e;
+      const size_t quads = (size_t)g.M * g.N / 4;
+      ksplit_reduce_kernel<typename Out::type><<<(unsigned)((quads + 255) / 256), 256, 0, s>>>(g.ks_part, g.ksplit, (typename Out::type*)g.C, g.M, g.N, g.ep);
+      return hipGetLastError();
+    } else {
+      return hipErrorInvalidValue;
+    }
+  }
   const int grid = grid_size(g, tm * tn, bn == 128 ? 2 : 1);  // 128 x 128: 80 KB of LDS, two workgroups per CU
   if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
     if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);

@@ -24,6 +24,8 @@ struct GemmArgs {
   uint32_t* clock_stamps = nullptr;  // tiled kernel, measurement only: four words for workgroup 0's clock / real-time counters at start and end
   int no_alloc = 0;                // skinny kernel: the K split keeps its partial tiles in the library's static scratch array instead of an allocated workspace
   int force_split = 0;             // skinny kernel, M <= 32: split K between this many workgroups (1, 2, 4, 8); 0 = by shape
+  int ksplit = 0;                  // tiled kernel: workgroups that share an output tile (from tiled_ksplit_plan, which also gives tile_rows); needs ks_part
+  float* ks_part = nullptr;        // ... their partial sums: ksplit matrices [M, N] of floats
 };
 
 // the LDS-staged kernels fetch operands and scales 16 bytes per lane: all four tensors must be 16-byte aligned
@@ -34,6 +36,9 @@ inline bool operands_aligned16(const GemmArgs& g) {
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
+// K split of the tiled kernel for this problem (want: 0 = by shape, 1 = never, n = n shares if possible): shares per output tile
+// (1 = none), rows of A per tile and workspace bytes for the partial sums
+int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes);
 bool gemm_tiled4_supports(const GemmArgs& g);  // the 4-wave variant of the tiled kernel (selectable, never chosen automatically)
 hipError_t launch_gemm_tiled4(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);

@@ -28,6 +28,8 @@ library behind include/mxfp6_gemm.h.
 """
 from __future__ import annotations
 
+import ctypes
+
 from . import _lib
 
 E2M3 = 2
@@ -261,6 +263,21 @@ def tile_scales(scales, K: int, untile: bool = False):
 def set_relayout(on: bool) -> bool:
     """Switch the re-layout pre-pass of large row-major GEMMs on / off; returns the previous setting."""
     return bool(_lib.lib().mxfp6_set_relayout(1 if on else 0))
+
+
+def set_k_split(shares: int) -> int:
+    """K split of the tiled kernel for this thread's later calls (measurement / tests): 0 = where it pays (default), 1 = never,
+    -1 = wherever the shape allows it, n > 1 = n workgroups per output tile; returns the previous setting."""
+    return _lib.lib().mxfp6_probe_ksplit(int(shares))
+
+
+def k_split_plan(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, shares: int = 0):
+    """(workgroups per output tile, rows of A per tile) the tiled kernel's K split would use for this shape; (1, 0) = none."""
+    rows = ctypes.c_int(0)
+    n = _lib.lib().mxfp6_probe_ksplit_plan(int(M), int(N), int(K), int(layout_a), int(shares), ctypes.byref(rows))
+    if n < 0:
+        _lib.check(n, "k_split_plan")
+    return n, rows.value
 
 
 def set_kernel(which: int) -> int:

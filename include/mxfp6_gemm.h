@@ -314,6 +314,24 @@ int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int *
 int mxfp6_probe_tiled_ablation(int mask);
 int mxfp6_probe_raster(int group_m, int xcd_remap);
 
+/*
+ * K split of the LDS-tiled kernel (per calling thread, measurement and tests; returns the previous setting).  Problems of
+ * few output tiles and long K (a few hundred rows of A against a wide weight matrix) run with several workgroups per
+ * output tile, each over a part of K: the shares leave their fp32 sums in this stream's workspace (shares * M * N * 4
+ * bytes, hipMallocAsync on the caller's stream at first use, kept until mxfp6_release_workspaces(); on a stream that is
+ * being captured only if it exists already, else the launch runs unsplit) and a second small kernel adds them in share
+ * order and applies the epilogue, so results do
+ * not depend on timing.  0 = where it pays (default: K >= 14336 and up to 512 rows of A, 768 from
+ * K = 24576 on; 8192 <= K < 14336 only with at most 32 tiles of 128 x 256 and no skinny kernel for the shape), 1 = never,
+ * -1 = wherever the shape allows it, n > 1 = n workgroups per output tile where the shape allows it (K a multiple of 512 n,
+ * at least 8 K-tiles of 128 per share, at most half as many output tiles as CUs), else unsplit.
+ * No counterpart in the reference (its GEMMs are one workgroup per 256 x 256 tile, analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61).
+ */
+int mxfp6_probe_ksplit(int shares);
+/* The split the automatic path (shares = 0) or a forced setting would use for a shape on the current device: workgroups per
+ * output tile (1 = none; negative = error code), and in *tile_rows (may be NULL) the rows of A per output tile (0 = none). */
+int mxfp6_probe_ksplit_plan(int M, int N, int K, int layout_a, int shares, int *tile_rows);
+
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);
 

@@ -141,6 +141,59 @@ def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
+@pytest.mark.parametrize("M,N,K,shares", [(256, 512, 4096, 2), (256, 512, 4096, 4), (300, 264, 8192, 4), (128, 768, 8192, 8), (100, 520, 2048, 2),
+                                          (512, 256, 16384, 0), (96, 1024, 14336, 0), (160, 2048, 8192, 0)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
+def test_tiled_kernel_k_split(hk, M, N, K, shares, fa, fb):
+    """The tiled kernel with the K range of every output tile split between several workgroups (few output tiles, long K):
+    fp32 partial matrices in the stream's workspace, summed in share order by a second kernel.  Forced share counts on the
+    forced tiled kernel, and shapes on which the automatic path chooses the split itself (asserted through the plan probe).
+    Against the fp64 oracle; bf16 output = RNE of the fp32 output; a second call gives the same bits; tile-major operands
+    give the same bits as row-major ones; the fused epilogue agrees with the unsplit kernel's."""
+    tk = hk.tk_kernel
+    n, rows = tk.k_split_plan(M, N, K, 0, shares)
+    assert n > 1 and rows in (128, 256), (n, rows)
+    if shares > 1:
+        assert n == shares
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + N + K + shares, kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    kernel = 2 if shares else 0
+    prev = tk.set_k_split(shares)
+    try:
+        got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel)
+        check(got, ref, fa, fb, ap, asc, bp, bsc)
+        assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel), got)
+        cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=kernel)
+        assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+        dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
+        pk = tk.set_kernel(kernel)
+        try:
+            if M % 32 == 0 and N % 32 == 0:
+                C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+                hk.dispatch_micro(hk.tile_operand(dA), hk.tile_operand(dB), hk.tile_scales(dAs, K), hk.tile_scales(dBs, K), C, fa, fb, layout_a=1, layout_b=1)
+                assert np.array_equal(C.cpu().numpy(), got)
+            rng = np.random.default_rng(M + K)
+            bias, rs = dev(rng.standard_normal(N).astype(np.float32)), dev((0.5 + rng.random(M)).astype(np.float32))
+            F = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(dA, dB, dAs, dBs, F, fa, fb, bias=bias, row_scale=rs, activation="silu")
+            tk.set_k_split(1)
+            U = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(dA, dB, dAs, dBs, U, fa, fb, bias=bias, row_scale=rs, activation="silu")
+            assert o.rel_err(F.cpu().numpy(), U.cpu().numpy()) <= 1e-5
+        finally:
+            tk.set_kernel(pk)
+    finally:
+        tk.set_k_split(prev)
+
+
+def test_k_split_is_not_chosen_where_it_does_not_pay(hk):
+    tk = hk.tk_kernel
+    for M, N, K in [(256, 8192, 4096), (1024, 8192, 28672), (4096, 4096, 16384), (256, 8192, 8192), (64, 264, 100 * 128)]:
+        assert tk.k_split_plan(M, N, K)[0] == 1, (M, N, K)
+    assert tk.k_split_plan(256, 8192, 28672)[0] > 1 and tk.k_split_plan(128, 4096, 14336)[0] > 1
+    assert tk.k_split_plan(96, 8192, 8192, 1)[0] > 1 and tk.k_split_plan(96, 8192, 8192, 0)[0] == 1  # the skinny kernel takes a row-major A
+
+
 def test_forced_kernels_reject_shapes_they_cannot_take(hk):
     ap, asc, bp, bsc = operands(64, 64, 64, 2, 2, seed=1)
     with pytest.raises(RuntimeError, match="bad shape"):
