@@ -56,12 +56,11 @@ static constexpr int g_tiled_walk = 1;  // 0 would launch one workgroup per outp
 
 constexpr int kBK = 128;  // the tile has 256 (TM = 4) or 128 (TM = 2) rows of A and 256 (TN = 2) or 128 (TN = 1) rows of B
 constexpr int kGroupM = 4;          // tile rows per raster group
-constexpr int kStages = 3;          // operand ring depth
 constexpr int WM = 2, WN = 4, NW = WM * WN;  // waves: 2 x 4, wave tile (TM * 32) x (TN * 32)
 constexpr int SCL = 1;                       // scale direct loads per wave per slot that carries scales
 // Per tile shape: TM (4 or 2) and TN (2 or 1) 32x32 MFMA tiles per wave in M and N.  A's tile of 128 rows against 256
-// of B is 12 loads of 1 KB for 8 waves: every wave issues two, and the last four of the sixteen lie past the end of
-// A's buffer resource (they fetch nothing and fill padding behind the tile).  128 x 128 (SPLIT): both tiles are 12
+// of B is 12 loads of 1 KB for 8 waves: waves 0-3 issue two each and waves 4-7 one (OPA1), so a batch is five loads for
+// the first wave group and four for the second; the groups are instantiated separately anyway.  128 x 128 (SPLIT): both tiles are 12
 // loads, waves 0-3 load A's and waves 4-7 B's, three each; no padding, and the scales take half the room (waves 2, 3,
 // 6, 7 fetch the same 64 rows as waves 0, 1, 4, 5 again, into the same place, so that every wave issues the same number
 // of loads): 80 KB, two workgroups per CU.
@@ -69,17 +68,23 @@ template <int TM, int TN>
 struct Shape {
   static constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   static constexpr bool SPLIT = TM == 2 && TN == 1;
-  static constexpr int OPA = SPLIT ? 3 : (BM * 96 / 1024 + NW - 1) / NW;  // direct loads per (loading) wave and K-tile for A
+  static constexpr int OPA = SPLIT ? 3 : (BM * 96 / 1024 + NW - 1) / NW;  // direct loads per (loading) wave and K-tile for A (waves 0-3)
+  static constexpr int OPA1 = SPLIT ? 3 : BM * 96 / 1024 / 4 - OPA;        // ... for waves 4-7: what is left of A's tile
   static constexpr int OPB = SPLIT ? 3 : (BN * 96 / 1024 + NW - 1) / NW;  // ... and for B
-  static constexpr int NL = SPLIT ? 3 : OPA + OPB;                        // operand loads per wave and K-tile
+  static constexpr int NL = SPLIT ? 3 : OPA + OPB;                        // operand loads per wave and K-tile, waves 0-3
+  static constexpr int NL1 = SPLIT ? 3 : OPA1 + OPB;                      // ... waves 4-7
+  static_assert(SPLIT || (OPA1 >= 0 && 4 * (OPA + OPA1) * 1024 == BM * 96), "A's tile in whole loads");
   // of the operand loads per wave and K-tile: issued between MFMAs, one after every second of the 2 TM TN
   static constexpr int kLoadsInCompute = TM * TN < 4 ? TM * TN : 4;
-  static constexpr int kAStage = SPLIT ? BM * 96 : OPA * NW * 1024;  // LDS bytes of A's tile (padded)
+  static constexpr int kAStage = BM * 96;                            // LDS bytes of A's tile
   static constexpr int kStage = kAStage + (SPLIT ? BN * 96 : OPB * NW * 1024);  // ... and of a ring slot
   static constexpr int kScStage = (SPLIT ? 128 : 256) * 16;  // bytes of one operand's scales for four K-tiles
   static constexpr int kScaleBuf = 2 * kScStage;
+  // operand ring depth: three slots (two K-tiles in flight); four for the 128 x 256 tile, whose slots are 36 KB (three in
+  // flight: that tile is used where few rows of A meet a wide B, and what bounds it there is how fast B streams from HBM)
+  static constexpr int kStages = TM == 2 && TN == 2 ? 4 : 3;
   static constexpr int kScaleBase = kStages * kStage, kLdsBytes = kScaleBase + 2 * kScaleBuf;
-  static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= NL && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
+  static_assert(kLoadsInCompute >= 0 && kLoadsInCompute <= NL && kLoadsInCompute <= NL1 && 2 * kLoadsInCompute <= 2 * TM * TN, "load slots");
   static_assert(kLdsBytes <= 163840, "LDS budget");
 };
 
@@ -134,8 +139,9 @@ struct TiledArgs {
 template <int FA, int FB, typename Out, int TM, int TN, bool FUSED, int ABL = 0, bool KSPLIT = false>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs args) {
   typedef Shape<TM, TN> S;
-  constexpr int kBM = S::BM, kBN = S::BN, OPA = S::OPA, OPB = S::OPB, NL = S::NL, kLoadsInCompute = S::kLoadsInCompute;
+  constexpr int kBM = S::BM, kBN = S::BN, OPA = S::OPA, OPA1 = S::OPA1, OPB = S::OPB, kLoadsInCompute = S::kLoadsInCompute;
   constexpr int kAStage = S::kAStage, kStage = S::kStage, kScaleBase = S::kScaleBase, kScStage = S::kScStage, kScaleBuf = S::kScaleBuf;
+  constexpr int kStages = S::kStages, D = kStages - 1;  // D: how many K-tiles ahead of the one being multiplied the loads run
   constexpr bool SPLIT = S::SPLIT;
   static_assert(TN == 2 || sizeof(typename Out::type) != 1, "the fp6 epilogue pairs a wave's two tiles of a band");
   // LDS map: [stage 0..2][A tile | B tile] then [scale buffer 0..1][A scales | B scales]
@@ -230,8 +236,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const int vtile = (q / 3) * (nkt_all * 3072) + (q % 3) * 1024 + lane * 16;
     return layout ? vtile : vrow;
   };
+  const int qa0 = wave < 4 ? wave * OPA : 4 * OPA + (wave - 4) * OPA1;  // this wave's first load of A's tile (waves 4-7 issue OPA1 of them)
 #pragma unroll
-  for (int i = 0; i < OPA; i++) voff_a[i] = SPLIT ? load_offset((wave & 3) * OPA + i, sc_a ? layout_a : layout_b) : load_offset(wave * OPA + i, layout_a);
+  for (int i = 0; i < OPA; i++) voff_a[i] = SPLIT ? load_offset((wave & 3) * OPA + i, sc_a ? layout_a : layout_b) : load_offset(qa0 + i, layout_a);
 #pragma unroll
   for (int i = 0; i < OPB; i++) voff_b[i] = SPLIT ? 0 : load_offset(wave * OPB + i, layout_b);
   const int kstep_a = (SPLIT && !sc_a ? layout_b : layout_a) ? 3072 : 96, kstep_b = layout_b ? 3072 : 96;
@@ -257,7 +264,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 
   int p0 = 0;  // scale buffer that holds group 0 of the current output tile
 
-  // ---- loads.  A wave's batch for K-tile t is its NL operand loads (n = 0..OPA-1: A, then B) and,
+  // ---- loads.  A wave's batch for K-tile t is its NL (waves 4-7: NL1) operand loads (n = 0..OPA-1: A, then B) and,
   // when t % 4 == 2, the scale load for the four K-tiles starting at t + 2 (at the end of the batch, so
   // that a wait that leaves a whole batch in flight also covers the scales of the batch before).
   // K-tile (or group of four K-tiles) number kk counts on from the current output tile into the next one.
@@ -273,7 +280,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const uint32_t dst = lds0 + kScaleBase + buf * kScaleBuf + swave * 1024;
     dma16(rS, sc_a ? dst : dst + kScStage, voff_s, (INSIDE || grp < nk4 ? grp : grp - nk4) * sstep);
   };
-  auto issue_one = [&]<bool INSIDE>(int kk, int slot, int n) __attribute__((always_inline)) {
+  auto issue_one = [&]<bool INSIDE, int GRP>(int kk, int slot, int n) __attribute__((always_inline)) {
+    constexpr int OPAg = GRP == 0 ? OPA : OPA1;
     if constexpr ((ABL & 2) != 0) {
       if (abl_started) return;
     }
@@ -282,8 +290,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     if constexpr (SPLIT) {
       dma16(rA, dst + split_base + n * 1024, voff_a[n], t * kstep_a);
     } else {
-      if (n < OPA) dma16(rA, dst + (wave * OPA + n) * 1024, voff_a[n], t * kstep_a);
-      else dma16(rB, dst + kAStage + (wave * OPB + n - OPA) * 1024, voff_b[n - OPA], t * kstep_b);
+      if (n < OPAg) dma16(rA, dst + (qa0 + n) * 1024, voff_a[n], t * kstep_a);
+      else dma16(rB, dst + kAStage + (wave * OPB + n - OPAg) * 1024, voff_b[n - OPAg], t * kstep_b);
     }
   };
 
@@ -369,22 +377,26 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   // (waves 4-7) does the same one barrier later.  A ring slot is refilled only after the barrier by
   // which both groups have finished reading it, and each wave waits for its own share of tile k+1
   // before the barrier that precedes the first read of that tile.
-  // Loads of step k.  Memory cluster, after the LDS reads, both groups: loads kLoadsInCompute.. of tile
-  // k+2 (slot of tile k-1, free since barrier 2k) and the scales.  Compute cluster: loads
-  // 0..kLoadsInCompute-1, for group 0 of the same tile k+2, for group 1 of tile k+3, whose slot is the
+  // Loads of step k, with D = ring slots - 1 (2, or 3 for the 128 x 256 tile).  Memory cluster, after the LDS reads, both
+  // groups: loads kLoadsInCompute.. of tile k+D (slot of tile k-1, free since barrier 2k) and the scales.  Compute
+  // cluster: loads 0..kLoadsInCompute-1, for group 0 of the same tile k+D, for group 1 of tile k+D+1, whose slot is the
   // one of tile k: group 1's compute cluster starts at barrier 2k+2, by which both groups have read
   // tile k.  In program order every tile's batch is contiguous for both groups, so one wait count
-  // serves both: everything older than the newest batch has landed.
-  // The K-tiles of all output tiles of a workgroup form ONE stream: K-tile k+2 or k+3 past the end of
-  // an output tile is K-tile 0, 1 or 2 of the workgroup's next output tile, so the ring never drains
+  // serves both: everything older than the D - 1 newest batches has landed.
+  // The K-tiles of all output tiles of a workgroup form ONE stream: K-tile k+D or k+D+1 past the end of
+  // an output tile is one of the first K-tiles of the workgroup's next output tile, so the ring never drains
   // between output tiles, and the finished tile's stores run while the other group still multiplies.
   // Past the last output tile the stream continues with loads through an empty buffer resource: they
   // fetch nothing and fill ring slots nobody reads, which keeps every step's load and wait pattern the same.
-  // The body is instantiated per group (GRP) and per k mod 4 (KM); STEADY means that tiles k+2, k+3 and
+  // The body is instantiated per group (GRP) and per k mod 4 (KM); STEADY means that tiles k+D, k+D+1 and
   // (for the scales) k+4 lie in the current output tile, so its loads need no choice of descriptor.
-  int stage = 0, stage2 = 2;  // ring slots of tile k and tile k+2
+  int stage = 0, stage2 = D;  // ring slots of tile k and tile k+D
   auto step = [&]<int GRP, int KM, bool STEADY, bool FIRST>(int kt) __attribute__((always_inline)) {
-    constexpr int AHEAD = GRP == 0 ? 2 : 3;
+    constexpr int AHEAD = GRP == 0 ? D : D + 1;
+    constexpr int NL = GRP == 0 ? S::NL : S::NL1;
+    // loads left in flight by this step's wait: the D - 1 newest batches (K-tiles k+2 .. k+D), and the scale loads among
+    // them (the batch of K-tile k+j was issued in step k+j-D and carries one if that step's k mod 4 is 0)
+    constexpr int kInFlight = (D - 1) * NL + SCL * (((KM + 2 - D + 4) % 4 == 0) + (D == 3 && KM == 0));
     // outside the steady state every step derives its offsets and choices from kt on the spot: related to each
     // other across the steps of a trip they become a few dozen induction variables in scalar registers
     if (!STEADY) asm volatile("" : "+s"(kt));
@@ -393,14 +405,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     __builtin_amdgcn_sched_barrier(0);
     // the loads reach the next output tile: group 0's with K-tile kt+2 at the start of a step, group 1's
     // with K-tile kt+3 in its compute cluster; the scales with group nk4
-    if (!STEADY && GRP == 0 && kt + 2 == nkt) operand_rsrc(tile_next, ktile0_of(bid_next));
+    if (!STEADY && GRP == 0 && kt + D == nkt) operand_rsrc(tile_next, ktile0_of(bid_next));
 #pragma unroll
-    for (int n = kLoadsInCompute; n < NL; n++) issue_one.template operator()<STEADY>(kt + 2, stage2, n);
+    for (int n = kLoadsInCompute; n < NL; n++) issue_one.template operator()<STEADY, GRP>(kt + D, stage2, n);
     if (KM == 0) {
       if (!STEADY && (kt + 4) >> 2 == nk4) scale_rsrc(tile_next, ktile0_of(bid_next));
       issue_scales.template operator()<STEADY>((kt + 4) >> 2);
     }
-    if (!STEADY && GRP == 1 && kt + 3 == nkt) operand_rsrc(tile_next, ktile0_of(bid_next));
+    if (!STEADY && GRP == 1 && kt + D + 1 == nkt) operand_rsrc(tile_next, ktile0_of(bid_next));
     wait_lds_reads();  // this tile's LDS reads are done before anyone may refill its slot
     // the middle 16-byte piece straddles the two operands; naming each fragment as one 384-bit value here
     // makes the register allocator keep it in one tuple, and the MFMAs read sub-tuples of it instead of
@@ -410,18 +422,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
 #pragma unroll
     for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
     // own share of the next K-tile has landed; the batch after it may be in flight
-    if (GRP == 1) wait_vmcnt<NL + (KM == 0 ? SCL : 0)>();
+    if (GRP == 1) wait_vmcnt<kInFlight>();
     barrier();
     __builtin_amdgcn_s_setprio(1);
     mma_tile.template operator()<FIRST, KM>([&](int i) __attribute__((always_inline)) {
       if ((i & 1) && i / 2 < kLoadsInCompute) {
         __builtin_amdgcn_sched_barrier(0);
-        issue_one.template operator()<STEADY>(kt + AHEAD, slotx, i / 2);
+        issue_one.template operator()<STEADY, GRP>(kt + AHEAD, slotx, i / 2);
         __builtin_amdgcn_sched_barrier(0);
       }
     });
     __builtin_amdgcn_s_setprio(0);
-    if (GRP == 0) wait_vmcnt<NL + (KM == 0 ? SCL : 0)>();
+    if (GRP == 0) wait_vmcnt<kInFlight>();
     barrier();
     stage = stage == kStages - 1 ? 0 : stage + 1;
     stage2 = stage2 == kStages - 1 ? 0 : stage2 + 1;
@@ -667,19 +679,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     }
   };
   clock_stamp(0);
-  // prologue: scales of the first four K-tiles, K-tiles 0 and 1 and, for group 1, the loads of tile 2
+  // prologue: scales of the first four K-tiles, K-tiles 0 .. D-1 and, for group 1, the loads of tile D
   // that its compute cluster of "step -1" would have issued; tile 0 must have landed everywhere
   issue_scales.template operator()<true>(0);
-#pragma unroll
-  for (int n = 0; n < NL; n++) issue_one.template operator()<true>(0, 0, n);
-#pragma unroll
-  for (int n = 0; n < NL; n++) issue_one.template operator()<false>(1, 1, n);
   if (wm == 1) {
 #pragma unroll
-    for (int n = 0; n < kLoadsInCompute; n++) issue_one.template operator()<false>(2, 2, n);
-    wait_vmcnt<NL + kLoadsInCompute>();
+    for (int n = 0; n < S::NL1; n++) issue_one.template operator()<true, 1>(0, 0, n);
+#pragma unroll
+    for (int t = 1; t < D; t++)
+#pragma unroll
+      for (int n = 0; n < S::NL1; n++) issue_one.template operator()<false, 1>(t, t, n);
+#pragma unroll
+    for (int n = 0; n < kLoadsInCompute; n++) issue_one.template operator()<false, 1>(D, D, n);
+    wait_vmcnt<(D - 1) * S::NL1 + kLoadsInCompute>();
   } else {
-    wait_vmcnt<NL>();
+#pragma unroll
+    for (int n = 0; n < S::NL; n++) issue_one.template operator()<true, 0>(0, 0, n);
+#pragma unroll
+    for (int t = 1; t < D; t++)
+#pragma unroll
+      for (int n = 0; n < S::NL; n++) issue_one.template operator()<false, 0>(t, t, n);
+    wait_vmcnt<(D - 1) * S::NL>();
   }
   barrier();
   abl_started = true;
