@@ -179,8 +179,8 @@ def probes(hk, torch, L, inputs, kinputs, C, M, N, K):
                                            "clocks_per_k_tile": clk / ((M // 256) * (N // 256) / 256.0 * (K // 128))}
         # what each part of the kernel costs: builds of the same kernel without its LDS reads (1), its loads (2), its MFMAs (4)
         abl = {}
-        names = {0: "full", 1: "no_lds_reads", 2: "no_loads", 3: "mfma_only", 4: "no_mfma", 5: "loads_only", 6: "lds_reads_only", 7: "barriers_and_epilogue_only"}
-        for mask in (0, 1, 2, 3, 4, 5, 6, 7, 0):
+        names = {0: "full", 1: "no_lds_reads", 2: "no_loads", 3: "mfma_only", 4: "no_mfma", 6: "lds_reads_only"}
+        for mask in (0, 1, 2, 3, 4, 6, 0):
             assert L.mxfp6_probe_tiled_ablation(mask) == 0
             _, ms = timed_loop(hk, torch, [kinputs[0]], C, 20, 10, 1, 1)
             ghz, clk = _clock_ghz(stats.cpu().numpy())

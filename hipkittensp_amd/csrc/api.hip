@@ -440,7 +440,7 @@ int mxfp6_blob_unpack(const void* blob, void* packed, void* scales, int rows, in
 }
 
 int mxfp6_probe_tiled_ablation(int mask) {
-  if (mask < 0 || mask > 7) return MXFP6_EINVAL_SHAPE;
+  if (mask < 0 || mask > 6 || mask == 5) return MXFP6_EINVAL_SHAPE;
   g_ablation = mask;
   return MXFP6_OK;
 }

@@ -887,9 +887,8 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
         case 2: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 2><<<grid, NW * 64, 0, s>>>(ta); break;
         case 3: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 3><<<grid, NW * 64, 0, s>>>(ta); break;
         case 4: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 4><<<grid, NW * 64, 0, s>>>(ta); break;
-        case 5: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 5><<<grid, NW * 64, 0, s>>>(ta); break;
         case 6: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 6><<<grid, NW * 64, 0, s>>>(ta); break;
-        default: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 7><<<grid, NW * 64, 0, s>>>(ta); break;
+        default: return hipErrorInvalidValue;  // 5 and 7 (no LDS reads and no MFMAs at once) are not built: the register allocator spills in them, which is all they would measure
       }
     } else {
       return hipErrorInvalidValue;

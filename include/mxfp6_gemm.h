@@ -308,8 +308,9 @@ int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int *
  * Ablations of the LDS-tiled kernel (per calling thread, measurement only, 0 = off): while mask != 0, e2m3 x e2m3 bf16
  * GEMMs on 256 x 256 tiles run a build of the kernel without its LDS reads of the operands (bit 0), without its
  * direct loads after the prologue (bit 1), without its MFMAs (bit 2); other calls fail with hipErrorInvalidValue.  The
- * output of such a launch is meaningless.  Timing the seven combinations next to the full kernel (with
- * mxfp6_probe_tiled_clock for the shader clock) shows what each part costs and which ones the power management charges.
+ * output of such a launch is meaningless.  Timing the combinations 1 - 4 and 6 next to the full kernel (with
+ * mxfp6_probe_tiled_clock for the shader clock) shows what each part costs and which ones the power management charges
+ * (5 and 7, no LDS reads and no MFMAs at once, are not built and rejected: those builds spill registers).
  */
 int mxfp6_probe_tiled_ablation(int mask);
 int mxfp6_probe_raster(int group_m, int xcd_remap);

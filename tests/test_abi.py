@@ -111,6 +111,11 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     L.mxfp6_set_kernel.restype = ci
     L.mxfp6_set_kernel.argtypes = [ci]
     assert L.mxfp6_set_kernel(99) == -9 and L.mxfp6_set_kernel(-1) == -9
+    # measurement switches validate their argument too (they only set per-thread state: no GPU needed)
+    assert L.mxfp6_probe_tiled_ablation(5) == -2 and L.mxfp6_probe_tiled_ablation(7) == -2 and L.mxfp6_probe_tiled_ablation(0) == 0
+    assert L.mxfp6_probe_ksplit(65) == -2 and L.mxfp6_probe_ksplit(-2) == -2
+    prev = L.mxfp6_probe_ksplit(1)
+    assert prev == 0 and L.mxfp6_probe_ksplit(0) == 1
     assert L.mxfp6_set_kernel(2) == 0
     import threading
     seen = []
