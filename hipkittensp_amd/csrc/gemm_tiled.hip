@@ -47,10 +47,26 @@
 // wave ride in the compute cluster, one after every second MFMA, and the rest follow the LDS reads of the
 // memory cluster (measured: memory cluster 1110 -> 720 clocks, 7 % / 11 % less time per GEMM for
 // row-major / tile-major operands).
+//
+// This file is compiled five times (build.py): once as it is, which gives the host-side part (shape checks, tile
+// shape and grid, time estimates, the K split's plan and reduction, the dispatcher), and once per pair of operand
+// formats with -DMXFP6_TILED_FMT=22 / 23 / 32 / 33, which gives that pair's kernel instantiations and launcher: the
+// instantiations are what takes the time to compile, and four objects compile side by side.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace mxfp6 {
+
+// defined in the host-side object, used by the launchers of the per-format objects
+int tiled_grid_size(const GemmArgs& g, int tiles, int per_cu);
+int tiled_tile_shape(const GemmArgs& g);
+hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s);
+constexpr int kMinShareTiles = 8;  // K-tiles a share of a K split has at least
+// defined in the per-format objects
+hipError_t launch_gemm_tiled_fmt22(const GemmArgs& g, hipStream_t s);
+hipError_t launch_gemm_tiled_fmt23(const GemmArgs& g, hipStream_t s);
+hipError_t launch_gemm_tiled_fmt32(const GemmArgs& g, hipStream_t s);
+hipError_t launch_gemm_tiled_fmt33(const GemmArgs& g, hipStream_t s);
 
 static constexpr int g_tiled_walk = 1;  // 0 would launch one workgroup per output tile everywhere (no walk)
 
@@ -714,6 +730,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   clock_stamp(1);
 }
 
+#ifndef MXFP6_TILED_FMT  // ---------------------------------------------------------------- the host-side object
+
 bool gemm_tiled_supports(const GemmArgs& g) {
   // any M; N % 8 keeps every run of 8 bf16 outputs whole and aligned; K in whole K-tiles; 32-bit byte
   // offsets inside one tile's operand rows and inside one tile's rows of C
@@ -738,7 +756,7 @@ static int cu_count() {
 // scales of the next output tile are fetched with the last group of four K-tiles of the current one
 // and must have two steps to land: K-tile counts of 4n+1 (and fewer than four K-tiles) keep one
 // workgroup per tile.
-static int grid_size(const GemmArgs& g, int tiles, int per_cu) {
+int tiled_grid_size(const GemmArgs& g, int tiles, int per_cu) {
   const int cus = (cu_count() & ~7) * per_cu;  // whole multiples of the 8 XCDs keep the tile -> XCD mapping of the walk
   const int nkt = g.K / kBK;
   if (g_tiled_walk == 0 || nkt < 4 || nkt % 4 == 1 || cus < 8) return tiles;
@@ -770,7 +788,7 @@ double tiled_estimate_us(const GemmArgs& g, int rows, int cols) {
 
 // Tile shape: 256 x 256 unless tiles of 128 rows of A, or of 128 x 128, fill the machine better (the fp6 output needs
 // 256 columns).  Returns rows | cols << 16.
-static int tile_shape(const GemmArgs& g) {
+int tiled_tile_shape(const GemmArgs& g) {
   if (g.tile_rows == 128 || g.tile_rows == 256) return g.tile_rows | (g.tile_cols == 128 && g.tile_rows == 128 && !g.fmt_c ? 128 : 256) << 16;
   const double t256 = tiled_estimate_us(g, 256, 256), t128 = tiled_estimate_us(g, 128, 256);
   const double t128n = g.fmt_c ? 1e30 : tiled_estimate_us(g, 128, 128);
@@ -813,7 +831,6 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
 // number 32 or fewer and the skinny kernel is not an option (more than 128 rows of A, or a tile-major A):
 // 256 x 2048 x 8192 28.5 -> 21 us.  Shorter K loses (the partial sums cost 12 - 25 us to write, read and add):
 // 256 x 8192 x 4096 19 -> 24 us.
-constexpr int kMinShareTiles = 8;
 int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes) {
   if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps || g.K % (4 * kBK) != 0) return 1;
   const int cus = cu_count() & ~7, groups = g.K / (4 * kBK), nkt = g.K / kBK;
@@ -846,10 +863,28 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
   return best;
 }
 
+hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s) {
+  const size_t quads = (size_t)g.M * g.N / 4;
+  const unsigned blocks = (unsigned)((quads + 255) / 256);
+  if (g.f32out) ksplit_reduce_kernel<float><<<blocks, 256, 0, s>>>(g.ks_part, g.ksplit, (float*)g.C, g.M, g.N, g.ep);
+  else ksplit_reduce_kernel<uint16_t><<<blocks, 256, 0, s>>>(g.ks_part, g.ksplit, (uint16_t*)g.C, g.M, g.N, g.ep);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s) {
+  if (g.fmt_a == 2 && g.fmt_b == 2) return launch_gemm_tiled_fmt22(g, s);
+  if (g.fmt_a == 2 && g.fmt_b == 3) return launch_gemm_tiled_fmt23(g, s);
+  if (g.fmt_a == 3 && g.fmt_b == 2) return launch_gemm_tiled_fmt32(g, s);
+  if (g.fmt_a == 3 && g.fmt_b == 3) return launch_gemm_tiled_fmt33(g, s);
+  return hipErrorInvalidValue;
+}
+
+#else  // ----------------------------------------------------------------------------------- one pair of operand formats
+
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const bool ksplit = g.ksplit > 1 && g.ks_part;
-  const int shape = ksplit ? g.tile_rows | 256 << 16 : tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
+  const int shape = ksplit ? g.tile_rows | 256 << 16 : tiled_tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
   const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, g.clock_stamps,
                         ksplit ? g.ksplit : 1};
@@ -858,19 +893,16 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
       if ((bm != 128 && bm != 256) || g.K % (4 * kBK * g.ksplit) != 0 || g.K / kBK / g.ksplit < kMinShareTiles || (size_t)g.M * g.N % 4) return hipErrorInvalidValue;
       TiledArgs tp = ta;  // the shares write fp32 partial matrices into the workspace, without the epilogue
       tp.C = g.ks_part, tp.ep = Epilogue{};
-      const int grid = grid_size(g, tm * tn * g.ksplit, 1);
+      const int grid = tiled_grid_size(g, tm * tn * g.ksplit, 1);
       if (bm == 128) gemm_tiled_kernel<FA, FB, OutF32, 2, 2, false, 0, true><<<grid, NW * 64, 0, s>>>(tp);
       else gemm_tiled_kernel<FA, FB, OutF32, 4, 2, false, 0, true><<<grid, NW * 64, 0, s>>>(tp);
-      hipError_t e = hipGetLastError();
-      if (e != hipSuccess) return e;
-      const size_t quads = (size_t)g.M * g.N / 4;
-      ksplit_reduce_kernel<typename Out::type><<<(unsigned)((quads + 255) / 256), 256, 0, s>>>(g.ks_part, g.ksplit, (typename Out::type*)g.C, g.M, g.N, g.ep);
-      return hipGetLastError();
+      const hipError_t e = hipGetLastError();
+      return e != hipSuccess ? e : launch_ksplit_reduce(g, s);
     } else {
       return hipErrorInvalidValue;
     }
   }
-  const int grid = grid_size(g, tm * tn, bn == 128 ? 2 : 1);  // 128 x 128: 80 KB of LDS, two workgroups per CU
+  const int grid = tiled_grid_size(g, tm * tn, bn == 128 ? 2 : 1);  // 128 x 128: 80 KB of LDS, two workgroups per CU
   if constexpr (sizeof(typename Out::type) == 1) {  // fp6 output: one instantiation, with the fused step (a no-op when nothing is fused)
     if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
     else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
@@ -901,12 +933,16 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   return hipGetLastError();
 }
 
-hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s) {
-#define MXFP6_CASE(FA, FB) \
-  if (g.fmt_a == FA && g.fmt_b == FB) return g.fmt_c ? launch<FA, FB, OutFp6>(g, s) : g.f32out ? launch<FA, FB, OutF32>(g, s) : launch<FA, FB, OutBf16>(g, s);
-  MXFP6_CASE(2, 2) MXFP6_CASE(2, 3) MXFP6_CASE(3, 2) MXFP6_CASE(3, 3)
-#undef MXFP6_CASE
-  return hipErrorInvalidValue;
+#define MXFP6_PASTE2(a, b) a##b
+#define MXFP6_PASTE(a, b) MXFP6_PASTE2(a, b)
+hipError_t MXFP6_PASTE(launch_gemm_tiled_fmt, MXFP6_TILED_FMT)(const GemmArgs& g, hipStream_t s) {
+  constexpr int FA = MXFP6_TILED_FMT / 10, FB = MXFP6_TILED_FMT % 10;
+  static_assert((FA == 2 || FA == 3) && (FB == 2 || FB == 3), "MXFP6_TILED_FMT: 22, 23, 32 or 33");
+  return g.fmt_c ? launch<FA, FB, OutFp6>(g, s) : g.f32out ? launch<FA, FB, OutF32>(g, s) : launch<FA, FB, OutBf16>(g, s);
 }
+#undef MXFP6_PASTE
+#undef MXFP6_PASTE2
+
+#endif  // MXFP6_TILED_FMT
 
 }  // namespace mxfp6
