@@ -312,6 +312,55 @@ def test_skinny_k_split_chosen_by_shape_streams_and_capture(hk):
         torch.cuda.synchronize()
 
 
+def test_tiled_k_split_streams_and_capture(hk):
+    """The tiled kernel's K split on a shape where the automatic path chooses it (a few hundred rows of A, long K):
+    against the generic kernel; two streams at once, each with its own workspace of partial sums; under stream capture
+    on a stream that has its workspace already (captured with the split) and replayed with eager work in between."""
+    M, N, K = 192, 1024, 16384
+    assert hk.tk_kernel.k_split_plan(M, N, K)[0] > 1
+    g = torch.Generator(device="cuda"); g.manual_seed(9)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2)
+    ref = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    prev = hk.tk_kernel.set_kernel(1)
+    try:
+        hk.dispatch_micro(a, b, asc, bsc, ref)
+    finally:
+        hk.tk_kernel.set_kernel(prev)
+    torch.cuda.synchronize()
+    refn = ref.cpu().numpy()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda") for _ in range(6)] for _ in streams]
+    torch.cuda.synchronize()
+    for i in range(6):
+        for st, out in zip(streams, outs):
+            with torch.cuda.stream(st):
+                hk.dispatch_micro(a, b, asc, bsc, out[i])
+    torch.cuda.synchronize()
+    for out in outs:
+        for C in out:
+            assert o.rel_err(C.cpu().numpy(), refn) <= TOL_TIGHT
+    # capture on a stream that has launched the split before (torch's recipe: warm up on the side stream, then capture there)
+    side = torch.cuda.Stream()
+    Cg = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        hk.dispatch_micro(a, b, asc, bsc, Cg)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = Cg.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        hk.dispatch_micro(a, b, asc, bsc, Cg)
+    for rep in range(3):
+        Cg.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Cg, eager), f"replay {rep}"
+        hk.dispatch_micro(a, b, asc, bsc, torch.empty_like(Cg))
+        torch.cuda.synchronize()
+
+
 # ------------------------------------------------------------------ mid-M kernel
 @pytest.mark.parametrize("M,N,K", [(33, 32, 1024), (64, 64, 1024), (48, 100, 2048), (64, 520, 3072), (65, 40, 1024), (128, 96, 4096), (100, 33, 2048),
                                    (200, 72, 1024), (256, 160, 5120), (129, 31, 3072),
