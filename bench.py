@@ -373,7 +373,7 @@ def main():
     dwall, dev_ms = timed_loop(hk, torch, dinputs, dC, args.steps, args.warmup)
     dbytes = algorithmic_bytes(dM, dN, dK)
     d_achieved = dbytes / (dev_ms * 1e-3) / 1e9
-    dtile = dbatched = None
+    dtile = dbatched = dmid = None
     if args.layouts == "both":
         dtin = [(ap, hk.tile_operand(bp), asc, hk.tile_scales(bsc, dK)) for ap, bp, asc, bsc in dinputs]
         dtwall, dtev_ms = timed_loop(hk, torch, dtin, dC, args.steps, args.warmup, 0, 1)
@@ -383,7 +383,26 @@ def main():
         bC = torch.empty(bM, dN, dtype=torch.bfloat16, device="cuda")
         bwall, bev_ms = timed_loop(hk, torch, [(ba, bt, bas, bst) for _, bt, _, bst in dtin], bC, args.steps, args.warmup, 0, 1)
         bbytes = algorithmic_bytes(bM, dN, dK)
-        del dtin
+        # a few hundred rows of A against the same weights: the tiled kernel with K split between workgroups, and the
+        # best kernel without the split (mxfp6_probe_ksplit(1))
+        mM = 256
+        ma, mas = hk.quantize(torch.randn(mM, dK, device="cuda"), 2, layout=hk.tk_kernel.LAYOUT_TILE)
+        mC = torch.empty(mM, dN, dtype=torch.bfloat16, device="cuda")
+        mins = [(ma, bt, mas, bst) for _, bt, _, bst in dtin]
+        _, mev_ms = timed_loop(hk, torch, mins, mC, args.steps, args.warmup, 1, 1)
+        prev_split = hk.tk_kernel.set_k_split(1)
+        try:
+            _, mev_ms_unsplit = timed_loop(hk, torch, mins, mC, args.steps, args.warmup, 1, 1)
+        finally:
+            hk.tk_kernel.set_k_split(prev_split)
+        mbytes, mflops = algorithmic_bytes(mM, dN, dK), 2.0 * mM * dN * dK
+        dmid = {
+            "what": "M=256 against the same tile-major weights (A tile-major too): gemm_tiled_kernel with K split between workgroups + ksplit_reduce_kernel",
+            "k_split_plan": list(hk.tk_kernel.k_split_plan(mM, dN, dK, 1)), "launch_ms_mean": mev_ms, "achieved": mbytes / (mev_ms * 1e-3) / 1e9,
+            "unit": "GB/s", "frac": mbytes / (mev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "tflops": mflops / (mev_ms * 1e-3) / 1e12,
+            "launch_ms_mean_without_split": mev_ms_unsplit, "algorithmic_bytes_per_launch": mbytes,
+        }
+        del dtin, mins
         dbatched = {
             "what": "M=64 against the same tile-major weights", "achieved": bbytes / (bev_ms * 1e-3) / 1e9, "unit": "GB/s",
             "frac": bbytes / (bev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "launch_ms_mean": bev_ms, "algorithmic_bytes_per_launch": bbytes,
@@ -444,6 +463,7 @@ def main():
         },
         "tile_major_weights": dtile,
         "batched_m64": dbatched,
+        "batched_m256": dmid,
     }
 
     line = {
