@@ -19,16 +19,18 @@
  * Work is queued on `hip_stream` (a hipStream_t; NULL = the null stream); no function synchronises the
  * device or the stream.
  *
- * Device memory.  Three entry-point families take a workspace from the stream-ordered allocator
- * (hipMallocAsync on `hip_stream`), at most once per (device, stream) and size class, and keep it until
- * mxfp6_release_workspaces():
+ * Device memory.  Four uses take a workspace from the stream-ordered allocator
+ * (hipMallocAsync on `hip_stream`), at most once per (device, stream) and use (regrown when a later call
+ * needs more), and keep it until mxfp6_release_workspaces():
  *   - the gemm entry points on large row-major problems (re-layout pre-pass, see mxfp6_set_relayout):
  *     up to 0.78 (M + N) K bytes;
  *   - mxfp6_gemm_fused_fp6 on shapes the LDS-tiled kernel does not run: 4 M N bytes;
  *   - the gemm entry points on decode shapes whose K range is split between workgroups (M <= 32, N <= 2048,
- *     K >= 24576): 2 MB.
- * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K split are left out
- * (same results, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
+ *     K >= 24576): 2 MB;
+ *   - the gemm entry points on problems of few output tiles and long K (a few hundred rows of A, K >= 8192; see
+ *     mxfp6_probe_ksplit), where the LDS-tiled kernel splits K between workgroups: shares * 4 M N bytes, at most 64 MB.
+ * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K splits are left out
+ * (same results up to the order of fp32 sums, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
  * hipErrorStreamCaptureUnsupported where it would need a new one.  mxfp6_gemm_noalloc never allocates.
  *
  * Alignment.  Pointers are accepted from 4-byte alignment on (C: its element size).  The fast kernels
