@@ -231,9 +231,9 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (force == 18) {
     if (!mxfp6::gemm_tiled4_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_tiled4(g, s);
-  } else if (!force_split && (M > 64 || layout_a) && launch_tiled_ksplit(g, s, e)) {
+  } else if (!force_split && launch_tiled_ksplit(g, s, e)) {
     // few output tiles, long K: the tiled kernel with K split between workgroups (before the skinny and mid-M kernels,
-    // which it beats there; up to 64 rows of a row-major A stay with the skinny kernel)
+    // which it beats there; the plan leaves up to 64 rows of a row-major A to the skinny kernel)
   } else if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) {
     e = mxfp6::launch_gemm_skinny(g, s);
   } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {

@@ -838,7 +838,7 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
   if (want == 0) {
     const long tiles128 = (long)((g.M + 127) / 128) * ((g.N + 255) / 256);
     const bool pays = nkt >= 112 ? (g.M <= 512 || (nkt >= 192 && g.M <= 768)) : (nkt >= 64 && tiles128 <= 32 && (g.M > 128 || g.layout_a));
-    if (!pays) return 1;
+    if (!pays || (g.M <= 64 && !g.layout_a)) return 1;  // up to 64 rows of a row-major A are the skinny kernel's
   }
   int best = 1, best_rows = 0;
   double best_us = 0;

@@ -972,16 +972,18 @@ def test_cfg3_decode_skinny(hk):
         check(got, ref, 2, 2)
 
 
-@pytest.mark.parametrize("M", [64, 128])
+@pytest.mark.parametrize("M", [64, 128, 256])
 def test_batched_decode_full_size(hk, M):
-    """cfg3's weights against 64 and 128 rows of A (the skinny kernel with two and four accumulator tiles per wave, the latter
-    in half chunks): sampled rows and columns against the fp64 oracle, the first 256 columns in full, and the whole result
-    against the generic kernel; row-major and tile-major weights."""
+    """cfg3's weights against 64, 128 and 256 rows of A.  The automatic path takes the skinny kernel for 64 rows (two
+    accumulator tiles per wave) and the tiled kernel with K split between workgroups for 128 and 256; the skinny kernel's
+    128-row form (four accumulator tiles, half chunks) is forced as well.  Sampled rows and columns against the fp64
+    oracle, the first 256 columns in full, and the whole result against the generic kernel; row-major and tile-major weights."""
     N, K = 8192, 28672
+    assert (hk.tk_kernel.k_split_plan(M, N, K)[0] > 1) == (M > 64)
     ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=30 + M, kind_a="normal", kind_b="weights")
     _sampled_check(hk, ap, asc, bp, bsc, 2, 2, 0, np.random.default_rng(M), ns=64)
     ref = o.gemm_ref(ap, bp[:256], asc, bsc[:256], acc=np.float64)
-    check(gemm(hk, ap, bp[:256], asc, bsc[:256], kernel=3), ref, 2, 2)
+    check(gemm(hk, ap, bp[:256], asc, bsc[:256], kernel=3 if M <= 128 else 0), ref, 2, 2)
     a, b, sa, sb = dev(ap), dev(bp), dev(asc), dev(bsc)
     full = torch.empty(M, N, dtype=torch.float32, device="cuda")
     prev = hk.tk_kernel.set_kernel(1)
@@ -990,11 +992,16 @@ def test_batched_decode_full_size(hk, M):
     finally:
         hk.tk_kernel.set_kernel(prev)
     bt, sbt = hk.tile_operand(b), hk.tile_scales(sb, K)
-    for B, Bs, lb in ((b, sb, 0), (bt, sbt, 1)):
-        C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
-        hk.dispatch_micro(a, B, sa, Bs, C, layout_b=lb)
-        torch.cuda.synchronize()
-        assert o.rel_err(C.cpu().numpy(), full.cpu().numpy()) <= TOL_TIGHT, lb
+    for kernel in ((0, 3) if M <= 128 else (0,)):
+        prev = hk.tk_kernel.set_kernel(kernel)
+        try:
+            for B, Bs, lb in ((b, sb, 0), (bt, sbt, 1)):
+                C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+                hk.dispatch_micro(a, B, sa, Bs, C, layout_b=lb)
+                torch.cuda.synchronize()
+                assert o.rel_err(C.cpu().numpy(), full.cpu().numpy()) <= TOL_TIGHT, (kernel, lb)
+        finally:
+            hk.tk_kernel.set_kernel(prev)
 
 
 def test_cfg4_mixed_formats(hk):
