@@ -236,7 +236,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     // which it beats there; the plan leaves up to 64 rows of a row-major A to the skinny kernel)
   } else if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) {
     e = mxfp6::launch_gemm_skinny(g, s);
-  } else if (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g))) {
+  } else if (!mxfp6::gemm_wide_n_prefers_tiled(g) && (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g)))) {
     e = mxfp6::launch_gemm_mid(g, s);
   } else if (mxfp6::gemm_tiled_supports(g)) {
     if (!relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);

@@ -48,6 +48,7 @@ double mid_estimate_us(const GemmArgs& g);
 hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
 bool gemm_skinny_preferred(const GemmArgs& g);  // over the mid-M kernel, by shape
+bool gemm_wide_n_prefers_tiled(const GemmArgs& g);  // 17 - 64 rows of A against a very wide B: the tiled kernel's 128-row tile beats the skinny and mid-M kernels
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_scratch_fits(const GemmArgs& g);  // no_alloc: the K split this call would use fits the static scratch array
 hipError_t release_split_workspaces();             // returns every K-split workspace to the stream-ordered allocator
