@@ -294,16 +294,19 @@ bool gemm_skinny_supports(const GemmArgs& g) {
 // against 22 at 64 x 8192 x 8192, 48 against 66 at K = 28672, level at N = 28672).  With 65 - 128 rows a wave's chunk is
 // mostly A (24 KB of 30), so few bytes of B are in flight per CU: it wins by 10 - 15 % while one round of workgroups covers
 // N and loses by 25 % beyond, where the mid-M kernel's 64 rows of B per workgroup halve the traffic of A.
-// Very wide N (a vocabulary projection, fused gate / up matrices) with 17 - 64 rows of A: the tiled kernel's 128-row
-// tile walks through hundreds of output tiles with all of A in every tile, while here every 32 or 64 rows of B pull A
-// through L2 again.  Measured (us, this kernel -> 128 x 256 tiles; tile-major B): 32 x 40960 x 8192 62 -> 55,
-// 64 x 57344 x 8192 102 -> 73, 64 x 128256 x 4096 128 -> 82, 24 x 128256 x 8192 164 -> 141; row-major B only from 33 rows
-// on: 64 x 57344 x 8192 105 -> 95, 64 x 128256 x 8192 212 -> 188 (24 - 32 rows level); at N = 28672 this kernel wins.
-// (The mid-M kernel is behind both there: 48 x 57344 x 8192 row-major 109 us.)
+// Wide N (a vocabulary projection, fused gate / up matrices) with 17 - 128 rows of A: the tiled kernel's tiles hold all
+// of A and walk through hundreds of output tiles, while here every 32 or 64 rows of B pull A through L2 again.  Measured
+// (us, this kernel -> tiled kernel; tile-major B): 32 x 40960 x 8192 62 -> 55, 64 x 57344 x 8192 102 -> 73,
+// 64 x 128256 x 4096 128 -> 82, 24 x 128256 x 8192 164 -> 141, and with its 128 x 128 tiles (two workgroups per CU) already
+// at N = 28672: 32 x 28672 x 8192 41 -> 38, 64 x 28672 x 8192 50 -> 42; row-major B from 33 rows on and N >= 57344:
+// 64 x 57344 x 8192 105 -> 95, 64 x 128256 x 8192 212 -> 188 (24 - 32 rows level), and from 65 rows on from N = 24576:
+// 128 x 28672 x 8192 72 (mid-M kernel) -> 60; with K <= 4096 already from 33 rows and N = 24576 (a workgroup's K range is
+// then eight chunks or fewer, mostly load latency): 64 x 28672 x 4096 29 -> 23.  At N = 14336 and below this kernel wins.
 bool gemm_wide_n_prefers_tiled(const GemmArgs& g) {
-  if (g.M <= 16 || g.M > 64 || !gemm_tiled_supports(g)) return false;
+  if (g.M <= 16 || g.M > 128 || !gemm_tiled_supports(g)) return false;
   const long tiles = (g.N + 255) / 256;
-  return g.layout_b ? tiles >= 160 : g.M > 32 && tiles >= 224;
+  if (g.layout_b) return tiles >= 160 || (tiles >= 96 && g.M >= 24);
+  return g.M > 64 ? tiles >= 96 : g.M > 32 && (tiles >= 224 || (tiles >= 96 && g.K <= 4096));
 }
 
 bool gemm_skinny_preferred(const GemmArgs& g) {

@@ -768,7 +768,12 @@ int tiled_grid_size(const GemmArgs& g, int tiles, int per_cu) {
 // at a higher clock and meet less L2 contention).  Constants measured on MI355X with tile-major B: 8192-wide
 // problems of 64 K-tiles took 57.7 / 62.7 / 70.1 / 86.9 us with 64 / 128 / 192 / 256 tiles of 256 rows and
 // 43.5 / 46.5 / 53.9 us with 128 / 192 / 256 tiles of 128 rows, 34.1 / 38.9 / 73.8 us with 128 / 256 / 512 tiles of
-// 128 x 128; row-major B costs about 28 % more, and no shape runs faster than its bytes stream.
+// 128 x 128; row-major B costs about 28 % more, and no shape runs faster than its bytes stream.  Rounds after the first
+// are cheaper for 256-row tiles (the walk overlaps tile changes, and the launch's slow start is paid once): 8192^3 is
+// four rounds in 290 - 300 us, not 4 x 87.  The streaming floor grows with the workgroups that stream side by side:
+// measured on problems whose B comes from HBM (N = 28672 and 57344, K = 8192, 8 - 128 rows of A), tile-major B: 4.5 TB/s
+// with 112 workgroups, 5.2 - 5.6 with 224 and more (128 x 128 tiles, two per CU, reach that at N = 28672 where 128 x 256
+// tiles have 112: 37 us against 42 - 45); row-major B: 2.7 - 2.9 TB/s with 112, 4.2 - 4.5 with 224.
 double tiled_estimate_us(const GemmArgs& g, int rows, int cols) {
   int cus = cu_count();
   if (cus <= 0) cus = 256;
@@ -776,12 +781,13 @@ double tiled_estimate_us(const GemmArgs& g, int rows, int cols) {
   const long full = tiles / cus;
   const double f = (double)(tiles % cus) / cus;
   const double c0 = cols == 128 ? 0.45 : rows == 128 ? 0.62 : 0.85, c1 = cols == 128 ? 0.10 : rows == 128 ? 0.22 : 0.50;
-  const double per_ktile = full * (c0 + c1) + (f > 0 ? c0 + c1 * f * f : 0.0);
+  const double later = rows == 256 && full >= 1 ? 0.82 : 1.0;  // what a round after the first costs against the first
+  const double per_ktile = (full >= 1 ? (c0 + c1) * (1.0 + (full - 1) * later) : 0.0) + (f > 0 ? (c0 + c1 * f * f) * later : 0.0);
   const double layout = 1.0 + (g.layout_b ? 0.0 : 0.28) - (g.layout_a ? 0.05 : 0.0);
-  // few rows of A against a large B is a streaming problem: measured 3.5 / 3.3 TB/s (tile-major B, 128- / 256-row
-  // tiles) and 2.35 / 2.1 TB/s (row-major B)
   const double bytes = (0.75 + 1.0 / 32) * g.K * ((double)g.M + g.N) + 2.0 * g.M * g.N;
-  const double stream = bytes / (g.layout_b ? (rows == 128 ? 3.5e6 : 3.3e6) : (rows == 128 ? 2.35e6 : 2.1e6));
+  const double side_by_side = (double)(tiles < (long)cus * (cols == 128 ? 2 : 1) ? tiles : (long)cus * (cols == 128 ? 2 : 1)) / 224.0;
+  const double conc = g.layout_b ? 0.6 + 0.4 * side_by_side : 0.3 + 0.7 * side_by_side;
+  const double stream = bytes / ((g.layout_b ? 5.4e6 : 4.5e6) * (conc < 1.0 ? conc : 1.0));
   const double compute = 3.0 + (g.K / kBK) * per_ktile * layout;
   return compute > stream ? compute : stream;
 }
@@ -825,19 +831,19 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
 // want: 0 = where it pays (below), -1 = wherever the shape allows it, 1 = never, n > 1 = n shares if the shape allows it
 // (the last three for measurement).  Returns the shares per tile (1: no split) and the tile height and workspace size
 // that go with them.
-// Where it pays (measured on MI355X against the best unsplit kernel, tile-major and row-major operands, N = 2048 .. 28672):
-// with K >= 14336 for up to 512 rows of A (768 from K = 24576 on): 0.45 - 0.85 of the unsplit time, e.g.
-// 256 x 8192 x 28672 108 -> 69 us, 128 x 4096 x 14336 46 -> 24 us; with 8192 <= K < 14336 only while 128-row tiles
-// number 32 or fewer and the skinny kernel is not an option (more than 128 rows of A, or a tile-major A):
-// 256 x 2048 x 8192 28.5 -> 21 us.  Shorter K loses (the partial sums cost 12 - 25 us to write, read and add):
-// 256 x 8192 x 4096 19 -> 24 us.
+// Where it pays (measured on MI355X against the best unsplit kernel over 360 shapes, M = 8 .. 2048, N = 1024 .. 57344,
+// tile-major and row-major B), in output tiles of 256 x 256: with K >= 14336 up to 64 tiles (128 from K = 24576 on):
+// 0.45 - 0.9 of the unsplit time, e.g. 256 x 8192 x 28672 108 -> 63 us, 128 x 4096 x 14336 46 -> 24 us, 1024 x 1024 x 16384
+// 60 -> 34 us; with 8192 <= K < 14336 up to 32 tiles where the skinny kernel is not an option (more than 128 rows of A, or
+// a tile-major A): 256 x 2048 x 8192 28.5 -> 21 us, 768 x 2048 x 8192 33 -> 27 us.  More tiles or a shorter K lose (the
+// partial sums cost 12 - 25 us to write, read and add): 256 x 8192 x 4096 19 -> 24 us, 512 x 8192 x 8192 36 -> 40 us.
 int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes) {
   if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps || g.K % (4 * kBK) != 0) return 1;
   const int cus = cu_count() & ~7, groups = g.K / (4 * kBK), nkt = g.K / kBK;
   if (cus < 8) return 1;
   if (want == 0) {
-    const long tiles128 = (long)((g.M + 127) / 128) * ((g.N + 255) / 256);
-    const bool pays = nkt >= 112 ? (g.M <= 512 || (nkt >= 192 && g.M <= 768)) : (nkt >= 64 && tiles128 <= 32 && (g.M > 128 || g.layout_a));
+    const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
+    const bool pays = nkt >= 112 ? (tiles256 <= 64 || (nkt >= 192 && tiles256 <= 128)) : (nkt >= 64 && tiles256 <= 32 && (g.M > 128 || g.layout_a));
     if (!pays || (g.M <= 64 && !g.layout_a)) return 1;  // up to 64 rows of a row-major A are the skinny kernel's
   }
   int best = 1, best_rows = 0;

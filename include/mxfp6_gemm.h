@@ -324,8 +324,8 @@ int mxfp6_probe_raster(int group_m, int xcd_remap);
  * bytes, hipMallocAsync on the caller's stream at first use, kept until mxfp6_release_workspaces(); on a stream that is
  * being captured only if it exists already, else the launch runs unsplit) and a second small kernel adds them in share
  * order and applies the epilogue, so results do
- * not depend on timing.  0 = where it pays (default: K >= 14336 and up to 512 rows of A, 768 from
- * K = 24576 on; 8192 <= K < 14336 only with at most 32 tiles of 128 x 256 and no skinny kernel for the shape), 1 = never,
+ * not depend on timing.  0 = where it pays (default: K >= 14336 and at most 64 output tiles of 256 x 256, 128 from
+ * K = 24576 on; 8192 <= K < 14336 only with at most 32 tiles and no skinny kernel for the shape), 1 = never,
  * -1 = wherever the shape allows it, n > 1 = n workgroups per output tile where the shape allows it (K a multiple of 512 n,
  * at least 8 K-tiles of 128 per share, at most half as many output tiles as CUs), else unsplit.
  * No counterpart in the reference (its GEMMs are one workgroup per 256 x 256 tile, analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61).

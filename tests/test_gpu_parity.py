@@ -188,9 +188,11 @@ def test_tiled_kernel_k_split(hk, M, N, K, shares, fa, fb):
 
 def test_k_split_is_not_chosen_where_it_does_not_pay(hk):
     tk = hk.tk_kernel
-    for M, N, K in [(256, 8192, 4096), (1024, 8192, 28672), (4096, 4096, 16384), (256, 8192, 8192), (64, 264, 100 * 128)]:
+    # short K, or more output tiles of 256 x 256 than the rule allows (64 from K = 14336, 32 from K = 8192), or the skinny kernel's shapes
+    for M, N, K in [(256, 8192, 4096), (4096, 4096, 16384), (512, 8192, 8192), (2048, 2048, 8192), (2048, 4096, 14336), (64, 264, 100 * 128)]:
         assert tk.k_split_plan(M, N, K)[0] == 1, (M, N, K)
-    assert tk.k_split_plan(256, 8192, 28672)[0] > 1 and tk.k_split_plan(128, 4096, 14336)[0] > 1
+    for M, N, K in [(256, 8192, 28672), (128, 4096, 14336), (1024, 1024, 16384), (768, 2048, 8192), (1024, 8192, 28672)]:
+        assert tk.k_split_plan(M, N, K)[0] > 1, (M, N, K)
     assert tk.k_split_plan(96, 8192, 8192, 1)[0] > 1 and tk.k_split_plan(96, 8192, 8192, 0)[0] == 1  # the skinny kernel takes a row-major A
 
 
