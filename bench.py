@@ -252,6 +252,72 @@ def cpu_baseline(inputs, M_sample, gpu_f32):
     }
 
 
+def dispatch_sweep(hk, torch, full):
+    """How good is the automatic kernel choice?  For every shape of a grid (rows of A x a set of (N, K) pairs x both
+    layouts of B; A row-major) the call is timed with the automatic choice and with every kernel / tile shape forced in
+    turn, the tiled kernel also with its K split wherever the shape allows one.  Reports, per shape, the automatic time,
+    the best forced time and which kernel that was, and the shapes where the automatic choice is more than 8 % behind.
+    Small shapes (below about 15 us) are bound by the host side of the Python operator and only scatter."""
+    tk = hk.tk_kernel
+    if full:
+        shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096),
+                  (8192, 28672), (2048, 8192), (5120, 16384), (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096)]
+        rows_of_a = [8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 2048]
+    else:
+        shapes = [(8192, 8192), (28672, 8192), (8192, 28672), (57344, 8192), (1024, 16384)]
+        rows_of_a = [16, 32, 64, 128, 256, 512, 1024]
+    forced = (("tiled", 2, 1), ("tiled_128x256", 5, 1), ("tiled_256x256", 6, 1), ("tiled_128x128", 17, 1), ("skinny", 3, 0), ("mid", 4, 0), ("tiled_k_split", 2, -1))
+
+    def time_us(sets, C, lay, kernel, k_split, reps=10):
+        prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
+        try:
+            for i in range(3):
+                hk.dispatch_micro(*sets[i % len(sets)], C, layout_b=lay)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(reps):
+                hk.dispatch_micro(*sets[i % len(sets)], C, layout_b=lay)
+            e1.record()
+            torch.cuda.synchronize()
+        except RuntimeError:
+            return None  # the forced kernel does not take this shape
+        finally:
+            tk.set_kernel(prev_k)
+            tk.set_k_split(prev_s)
+        return e0.elapsed_time(e1) / reps * 1e3
+
+    per_shape, behind = [], []
+    for N, K in shapes:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1)
+        bs = [hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2) for _ in range(2)]
+        bts = [(hk.tile_operand(b), hk.tile_scales(sc, K)) for b, sc in bs]
+        for M in rows_of_a:
+            a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+            C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+            for lay in (1, 0):
+                sets = [(a, (bts if lay else bs)[i][0], asc, (bts if lay else bs)[i][1]) for i in range(2)]
+                auto = time_us(sets, C, lay, 0, 0)
+                times = {}
+                for name, kernel, k_split in forced:
+                    if (name == "skinny" and M > 128) or (name == "mid" and (M <= 32 or M > 512)):
+                        continue
+                    t = time_us(sets, C, lay, kernel, k_split)
+                    if t is not None:
+                        times[name] = t
+                best = min(times, key=times.get)
+                rec = {"M": M, "N": N, "K": K, "layout_b": "tile" if lay else "row", "auto_us": round(auto, 1), "best_us": round(times[best], 1),
+                       "best": best, "auto_over_best": round(auto / times[best], 3)}
+                per_shape.append(rec)
+                if rec["auto_over_best"] > 1.08:
+                    behind.append(rec)
+    ratios = sorted(r["auto_over_best"] for r in per_shape)
+    return {"what": "automatic kernel choice against every forced kernel, tile shape and K split; e2m3 x e2m3, bf16 out, A row-major", "shapes": len(per_shape),
+            "within_8_percent": sum(1 for r in ratios if r <= 1.08), "median_auto_over_best": ratios[len(ratios) // 2], "worst_auto_over_best": ratios[-1],
+            "behind_by_more_than_8_percent": behind, "per_shape": per_shape}
+
+
 def main():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -263,6 +329,8 @@ def main():
     p.add_argument("--kernel", type=int, default=0, help="with --raster-sweep: kernel code to time as well (18 = the 4-wave schedule)")
     p.add_argument("--shape", type=int, nargs=3, metavar=("M", "N", "K"), default=None, help="with --raster-sweep: the problem shape (default 8192 8192 8192)")
     p.add_argument("--sweep-settings", choices=["all", "default"], default="all", help="with --raster-sweep: all raster settings, or only the kernel's own (to compare schedules under a profiler)")
+    p.add_argument("--dispatch-sweep", choices=["small", "full"], default=None,
+                   help="only compare the automatic kernel choice with every forced kernel / tile shape / K split over a grid of shapes and print one JSON line")
     p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the decode run with tile-major weights (used for profiling one layout of the skinny kernel)")
     args = p.parse_args()
     if args.gpus != 1:
@@ -276,6 +344,10 @@ def main():
     from hipkittensp_amd import _lib
 
     _lib.lib()  # fail loudly if the HIP library is missing
+
+    if args.dispatch_sweep:
+        print(json.dumps(dispatch_sweep(hk, torch, args.dispatch_sweep == "full")))
+        return
 
     # ---- headline: configs[1], 8192^3 e2m3 x e2m3 -> bf16
     M = N = K = 8192

@@ -302,9 +302,12 @@ bool gemm_skinny_supports(const GemmArgs& g) {
 // 64 x 57344 x 8192 105 -> 95, 64 x 128256 x 8192 212 -> 188 (24 - 32 rows level), and from 65 rows on from N = 24576:
 // 128 x 28672 x 8192 72 (mid-M kernel) -> 60; with K <= 4096 already from 33 rows and N = 24576 (a workgroup's K range is
 // then eight chunks or fewer, mostly load latency): 64 x 28672 x 4096 29 -> 23.  At N = 14336 and below this kernel wins.
+// Up to 16 rows only with tile-major B, K <= 4096 and N >= 65536: 16 x 128256 x 4096 82 -> 73, 16 x 65536 x 4096 45 -> 39
+// (level at K = 8192).
 bool gemm_wide_n_prefers_tiled(const GemmArgs& g) {
-  if (g.M <= 16 || g.M > 128 || !gemm_tiled_supports(g)) return false;
+  if (g.M > 128 || !gemm_tiled_supports(g)) return false;
   const long tiles = (g.N + 255) / 256;
+  if (g.M <= 16) return g.layout_b && tiles >= 256 && g.K <= 4096;
   if (g.layout_b) return tiles >= 160 || (tiles >= 96 && g.M >= 24);
   return g.M > 64 ? tiles >= 96 : g.M > 32 && (tiles >= 224 || (tiles >= 96 && g.K <= 4096));
 }

@@ -835,7 +835,9 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
 // tile-major and row-major B), in output tiles of 256 x 256: with K >= 14336 up to 64 tiles (128 from K = 24576 on):
 // 0.45 - 0.9 of the unsplit time, e.g. 256 x 8192 x 28672 108 -> 63 us, 128 x 4096 x 14336 46 -> 24 us, 1024 x 1024 x 16384
 // 60 -> 34 us; with 8192 <= K < 14336 up to 32 tiles where the skinny kernel is not an option (more than 128 rows of A, or
-// a tile-major A): 256 x 2048 x 8192 28.5 -> 21 us, 768 x 2048 x 8192 33 -> 27 us.  More tiles or a shorter K lose (the
+// a tile-major A): 256 x 2048 x 8192 28.5 -> 21 us, 768 x 2048 x 8192 33 -> 27 us; and up to 64 tiles for 65 - 128 rows of A
+// against more than 8192 rows of B, where the skinny kernel needs more than one round of workgroups:
+// 96 x 10240 x 8192 35 -> 27 us, 96 x 10240 x 12288 66 -> 37 us.  More tiles or a shorter K lose (the
 // partial sums cost 12 - 25 us to write, read and add): 256 x 8192 x 4096 19 -> 24 us, 512 x 8192 x 8192 36 -> 40 us.
 int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes) {
   if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps || g.K % (4 * kBK) != 0) return 1;
@@ -843,7 +845,10 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
   if (cus < 8) return 1;
   if (want == 0) {
     const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const bool pays = nkt >= 112 ? (tiles256 <= 64 || (nkt >= 192 && tiles256 <= 128)) : (nkt >= 64 && tiles256 <= 32 && (g.M > 128 || g.layout_a));
+    const bool pays = nkt >= 112 ? (tiles256 <= 64 || (nkt >= 192 && tiles256 <= 128))
+                                 : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
+                                                 // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
+                                                 (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192));
     if (!pays || (g.M <= 64 && !g.layout_a)) return 1;  // up to 64 rows of a row-major A are the skinny kernel's
   }
   int best = 1, best_rows = 0;
