@@ -63,22 +63,25 @@ def _as_tensor(obj, name: str):
 
 def _rows_cols(t, name: str):
     # leading dimensions are folded into rows, like the reference's left padding to 4-D
-    if t.dim() < 1:
+    sh = t.shape
+    if len(sh) == 2:
+        return sh[0], sh[1]
+    if len(sh) < 1:
         raise RuntimeError(f"{name}: expected at least 1 dimension")
-    cols = t.shape[-1]
     rows = 1
-    for d in t.shape[:-1]:
+    for d in sh[:-1]:
         rows *= d
-    return rows, cols
+    return rows, sh[-1]
 
 
-def _stream():
+def _stream(device=None):
+    """The current stream's raw handle on `device` (default: the current device)."""
     import torch
 
     try:  # the raw handle, without building a Stream object per call
-        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if device is None or device.index is None else device.index)
     except AttributeError:
-        return torch.cuda.current_stream().cuda_stream
+        return torch.cuda.current_stream(device).cuda_stream
 
 
 class _on_device:
@@ -175,24 +178,25 @@ def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2
         extras.append(t)
     if fp6_out:
         extras.append(C_scale)
-    devs = {t.device for t in (A, B, A_scale, B_scale, C, *extras)}
-    if len(devs) != 1:
-        raise RuntimeError(f"all tensors must be on one device, got {sorted(map(str, devs))}")
+    dev = C.device
+    for t in (A, B, A_scale, B_scale, *extras):
+        if t.device != dev:
+            raise RuntimeError(f"all tensors must be on one device, got {sorted({str(x.device) for x in (A, B, A_scale, B_scale, C, *extras)})}")
     L = _lib.lib()
     ptr = lambda t: 0 if t is None else t.data_ptr()
     if fp6_out:
-        with _on_device(C.device):
+        with _on_device(dev):
             rc = L.mxfp6_gemm_fused_fp6(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), C_scale.data_ptr(),
                                         M, N, K, fmt_a, fmt_b, layout_a, layout_b, fmt_c, ptr(bias),
                                         int(bias is not None and bias.dtype == torch.bfloat16), ptr(row_scale), ptr(col_scale),
-                                        _ACTS[activation], _stream())
+                                        _ACTS[activation], _stream(dev))
         _lib.check(rc, "dispatch_micro")
         return
-    with _on_device(C.device):
+    with _on_device(dev):
         rc = L.mxfp6_gemm_fused(A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
                                 fmt_a, fmt_b, layout_a, layout_b, int(C.dtype == torch.float32), ptr(bias),
                                 int(bias is not None and bias.dtype == torch.bfloat16), ptr(row_scale), ptr(col_scale),
-                                _ACTS[activation], _stream())
+                                _ACTS[activation], _stream(dev))
     _lib.check(rc, "dispatch_micro")
 
 
