@@ -452,11 +452,14 @@ int mxfp6_probe_ksplit(int shares) {
   return prev;
 }
 
-int mxfp6_probe_ksplit_plan(int M, int N, int K, int layout_a, int shares, int* tile_rows) {
+int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int* tile_rows) {
   if (M <= 0 || N <= 0 || K <= 0 || shares < -1 || shares > 64) return MXFP6_EINVAL_SHAPE;
+  if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;
+  const int layout_a = layouts & 1, layout_b = layouts >> 1;
+  if ((layout_a && M % 32) || (layout_b && N % 32)) return MXFP6_EINVAL_SHAPE;
   const int rc = check_device();
   if (rc) return rc;
-  mxfp6::GemmArgs g{nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, 2, 2, false, layout_a, 0};
+  mxfp6::GemmArgs g{nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, 2, 2, false, layout_a, layout_b};
   int rows = 0;
   size_t part = 0;
   const int n = N % 8 == 0 && K % 128 == 0 ? mxfp6::tiled_ksplit_plan(g, shares, &rows, &part) : 1;
@@ -560,7 +563,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 115; }
+int mxfp6_abi_version(void) { return 116; }
 
 #pragma GCC visibility pop
 }  // extern "C"

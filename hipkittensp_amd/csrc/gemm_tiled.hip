@@ -849,7 +849,13 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
                                  : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
                                                  // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
                                                  (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192));
-    if (!pays || (g.M <= 64 && !g.layout_a)) return 1;  // up to 64 rows of a row-major A are the skinny kernel's
+    if (!pays) return 1;
+    if (g.M <= 64 && !g.layout_a) {
+      // up to 64 rows of a row-major A are the skinny kernel's, except more than 32 against tile-major weights with a
+      // very long K, or a long K and a width that leaves the skinny kernel's last round of workgroups part empty
+      const bool ragged = g.N > 8192 && g.N % 8192 != 0;
+      if (!(g.M > 32 && g.layout_b && tiles256 <= 64 && (nkt >= 192 || ragged))) return 1;
+    }
   }
   int best = 1, best_rows = 0;
   double best_us = 0;

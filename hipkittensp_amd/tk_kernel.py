@@ -275,10 +275,10 @@ def set_k_split(shares: int) -> int:
     return _lib.lib().mxfp6_probe_ksplit(int(shares))
 
 
-def k_split_plan(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, shares: int = 0):
+def k_split_plan(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, shares: int = 0, layout_b: int = LAYOUT_ROW):
     """(workgroups per output tile, rows of A per tile) the tiled kernel's K split would use for this shape; (1, 0) = none."""
     rows = ctypes.c_int(0)
-    n = _lib.lib().mxfp6_probe_ksplit_plan(int(M), int(N), int(K), int(layout_a), int(shares), ctypes.byref(rows))
+    n = _lib.lib().mxfp6_probe_ksplit_plan(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1, int(shares), ctypes.byref(rows))
     if n < 0:
         _lib.check(n, "k_split_plan")
     return n, rows.value

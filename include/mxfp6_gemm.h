@@ -325,15 +325,19 @@ int mxfp6_probe_raster(int group_m, int xcd_remap);
  * being captured only if it exists already, else the launch runs unsplit) and a second small kernel adds them in share
  * order and applies the epilogue, so results do
  * not depend on timing.  0 = where it pays (default: K >= 14336 and at most 64 output tiles of 256 x 256, 128 from
- * K = 24576 on; 8192 <= K < 14336 only with at most 32 tiles and no skinny kernel for the shape), 1 = never,
+ * K = 24576 on; 8192 <= K < 14336 only with at most 32 tiles and no skinny kernel for the shape; up to 64 rows of a
+ * row-major A stay with the skinny kernel, except 33 - 64 rows against tile-major weights with K >= 24576 or N above 8192
+ * and no multiple of it), 1 = never,
  * -1 = wherever the shape allows it, n > 1 = n workgroups per output tile where the shape allows it (K a multiple of 512 n,
  * at least 8 K-tiles of 128 per share, at most half as many output tiles as CUs), else unsplit.
  * No counterpart in the reference (its GEMMs are one workgroup per 256 x 256 tile, analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61).
  */
 int mxfp6_probe_ksplit(int shares);
 /* The split the automatic path (shares = 0) or a forced setting would use for a shape on the current device: workgroups per
- * output tile (1 = none; negative = error code), and in *tile_rows (may be NULL) the rows of A per output tile (0 = none). */
-int mxfp6_probe_ksplit_plan(int M, int N, int K, int layout_a, int shares, int *tile_rows);
+ * output tile (1 = none; negative = error code), and in *tile_rows (may be NULL) the rows of A per output tile (0 = none).
+ * layouts: bit 0 set = A tile-major, bit 1 set = B tile-major (the e2m3 x e2m3 formats are assumed; the plan does not depend
+ * on them). */
+int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int *tile_rows);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

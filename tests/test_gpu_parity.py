@@ -194,6 +194,10 @@ def test_k_split_is_not_chosen_where_it_does_not_pay(hk):
     for M, N, K in [(256, 8192, 28672), (128, 4096, 14336), (1024, 1024, 16384), (768, 2048, 8192), (1024, 8192, 28672)]:
         assert tk.k_split_plan(M, N, K)[0] > 1, (M, N, K)
     assert tk.k_split_plan(96, 8192, 8192, 1)[0] > 1 and tk.k_split_plan(96, 8192, 8192, 0)[0] == 1  # the skinny kernel takes a row-major A
+    # up to 64 rows of a row-major A: the skinny kernel's, except 33 - 64 against tile-major weights with a very long K or a ragged width
+    for M, N, K, lb, split in [(64, 8192, 28672, 0, False), (64, 8192, 28672, 1, True), (32, 8192, 28672, 1, False), (48, 12288, 14336, 1, True),
+                               (48, 8192, 14336, 1, False), (64, 12288, 8192, 1, False)]:
+        assert (tk.k_split_plan(M, N, K, 0, 0, lb)[0] > 1) == split, (M, N, K, lb)
 
 
 def test_forced_kernels_reject_shapes_they_cannot_take(hk):
@@ -976,12 +980,12 @@ def test_cfg3_decode_skinny(hk):
 
 @pytest.mark.parametrize("M", [64, 128, 256])
 def test_batched_decode_full_size(hk, M):
-    """cfg3's weights against 64, 128 and 256 rows of A.  The automatic path takes the skinny kernel for 64 rows (two
-    accumulator tiles per wave) and the tiled kernel with K split between workgroups for 128 and 256; the skinny kernel's
-    128-row form (four accumulator tiles, half chunks) is forced as well.  Sampled rows and columns against the fp64
+    """cfg3's weights against 64, 128 and 256 rows of A.  The automatic path takes the skinny kernel for 64 rows against
+    row-major weights (two accumulator tiles per wave) and the tiled kernel with K split between workgroups otherwise; the
+    skinny kernel (for 128 rows: four accumulator tiles, half chunks) is forced as well.  Sampled rows and columns against the fp64
     oracle, the first 256 columns in full, and the whole result against the generic kernel; row-major and tile-major weights."""
     N, K = 8192, 28672
-    assert (hk.tk_kernel.k_split_plan(M, N, K)[0] > 1) == (M > 64)
+    assert (hk.tk_kernel.k_split_plan(M, N, K)[0] > 1) == (M > 64) and hk.tk_kernel.k_split_plan(M, N, K, 0, 0, 1)[0] > 1
     ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=30 + M, kind_a="normal", kind_b="weights")
     _sampled_check(hk, ap, asc, bp, bsc, 2, 2, 0, np.random.default_rng(M), ns=64)
     ref = o.gemm_ref(ap, bp[:256], asc, bsc[:256], acc=np.float64)
