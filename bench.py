@@ -266,7 +266,7 @@ def dispatch_sweep(hk, torch, full):
     else:
         shapes = [(8192, 8192), (28672, 8192), (8192, 28672), (57344, 8192), (1024, 16384)]
         rows_of_a = [16, 32, 64, 128, 256, 512, 1024]
-    forced = (("tiled", 2, 1), ("tiled_128x256", 5, 1), ("tiled_256x256", 6, 1), ("tiled_128x128", 17, 1), ("skinny", 3, 0), ("mid", 4, 0), ("tiled_k_split", 2, -1))
+    forced = (("tiled", 2, 1), ("tiled_128x256", 5, 1), ("tiled_256x256", 6, 1), ("tiled_128x128", 17, 1), ("block", 22, 1), ("skinny", 3, 0), ("mid", 4, 0), ("tiled_k_split", 2, -1))
 
     def time_us(sets, C, lay, kernel, k_split, reps=10):
         prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
@@ -373,7 +373,7 @@ def main():
                 _, ms = timed_loop(hk, torch, kin, C, args.steps, args.warmup, 1, 1)
                 hk.tk_kernel.set_kernel(prevk)
                 res[f"kernel={args.kernel}"] = {"launch_ms_mean": ms, "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12}
-        print(json.dumps({"what": f"gemm_tiled_kernel, {M} x {N} x {K} e2m3, operands and scales tile-major, per raster setting", "steps": args.steps, "warmup": args.warmup, "settings": res}))
+        print(json.dumps({"what": f"the kernel the library chooses ({hk.tk_kernel.kernel_choice(M, N, K, 1, 1)}: 2 = gemm_tiled_kernel, 22 = gemm_block_kernel, 25 = tiled with K split), {M} x {N} x {K} e2m3, operands and scales tile-major, per raster setting", "steps": args.steps, "warmup": args.warmup, "settings": res}))
         return
     # the operator as a caller gets it: for this size the library re-lays both operands out tile-major in a
     # pre-pass (one small kernel each) and runs the tiled kernel on them; `value` is the whole step
@@ -445,7 +445,7 @@ def main():
     dwall, dev_ms = timed_loop(hk, torch, dinputs, dC, args.steps, args.warmup)
     dbytes = algorithmic_bytes(dM, dN, dK)
     d_achieved = dbytes / (dev_ms * 1e-3) / 1e9
-    dtile = dbatched = dmid = None
+    dtile = dbatched = dmid = dprefill = None
     if args.layouts == "both":
         dtin = [(ap, hk.tile_operand(bp), asc, hk.tile_scales(bsc, dK)) for ap, bp, asc, bsc in dinputs]
         dtwall, dtev_ms = timed_loop(hk, torch, dtin, dC, args.steps, args.warmup, 0, 1)
@@ -475,6 +475,25 @@ def main():
             "launch_ms_mean_without_split": mev_ms_unsplit, "algorithmic_bytes_per_launch": mbytes,
         }
         del dtin, mins
+        # a few hundred rows of A at a K that is too short to split: gemm_block_kernel (128 x 128 tiles, four waves in
+        # step) against the 8-wave tiled kernel's 128 x 128 tiles, both operands tile-major
+        pM, pN, pK = 512, 8192, 8192
+        pa, pas = hk.quantize(torch.randn(pM, pK, device="cuda"), 2, layout=hk.tk_kernel.LAYOUT_TILE)
+        pbs = [hk.quantize(torch.randn(pN, pK, device="cuda") * 0.02, 2, layout=hk.tk_kernel.LAYOUT_TILE) for _ in range(3)]
+        pins = [(pa, b, pas, bs) for b, bs in pbs]
+        pC = torch.empty(pM, pN, dtype=torch.bfloat16, device="cuda")
+        _, pev_ms = timed_loop(hk, torch, pins, pC, args.steps, args.warmup, 1, 1)
+        prevk = hk.tk_kernel.set_kernel(hk.tk_kernel.KERNEL_TILED_128x128)
+        try:
+            _, pev_ms_tiled = timed_loop(hk, torch, pins, pC, args.steps, args.warmup, 1, 1)
+        finally:
+            hk.tk_kernel.set_kernel(prevk)
+        dprefill = {
+            "what": "M=512, N=K=8192, operands tile-major: the automatic choice (gemm_block_kernel) and the 8-wave tiled kernel with the same 128 x 128 tiles",
+            "kernel_choice": hk.tk_kernel.kernel_choice(pM, pN, pK, 1, 1), "launch_ms_mean": pev_ms, "tflops": 2.0 * pM * pN * pK / (pev_ms * 1e-3) / 1e12,
+            "launch_ms_mean_tiled_128x128": pev_ms_tiled,
+        }
+        del pins, pbs, pa, pas, pC
         dbatched = {
             "what": "M=64 (row-major A) against the same tile-major weights", "k_split_plan": list(hk.tk_kernel.k_split_plan(bM, dN, dK, 0, 0, 1)), "achieved": bbytes / (bev_ms * 1e-3) / 1e9, "unit": "GB/s",
             "frac": bbytes / (bev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "launch_ms_mean": bev_ms, "algorithmic_bytes_per_launch": bbytes,
@@ -536,6 +555,7 @@ def main():
         "tile_major_weights": dtile,
         "batched_m64": dbatched,
         "batched_m256": dmid,
+        "prefill_m512": dprefill,
     }
 
     line = {

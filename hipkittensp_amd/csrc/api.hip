@@ -90,6 +90,27 @@ bool launch_tiled_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
   return true;
 }
 
+// The kernel the automatic path takes for a call, by shape, layouts and alignment alone (codes of mxfp6_set_kernel; the
+// tiled kernel with its K split: kChoiceTiledKsplit).  allow_ksplit = false: what it takes when the split's workspace is
+// not to be had (a stream that is being captured, the allocator's refusal).
+constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceMid = 4, kChoiceBlock = 22, kChoiceTiledKsplit = 25;
+int auto_choice(const mxfp6::GemmArgs& g, int force_split, bool allow_ksplit) {
+  if (g.K == 0) return kChoiceGeneric;  // act(bias) everywhere: the generic kernel's K loop runs zero times
+  // 128 x 128 tiles that fill more than half the CUs (a quarter with K <= 8192), K of moderate length: ahead of the K split too
+  if (!force_split && mxfp6::gemm_block_preferred(g, true)) return kChoiceBlock;
+  // few output tiles, long K: the tiled kernel with K split between workgroups (before the skinny and mid-M kernels,
+  // which it beats there; the plan leaves up to 64 rows of a row-major A to the skinny kernel)
+  if (!force_split && allow_ksplit && !g.no_alloc && mxfp6::gemm_tiled_supports(g)) {
+    int rows = 0;
+    size_t part = 0;
+    if (mxfp6::tiled_ksplit_plan(g, g_ksplit, &rows, &part) > 1) return kChoiceTiledKsplit;
+  }
+  if (!force_split && mxfp6::gemm_block_preferred(g, false)) return kChoiceBlock;
+  if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) return kChoiceSkinny;
+  if (!mxfp6::gemm_wide_n_prefers_tiled(g) && (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g)))) return kChoiceMid;
+  return mxfp6::gemm_tiled_supports(g) ? kChoiceTiled : kChoiceGeneric;
+}
+
 hipError_t release_stream_workspaces() {
   std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);
   std::lock_guard<std::mutex> lock(g_sws_mutex);
@@ -211,37 +232,43 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   hipError_t e;
   if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
   if (no_alloc && (force_split || mxfp6::gemm_skinny_preferred(g)) && mxfp6::gemm_skinny_supports(g) && !mxfp6::gemm_skinny_scratch_fits(g)) return MXFP6_ESCRATCH;
-  if (K == 0) {
-    e = mxfp6::launch_gemm_generic(g, s);  // act(bias) everywhere: the generic kernel's K loop runs zero times
-  } else if (force == 1) {
+  if (K != 0 && force == 1) {
     e = mxfp6::launch_gemm_generic(g, s);
-  } else if (force == 2 || force == 5 || force == 6 || force == 17) {
+  } else if (K != 0 && (force == 2 || force == 5 || force == 6 || force == 17)) {
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
     std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
     plan_ksplit(g, s);
     e = mxfp6::launch_gemm_tiled(g, s);
-  } else if (force == 3 || (force >= 7 && force <= 16) || (force >= 19 && force <= 21)) {
+  } else if (K != 0 && (force == 3 || (force >= 7 && force <= 16) || (force >= 19 && force <= 21))) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.skinny_geometry = force == 3 ? 0 : force >= 19 ? force - 8 : force - 6;
     e = mxfp6::launch_gemm_skinny(g, s);
-  } else if (force == 4) {
+  } else if (K != 0 && force == 4) {
     if (!mxfp6::gemm_mid_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_mid(g, s);
-  } else if (force == 18) {
+  } else if (K != 0 && force == 18) {
     if (!mxfp6::gemm_tiled4_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_tiled4(g, s);
-  } else if (!force_split && launch_tiled_ksplit(g, s, e)) {
-    // few output tiles, long K: the tiled kernel with K split between workgroups (before the skinny and mid-M kernels,
-    // which it beats there; the plan leaves up to 64 rows of a row-major A to the skinny kernel)
-  } else if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) {
-    e = mxfp6::launch_gemm_skinny(g, s);
-  } else if (!mxfp6::gemm_wide_n_prefers_tiled(g) && (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g)))) {
-    e = mxfp6::launch_gemm_mid(g, s);
-  } else if (mxfp6::gemm_tiled_supports(g)) {
-    if (!relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
+  } else if (K != 0 && force >= 22 && force <= 24) {
+    if (!mxfp6::gemm_block_supports(g)) return MXFP6_EINVAL_SHAPE;
+    g.tile_rows = force == 22 ? 0 : force == 23 ? 3 : 6;
+    e = mxfp6::launch_gemm_block(g, s);
   } else {
-    e = mxfp6::launch_gemm_generic(g, s);
+    int choice = auto_choice(g, force_split, true);
+    // the split needs this stream's workspace: without it, what the shape gets otherwise
+    if (choice == kChoiceTiledKsplit && !launch_tiled_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
+    if (choice == kChoiceBlock) {
+      e = mxfp6::launch_gemm_block(g, s);
+    } else if (choice == kChoiceSkinny) {
+      e = mxfp6::launch_gemm_skinny(g, s);
+    } else if (choice == kChoiceMid) {
+      e = mxfp6::launch_gemm_mid(g, s);
+    } else if (choice == kChoiceTiled) {
+      if (!relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
+    } else if (choice == kChoiceGeneric) {
+      e = mxfp6::launch_gemm_generic(g, s);
+    }
   }
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
@@ -349,7 +376,7 @@ int mxfp6_set_relayout(int on) {
 }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 21) return MXFP6_EINVAL_KERNEL;
+  if (which < 0 || which > 24) return MXFP6_EINVAL_KERNEL;
   const int prev = g_force;
   g_force = which;
   return prev;
@@ -467,6 +494,19 @@ int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int* t
   return n;
 }
 
+int mxfp6_probe_choice(int M, int N, int K, int layouts) {
+  if (M <= 0 || N <= 0 || K < 0 || K % 32) return MXFP6_EINVAL_SHAPE;
+  if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;
+  const int layout_a = layouts & 1, layout_b = layouts >> 1;
+  if ((layout_a && (M % 32 || K % 128)) || (layout_b && (N % 32 || K % 128))) return MXFP6_EINVAL_SHAPE;
+  const int rc = check_device();
+  if (rc) return rc;
+  // aligned stand-ins for the pointers: the choice looks at their alignment only
+  const uint8_t* p = reinterpret_cast<const uint8_t*>((uintptr_t)4096);
+  mxfp6::GemmArgs g{p, p, p, p, const_cast<uint8_t*>(p), M, N, K, 2, 2, false, layout_a, layout_b};
+  return auto_choice(g, 0, true);
+}
+
 int mxfp6_probe_raster(int group_m, int xcd_remap) {
   if (group_m < 0 || group_m > 4096) return MXFP6_EINVAL_SHAPE;
   g_raster_group_m = group_m, g_raster_no_xcd = xcd_remap ? 0 : 1;
@@ -563,7 +603,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 116; }
+int mxfp6_abi_version(void) { return 117; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -41,6 +41,9 @@ hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
 int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes);
 bool gemm_tiled4_supports(const GemmArgs& g);  // the 4-wave variant of the tiled kernel (selectable, never chosen automatically)
 hipError_t launch_gemm_tiled4(const GemmArgs& g, hipStream_t s);
+bool gemm_block_supports(const GemmArgs& g);  // 128 x 128 tiles, four waves in step (a few hundred to a few thousand rows of A)
+bool gemm_block_preferred(const GemmArgs& g, bool first);  // by shape; first: even before the tiled kernel's K split is considered
+hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
 bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
 double tiled_estimate_us(const GemmArgs& g, int rows, int cols = 256);  // estimated time of the tiled kernel with tiles of rows x cols

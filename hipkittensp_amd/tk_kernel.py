@@ -45,6 +45,8 @@ KERNEL_SKINNY_2WAVES = 16  # 32 rows of B, two waves per workgroup (wide N, shor
 KERNEL_TILED_128x128 = 17  # tiled kernel with output tiles of 128 x 128
 KERNEL_SKINNY_64 = 19  # skinny kernel with 64 rows of B per workgroup (two tiles of B against every fragment of A), K unsplit
 KERNEL_SKINNY_64_SPLIT = (20, 21)  # the same with the K range split between 2 / 4 workgroups
+KERNEL_BLOCK = 22  # 128 x 128 tiles, four waves in step: one barrier per K-tile, fragments double-buffered in registers
+KERNEL_BLOCK_3SLOTS, KERNEL_BLOCK_6SLOTS = 23, 24  # the same with its operand ring forced to three / six slots
 KERNEL_TILED_4WAVE = 18  # the 4-wave interleaved schedule of the tiled kernel (measurement: never chosen automatically)
 
 
@@ -282,6 +284,17 @@ def k_split_plan(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, shares: int
     if n < 0:
         _lib.check(n, "k_split_plan")
     return n, rows.value
+
+
+CHOICE_TILED_K_SPLIT = 25  # kernel_choice(): the tiled kernel with its K split between workgroups
+
+
+def kernel_choice(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, layout_b: int = LAYOUT_ROW) -> int:
+    """The kernel (KERNEL_* code, or CHOICE_TILED_K_SPLIT) the automatic path takes for this shape; launches nothing."""
+    n = _lib.lib().mxfp6_probe_choice(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1)
+    if n < 0:
+        _lib.check(n, "kernel_choice")
+    return n
 
 
 def set_kernel(which: int) -> int:

@@ -117,6 +117,10 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *    4  mid-M kernel (needs 32 < M <= 512, K % 1024 == 0, row-major A)
  *   18  the 4-wave interleaved schedule of the LDS-tiled kernel (one wave per SIMD with a 128 x 128 wave tile; shapes
  *       of kernel 2, no fused epilogue); never chosen automatically, kept to compare the two schedules
+ *   22  block kernel: output tiles of 128 x 128, four waves in step with the operand fragments double-buffered in
+ *       registers, one barrier per K-tile (needs N % 8 == 0, K % 512 == 0, no fused epilogue); chosen automatically where
+ *       its tiles do not outnumber the CUs and K is of moderate length (a few hundred rows of A);
+ *       23 / 24: with an operand ring of three slots (two workgroups per CU) / six slots (one)
  * No counterpart in the reference, whose shapes are compile-time constants per binary
  * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
  */
@@ -338,6 +342,12 @@ int mxfp6_probe_ksplit(int shares);
  * layouts: bit 0 set = A tile-major, bit 1 set = B tile-major (the e2m3 x e2m3 formats are assumed; the plan does not depend
  * on them). */
 int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int *tile_rows);
+
+/* The kernel the automatic path takes for a problem of this shape on the current device (e2m3 x e2m3, bf16 output, no fused
+ * epilogue, 16-byte aligned tensors): a code of mxfp6_set_kernel (1 generic, 2 tiled, 3 skinny, 4 mid-M, 22 block), or 25
+ * for the tiled kernel with its K split between workgroups; negative = error code.  layouts as in
+ * mxfp6_probe_ksplit_plan.  Reads the thread's mxfp6_probe_ksplit setting; launches nothing. */
+int mxfp6_probe_choice(int M, int N, int K, int layouts);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);

@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 116
+    assert L.mxfp6_abi_version() == 117
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -116,6 +116,10 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     assert L.mxfp6_probe_ksplit(65) == -2 and L.mxfp6_probe_ksplit(-2) == -2
     prev = L.mxfp6_probe_ksplit(1)
     assert prev == 0 and L.mxfp6_probe_ksplit(0) == 1
+    L.mxfp6_probe_choice.restype = ci
+    L.mxfp6_probe_choice.argtypes = [ci, ci, ci, ci]
+    assert L.mxfp6_probe_choice(0, 16, 512, 0) == -2 and L.mxfp6_probe_choice(16, 16, 48, 0) == -2    # shape
+    assert L.mxfp6_probe_choice(16, 16, 512, 4) == -6 and L.mxfp6_probe_choice(40, 64, 512, 1) == -2  # layouts; tile-major needs rows % 32
     assert L.mxfp6_set_kernel(2) == 0
     import threading
     seen = []

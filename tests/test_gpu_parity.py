@@ -141,6 +141,77 @@ def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
+# ------------------------------------------------------------------ block kernel (128 x 128 tiles, four waves in step)
+@pytest.mark.parametrize("M,N,K", [(128, 128, 512), (256, 384, 1024), (512, 256, 2560), (300, 264, 1536), (129, 8, 512), (100, 1000, 1024), (33, 520, 2048),
+                                   (1, 128, 512), (640, 1024, 4096)])  # edge tiles too; K in whole groups of four K-tiles
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
+@pytest.mark.parametrize("kernel", [23, 24])  # ring of three slots (two workgroups per CU) and of six (one)
+def test_block_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M * 5 + N + K, kind_a="laplace" if fa == 3 else "normal", kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel)
+    check(got, ref, fa, fb, ap, asc, bp, bsc)
+    cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=kernel)
+    assert np.array_equal(cb, o.f32_to_bf16_bits(got))
+    assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=22), got)   # ring depth chosen by the library: same bits
+
+
+@pytest.mark.parametrize("M,N,K,la,lb", [(256, 8192, 2048, 1, 1), (192, 4096, 4096, 0, 1), (512, 3072, 3072, 0, 0), (1024, 2048, 8192, 1, 1), (96, 16384, 1024, 0, 1),
+                                         (384, 6144, 4096, 1, 0)])
+def test_block_kernel_is_chosen_and_matches_the_tiled_kernel(hk, M, N, K, la, lb):
+    """Shapes on which the automatic path takes the block kernel (its tiles do not outnumber the CUs, K of moderate length):
+    the result is the forced block kernel's bit for bit (the two agree on the dispatch), equals the 8-wave tiled kernel's
+    (same order of summation along K) and passes against the fp64 oracle on sampled rows."""
+    prev_split = hk.tk_kernel.set_k_split(1)
+    try:
+        assert hk.tk_kernel.kernel_choice(M, N, K, la, lb) == hk.tk_kernel.KERNEL_BLOCK
+    finally:
+        hk.tk_kernel.set_k_split(prev_split)
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=M + N + K, kind_b="weights")
+    A, As = (hk.tile_operand(dev(ap)), hk.tile_scales(dev(asc), K)) if la else (dev(ap), dev(asc))
+    B, Bs = (hk.tile_operand(dev(bp)), hk.tile_scales(dev(bsc), K)) if lb else (dev(bp), dev(bsc))
+    outs = {}
+    for kernel in (0, 22, 2):
+        C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        prev, prev_split = hk.tk_kernel.set_kernel(kernel), hk.tk_kernel.set_k_split(1)
+        try:
+            hk.dispatch_micro(A, B, As, Bs, C, layout_a=la, layout_b=lb)
+            torch.cuda.synchronize()
+        finally:
+            hk.tk_kernel.set_kernel(prev)
+            hk.tk_kernel.set_k_split(prev_split)
+        outs[kernel] = C.cpu().numpy()
+    assert np.array_equal(outs[0], outs[22]) and np.array_equal(outs[22], outs[2])
+    rows = np.random.default_rng(M).choice(M, 16, replace=False)
+    check(outs[22][rows], o.gemm_ref(ap[rows], bp, asc[rows], bsc, acc=np.float64), 2, 2)
+
+
+def test_kernel_choice_by_shape(hk):
+    """The automatic choice over the library's kernels, as mxfp6_probe_choice reports it (A row-major unless stated)."""
+    tk = hk.tk_kernel
+    assert tk.kernel_choice(8192, 8192, 8192) == tk.KERNEL_TILED
+    assert tk.kernel_choice(16, 8192, 28672) == tk.KERNEL_SKINNY and tk.kernel_choice(64, 8192, 8192, 0, 1) == tk.KERNEL_SKINNY
+    assert tk.kernel_choice(256, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT
+    assert tk.kernel_choice(256, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(512, 4096, 4096, 0, 1) == tk.KERNEL_BLOCK
+    assert tk.kernel_choice(2048, 8192, 8192, 1, 1) == tk.KERNEL_TILED      # more 128 x 128 tiles than CUs
+    assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_TILED  # K % 512
+    assert tk.kernel_choice(40, 36, 96) == tk.KERNEL_GENERIC
+    prev = tk.set_k_split(1)
+    try:
+        assert tk.kernel_choice(256, 8192, 28672, 1, 1) != tk.CHOICE_TILED_K_SPLIT
+    finally:
+        tk.set_k_split(prev)
+
+
+def test_block_kernel_rejects_what_it_cannot_take(hk):
+    ap, asc, bp, bsc = operands(128, 128, 384, 2, 2, seed=1)      # K % 512
+    with pytest.raises(RuntimeError, match="bad shape"):
+        gemm(hk, ap, bp, asc, bsc, kernel=22)
+    ap, asc, bp, bsc = operands(128, 36, 512, 2, 2, seed=1)       # N % 8
+    with pytest.raises(RuntimeError, match="bad shape"):
+        gemm(hk, ap, bp, asc, bsc, kernel=23)
+
+
 @pytest.mark.parametrize("M,N,K,shares", [(256, 512, 4096, 2), (256, 512, 4096, 4), (300, 264, 8192, 4), (128, 768, 8192, 8), (100, 520, 2048, 2),
                                           (512, 256, 16384, 0), (96, 1024, 14336, 0), (160, 2048, 8192, 0)])
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
@@ -414,7 +485,7 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
     assert np.array_equal(hk.tile_scales(ts, K, untile=True).cpu().numpy(), sr)
 
 
-@pytest.mark.parametrize("kernel,M,N,K", [(1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
+@pytest.mark.parametrize("kernel,M,N,K", [(23, 256, 512, 1024), (24, 320, 544, 1536), (1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
                                           (18, 256, 512, 640), (18, 320, 544, 1152), (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
