@@ -449,7 +449,7 @@ def main():
     if args.layouts == "both":
         dtin = [(ap, hk.tile_operand(bp), asc, hk.tile_scales(bsc, dK)) for ap, bp, asc, bsc in dinputs]
         dtwall, dtev_ms = timed_loop(hk, torch, dtin, dC, args.steps, args.warmup, 0, 1)
-        # batched decode: 64 rows of a row-major A against the same tile-major weights (K this long: the tiled kernel with K split)
+        # batched decode: 64 rows of a row-major A against the same tile-major weights (K this long: a K split between workgroups)
         bM = 64
         ba, bas = hk.quantize(torch.randn(bM, dK, device="cuda"), 2)
         bC = torch.empty(bM, dN, dtype=torch.bfloat16, device="cuda")
@@ -469,8 +469,8 @@ def main():
             hk.tk_kernel.set_k_split(prev_split)
         mbytes, mflops = algorithmic_bytes(mM, dN, dK), 2.0 * mM * dN * dK
         dmid = {
-            "what": "M=256 against the same tile-major weights (A tile-major too): gemm_tiled_kernel with K split between workgroups + ksplit_reduce_kernel",
-            "k_split_plan": list(hk.tk_kernel.k_split_plan(mM, dN, dK, 1)), "launch_ms_mean": mev_ms, "achieved": mbytes / (mev_ms * 1e-3) / 1e9,
+            "what": "M=256 against the same tile-major weights (A tile-major too): K split between workgroups (kernel_choice 25: gemm_tiled_kernel, 27: gemm_block_kernel) + ksplit_reduce_kernel",
+            "kernel_choice": hk.tk_kernel.kernel_choice(mM, dN, dK, 1, 1), "launch_ms_mean": mev_ms, "achieved": mbytes / (mev_ms * 1e-3) / 1e9,
             "unit": "GB/s", "frac": mbytes / (mev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "tflops": mflops / (mev_ms * 1e-3) / 1e12,
             "launch_ms_mean_without_split": mev_ms_unsplit, "algorithmic_bytes_per_launch": mbytes,
         }
@@ -495,7 +495,7 @@ def main():
         }
         del pins, pbs, pa, pas, pC
         dbatched = {
-            "what": "M=64 (row-major A) against the same tile-major weights", "k_split_plan": list(hk.tk_kernel.k_split_plan(bM, dN, dK, 0, 0, 1)), "achieved": bbytes / (bev_ms * 1e-3) / 1e9, "unit": "GB/s",
+            "what": "M=64 (row-major A) against the same tile-major weights (kernel_choice 3: gemm_skinny_kernel, 25 / 27: gemm_tiled_kernel / gemm_block_kernel with K split between workgroups)", "kernel_choice": hk.tk_kernel.kernel_choice(bM, dN, dK, 0, 1), "achieved": bbytes / (bev_ms * 1e-3) / 1e9, "unit": "GB/s",
             "frac": bbytes / (bev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "launch_ms_mean": bev_ms, "algorithmic_bytes_per_launch": bbytes,
         }
         dtile = {

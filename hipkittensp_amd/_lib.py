@@ -81,6 +81,8 @@ def lib() -> ctypes.CDLL:
         L.mxfp6_probe_ksplit.argtypes = [ci]
         L.mxfp6_probe_ksplit_plan.restype = ci
         L.mxfp6_probe_ksplit_plan.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
+        L.mxfp6_probe_block.restype = ci
+        L.mxfp6_probe_block.argtypes = [ci]
         L.mxfp6_probe_choice.restype = ci
         L.mxfp6_probe_choice.argtypes = [ci, ci, ci, ci]
         L.mxfp6_release_workspaces.restype = ci

@@ -22,6 +22,7 @@ thread_local int g_relayout = 1;
 thread_local uint32_t* g_clock_stamps = nullptr;  // mxfp6_probe_tiled_clock
 thread_local int g_raster_group_m = 0, g_raster_no_xcd = 0;  // mxfp6_probe_raster
 thread_local int g_ablation = 0;                              // mxfp6_probe_tiled_ablation
+thread_local int g_block = 1;                                 // mxfp6_probe_block: 0 keeps the block kernel out of the automatic choice
 thread_local int g_ksplit = 0;                                // mxfp6_probe_ksplit: 0 = where it pays, -1 = wherever possible, 1 = never, n = n shares per output tile
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
@@ -80,6 +81,23 @@ void plan_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
   g.ks_part = reinterpret_cast<float*>(pp);
 }
 
+// The block kernel's K split for this call, likewise.
+void plan_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
+  size_t part = 0;
+  const int shares = mxfp6::block_ksplit_plan(g, g_ksplit, &part);
+  if (shares <= 1) return;
+  uint8_t* pp = stream_workspace(s, 2, part);
+  if (!pp) return;
+  g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp);
+}
+bool launch_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
+  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
+  plan_block_ksplit(g, s);
+  if (g.ksplit <= 1) return false;
+  e = mxfp6::launch_gemm_block(g, s);
+  return true;
+}
+
 // Automatic path: launches the tiled kernel with its K split if the shape calls for one (and the workspace is there).
 bool launch_tiled_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
   if (g.no_alloc || g.K == 0 || !mxfp6::gemm_tiled_supports(g)) return false;
@@ -93,11 +111,17 @@ bool launch_tiled_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
 // The kernel the automatic path takes for a call, by shape, layouts and alignment alone (codes of mxfp6_set_kernel; the
 // tiled kernel with its K split: kChoiceTiledKsplit).  allow_ksplit = false: what it takes when the split's workspace is
 // not to be had (a stream that is being captured, the allocator's refusal).
-constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceMid = 4, kChoiceBlock = 22, kChoiceTiledKsplit = 25;
+constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceMid = 4, kChoiceBlock = 22, kChoiceTiledKsplit = 25, kChoiceBlockWide = 26, kChoiceBlockKsplit = 27;
 int auto_choice(const mxfp6::GemmArgs& g, int force_split, bool allow_ksplit) {
   if (g.K == 0) return kChoiceGeneric;  // act(bias) everywhere: the generic kernel's K loop runs zero times
+  const bool block = g_block && !force_split;  // the block kernel may be chosen
+  // 128 x 128 tiles on at most half the CUs: the block kernel with its K split between workgroups
+  if (block && allow_ksplit) {
+    size_t part = 0;
+    if (mxfp6::block_ksplit_plan(g, g_ksplit, &part) > 1) return kChoiceBlockKsplit;
+  }
   // 128 x 128 tiles that fill more than half the CUs (a quarter with K <= 8192), K of moderate length: ahead of the K split too
-  if (!force_split && mxfp6::gemm_block_preferred(g, true)) return kChoiceBlock;
+  if (block && mxfp6::gemm_block_preferred(g, true)) return kChoiceBlock;
   // few output tiles, long K: the tiled kernel with K split between workgroups (before the skinny and mid-M kernels,
   // which it beats there; the plan leaves up to 64 rows of a row-major A to the skinny kernel)
   if (!force_split && allow_ksplit && !g.no_alloc && mxfp6::gemm_tiled_supports(g)) {
@@ -105,7 +129,8 @@ int auto_choice(const mxfp6::GemmArgs& g, int force_split, bool allow_ksplit) {
     size_t part = 0;
     if (mxfp6::tiled_ksplit_plan(g, g_ksplit, &rows, &part) > 1) return kChoiceTiledKsplit;
   }
-  if (!force_split && mxfp6::gemm_block_preferred(g, false)) return kChoiceBlock;
+  if (block && mxfp6::gemm_block_preferred(g, false)) return kChoiceBlock;
+  if (block && mxfp6::gemm_block_wide_preferred(g)) return kChoiceBlockWide;
   if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) return kChoiceSkinny;
   if (!mxfp6::gemm_wide_n_prefers_tiled(g) && (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g)))) return kChoiceMid;
   return mxfp6::gemm_tiled_supports(g) ? kChoiceTiled : kChoiceGeneric;
@@ -250,15 +275,21 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (K != 0 && force == 18) {
     if (!mxfp6::gemm_tiled4_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_tiled4(g, s);
-  } else if (K != 0 && force >= 22 && force <= 24) {
+  } else if (K != 0 && ((force >= 22 && force <= 24) || force == 26)) {
     if (!mxfp6::gemm_block_supports(g)) return MXFP6_EINVAL_SHAPE;
-    g.tile_rows = force == 22 ? 0 : force == 23 ? 3 : 6;
+    g.tile_rows = force == 23 ? 3 : force == 24 ? 6 : 0, g.tile_cols = force == 26 ? 256 : 0;
+    std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
+    if (force != 26) plan_block_ksplit(g, s);
     e = mxfp6::launch_gemm_block(g, s);
   } else {
     int choice = auto_choice(g, force_split, true);
     // the split needs this stream's workspace: without it, what the shape gets otherwise
+    if (choice == kChoiceBlockKsplit && !launch_block_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
     if (choice == kChoiceTiledKsplit && !launch_tiled_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
     if (choice == kChoiceBlock) {
+      e = mxfp6::launch_gemm_block(g, s);
+    } else if (choice == kChoiceBlockWide) {
+      g.tile_cols = 256;
       e = mxfp6::launch_gemm_block(g, s);
     } else if (choice == kChoiceSkinny) {
       e = mxfp6::launch_gemm_skinny(g, s);
@@ -376,7 +407,7 @@ int mxfp6_set_relayout(int on) {
 }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 24) return MXFP6_EINVAL_KERNEL;
+  if (which < 0 || which > 26 || which == 25) return MXFP6_EINVAL_KERNEL;
   const int prev = g_force;
   g_force = which;
   return prev;
@@ -494,6 +525,12 @@ int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int* t
   return n;
 }
 
+int mxfp6_probe_block(int enable) {
+  const int prev = g_block;
+  g_block = enable ? 1 : 0;
+  return prev;
+}
+
 int mxfp6_probe_choice(int M, int N, int K, int layouts) {
   if (M <= 0 || N <= 0 || K < 0 || K % 32) return MXFP6_EINVAL_SHAPE;
   if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;
@@ -603,7 +640,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 117; }
+int mxfp6_abi_version(void) { return 119; }
 
 #pragma GCC visibility pop
 }  // extern "C"

@@ -23,10 +23,10 @@
 namespace mxfp6 {
 namespace {
 
-constexpr int kBM = 128, kBN = 128, kBK = 128, NW = 4;
-constexpr int kATile = kBM * 96, kSlot = kATile + kBN * 96;  // bytes of A's tile and of a ring slot
-constexpr int kScOp = 128 * 16, kScBuf = 2 * kScOp;  // scales of one operand / of both for four K-tiles
-constexpr int kGroupM = 8;  // tile rows per raster group
+constexpr int kBM = 128, kBK = 128;
+constexpr int kATile = kBM * 96;  // bytes of A's tile in a ring slot
+constexpr int kScA = kBM * 16;    // bytes of A's scales for four K-tiles
+constexpr int kGroupM = 8;        // tile rows per raster group
 
 // one direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff, the hardware writes them at LDS
 // address lds_base + 16 * lane; the VMEM counter is managed by hand (wait_vmcnt)
@@ -51,48 +51,64 @@ struct BlockArgs {
   const uint8_t *A, *B, *As, *Bs;
   void* C;
   int M, N, K, tiles_m, tiles_n, layout_a, layout_b, group_m, xcd_remap;
+  int nsplit;  // workgroups that share an output tile, each over K / nsplit (a whole number of groups of four K-tiles); 1 = no split
 };
 
 // STAGES: ring slots, 3 (80 KB of LDS, two workgroups per CU) to 6 (152 KB, one).  Loads run STAGES K-tiles ahead of the
 // MFMAs and have STAGES - 1 steps to land; from five slots on the scales are fetched two groups ahead instead of one, so
 // that they are older than every load a step's wait leaves in flight.
-template <int FA, int FB, typename Out, int STAGES>
-__global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kernel(const BlockArgs args) {
+// WN: waves side by side along N, 2 (tile of 128 x 128, four waves) or 4 (128 x 256, eight waves: waves 0-3 load A's tile
+// and half of B's, six loads per K-tile, waves 4-7 the other half of B's, three loads).
+template <int FA, int FB, typename Out, int STAGES, int WN>
+__global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_block_kernel(const BlockArgs args) {
   typedef typename Out::type OutT;
-  static_assert(STAGES >= 3 && STAGES <= 6, "ring depth");
+  static_assert(STAGES >= 3 && STAGES <= 6 && (WN == 2 || WN == 4), "ring depth, tile width");
+  constexpr int NW = 2 * WN, kBN = WN * 64, kSlot = kATile + kBN * 96, kScBuf = kScA + kBN * 16;
   constexpr int kStages = STAGES, E = STAGES > 4 ? 1 : 0;  // E: extra groups of four K-tiles the scale loads run ahead
   constexpr int kScBase = kStages * kSlot, kLdsBytes = kScBase + 2 * kScBuf;
-  static_assert(kLdsBytes <= (STAGES <= 3 ? 81920 : 163840), "LDS budget");
+  static_assert(kLdsBytes <= (STAGES <= 3 && WN == 2 ? 81920 : 163840), "LDS budget");
   __shared__ __attribute__((aligned(1024))) uint8_t smem[kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
   const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
-  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt = K / kBK, nk4 = nkt / 4;
+  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt_all = K / kBK, nk4_all = nkt_all / 4;
+  // K split: workgroup b takes share b / tiles of tile b % tiles, K-tiles [share, share + 1) * nkt, and leaves its fp32
+  // sums in matrix `share` of args.C, then a workspace of nsplit matrices [M, N] (ksplit_reduce_kernel adds them up)
+  const int ntiles = args.tiles_m * args.tiles_n, share = blockIdx.x / ntiles;
+  const int nkt = nkt_all / args.nsplit, nk4 = nkt / 4, kt0 = share * nkt;
 
-  const int tile = tile_order(blockIdx.x, args.tiles_m, args.tiles_n, args.group_m, args.xcd_remap);
-  if (tile < 0) return;  // never: the grid is the tile count
+  const int tile = tile_order(blockIdx.x - share * ntiles, args.tiles_m, args.tiles_n, args.group_m, args.xcd_remap);
+  if (tile < 0) return;  // never: the grid is the tile count times the shares
   const int pm = tile & 0xffff, pn = tile >> 16;
   const int rows_a = min(kBM, args.M - pm * kBM), rows_b = min(kBN, args.N - pn * kBN);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
+  const bool loads_a = wave < 4;  // this wave loads row-tile `wave` of A's tile (every wave loads row-tile `wave` of B's)
   const int h = lane >> 5, r32 = lane & 31;
 
   // operand rows of this tile; rZ: a resource of length zero, loads through it fetch nothing (K-tiles past the end)
-  const __amdgpu_buffer_rsrc_t rA = make_rsrc(args.A + (size_t)pm * kBM * rowbytes, (uint32_t)rows_a * rowbytes);
-  const __amdgpu_buffer_rsrc_t rB = make_rsrc(args.B + (size_t)pn * kBN * rowbytes, (uint32_t)rows_b * rowbytes);
+  // (a share's resources start at its first K-tile, 96 or 3072 bytes times kt0 into a row or row-tile, and end that much
+  // earlier, so that rows past the tile's last still lie beyond the end)
+  const uint32_t oa = (uint32_t)kt0 * (layout_a ? 3072 : 96), ob = (uint32_t)kt0 * (layout_b ? 3072 : 96);
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(args.A + (size_t)pm * kBM * rowbytes + oa, (uint32_t)rows_a * rowbytes - oa);
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(args.B + (size_t)pn * kBN * rowbytes + ob, (uint32_t)rows_b * rowbytes - ob);
   const __amdgpu_buffer_rsrc_t rZ = make_rsrc(args.A, 0);
-  // scales: waves 0, 1 fetch A's (rows 0-63, 64-127 of the tile), waves 2, 3 B's; a lane fetches the 16 bytes one row
-  // has for four K-tiles
-  const bool sc_a = wave < 2;
+  // scales: the first half of the waves fetch A's (rows 0-63, 64-127 of the tile; with eight waves, waves 2, 3 fetch what
+  // waves 0, 1 fetch, into the same place, so that every wave issues one scale load per group), the second half B's, 64
+  // rows each; a lane fetches the 16 bytes one row has for four K-tiles
+  const bool sc_a = wave < NW / 2;
   const int slay = sc_a ? layout_a : layout_b, srows = sc_a ? rows_a : rows_b, stile = sc_a ? pm : pn;
   const uint8_t* sp = sc_a ? args.As : args.Bs;
-  const __amdgpu_buffer_rsrc_t rS = slay ? make_rsrc(sp + (size_t)stile * 4 * nk4 * 512, (uint32_t)((srows + 31) / 32) * nk4 * 512)
-                                         : make_rsrc(sp + (size_t)stile * 128 * sbytes, (uint32_t)srows * sbytes);
-  const int srow = (wave & 1) * 64 + lane;
-  const int voff_s = slay ? (srow >> 5) * nk4 * 512 + (srow & 31) * 16 : srow * sbytes;
+  const int sheight = sc_a ? kBM : kBN;  // rows per tile of the operand whose scales these are
+  const uint32_t os = (uint32_t)(kt0 >> 2) * (slay ? 512 : 16);  // the share's first group of four K-tiles
+  const __amdgpu_buffer_rsrc_t rS = slay ? make_rsrc(sp + (size_t)stile * (sheight / 32) * nk4_all * 512 + os, (uint32_t)((srows + 31) / 32) * nk4_all * 512 - os)
+                                         : make_rsrc(sp + (size_t)stile * sheight * sbytes + os, (uint32_t)srows * sbytes - os);
+  const int spart = sc_a ? wave & 1 : wave - NW / 2;  // which 64 rows
+  const int srow = spart * 64 + lane;
+  const int voff_s = slay ? (srow >> 5) * nk4_all * 512 + (srow & 31) * 16 : srow * sbytes;
   const int sstep = slay ? 512 : 16;
-  const uint32_t sdst = lds0 + kScBase + (sc_a ? 0 : kScOp) + (wave & 1) * 1024;
+  const uint32_t sdst = lds0 + kScBase + (sc_a ? 0 : kScA) + spart * 1024;
 
   // per-lane global byte offsets of the direct loads: load q = 3 wave + i fills LDS bytes [q * 1024, + 1024) of an
   // operand's tile.  Row-major: 16-byte slot o holds piece (o % 6) ^ ((row >> 3) & 1) of row o / 6.  Tile-major: the
@@ -102,7 +118,7 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
   for (int i = 0; i < 3; i++) {
     const int q = wave * 3 + i, o = q * 64 + lane;
     const int r = o / 6, c = (o - r * 6) ^ ((r >> 3) & 1);
-    const int vrow = r * rowbytes + c * 16, vtile = wave * (nkt * 3072) + i * 1024 + lane * 16;
+    const int vrow = r * rowbytes + c * 16, vtile = wave * (nkt_all * 3072) + i * 1024 + lane * 16;
     voff_a[i] = layout_a ? vtile : vrow;
     voff_b[i] = layout_b ? vtile : vrow;
   }
@@ -116,7 +132,7 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
     a_rd[c] = (wm * 64 + r32) * 96 + ((3 * h + c) ^ sw) * 16;
     b_rd[c] = kATile + (wn * 64 + r32) * 96 + ((3 * h + c) ^ sw) * 16;
   }
-  const int sa_rd = kScBase + (wm * 64 + r32) * 16, sb_rd = kScBase + kScOp + (wn * 64 + r32) * 16;
+  const int sa_rd = kScBase + (wm * 64 + r32) * 16, sb_rd = kScBase + kScA + (wn * 64 + r32) * 16;
   const int sc_shift = 16 * h;  // a lane's two scale bytes of a K-tile: bytes 2h, 2h + 1 of the K-tile's four
 
   v16f acc[2][2];
@@ -130,16 +146,19 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
   int sca[2][4], scb[2][4];  // [tile][K-tile of the group]: scale bytes in bytes 0, 1
   v4i raw_a[2], raw_b[2];
 
-  // load n (0-2: A's, 3-5: B's) of this wave's six for K-tile t
-  auto load_one = [&](int t, int slot, int n) __attribute__((always_inline)) {
+  // load n of this wave's for K-tile t: 0-2 the three of row-tile `wave` of A's tile (LA: this wave loads A at all), 3-5 of B's
+  auto load_one = [&]<bool LA>(int t, int slot, int n) __attribute__((always_inline)) {
     const bool in = t < nkt;
     const uint32_t dst = lds0 + slot * kSlot + wave * 3072;
-    if (n < 3) dma16(in ? rA : rZ, dst + n * 1024, voff_a[n], t * kstep_a);
-    else dma16(in ? rB : rZ, dst + kATile + (n - 3) * 1024, voff_b[n - 3], t * kstep_b);
+    if (n < 3) {
+      if constexpr (LA) dma16(in ? rA : rZ, dst + n * 1024, voff_a[n], t * kstep_a);
+    } else {
+      dma16(in ? rB : rZ, dst + kATile + (n - 3) * 1024, voff_b[n - 3], t * kstep_b);
+    }
   };
-  auto load_tile = [&](int t, int slot) __attribute__((always_inline)) {
+  auto load_tile = [&]<bool LA>(int t, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int n = 0; n < 6; n++) load_one(t, slot, n);
+    for (int n = 0; n < 6; n++) load_one.template operator()<LA>(t, slot, n);
   };
   auto load_scales = [&](int grp) __attribute__((always_inline)) {
     const __amdgpu_buffer_rsrc_t rs = grp < nk4 ? rS : rZ;
@@ -207,7 +226,9 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
   int slot[kStages];
 #pragma unroll
   for (int i = 0; i < kStages; i++) slot[i] = i;
-  auto step = [&]<int KM>(int k) __attribute__((always_inline)) {
+  // LA: this wave loads A's tile too (six loads per K-tile, else three); instantiated per wave class, so that no branch
+  // sits between the MFMAs (a branch there makes the compiler keep a second copy of the accumulators)
+  auto step = [&]<int KM, bool LA>(int k) __attribute__((always_inline)) {
     constexpr int CUR = KM & 1, NXT = CUR ^ 1;
     // LDS reads of K-tile k + 1 first, then the MFMAs of K-tile k with the direct loads of K-tile k + STAGES (into K-tile
     // k's slot) between them, one after each of the first six, and after the seventh the scales of a later group of four
@@ -218,7 +239,7 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
     __builtin_amdgcn_s_setprio(1);
     mma_tile.template operator()<CUR, KM>([&](int q) __attribute__((always_inline)) {
       __builtin_amdgcn_sched_barrier(0);
-      if (q < 6) load_one(k + kStages, slot[0], q);
+      if (q < 6) load_one.template operator()<LA>(k + kStages, slot[0], q);
       if (q == 6 && KM == 0) load_scales((k >> 2) + 1 + E);
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -233,7 +254,7 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
     // K-tile k + 2 has landed: everything older than the loads of the last STAGES - 2 steps (six each, and a scale load
     // in steps with KM == 0)
     constexpr int kScalesInFlight = (KM % 4 == 0) + (STAGES >= 4 && (KM + 3) % 4 == 0) + (STAGES >= 5 && (KM + 2) % 4 == 0) + (STAGES >= 6 && (KM + 1) % 4 == 0);
-    wait_vmcnt<6 * (STAGES - 2) + kScalesInFlight>();
+    wait_vmcnt<(LA ? 6 : 3) * (STAGES - 2) + kScalesInFlight>();
     barrier();
     const int t = slot[0];
 #pragma unroll
@@ -241,24 +262,33 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
     slot[kStages - 1] = t;
   };
 
-  // prologue: scales of the first group(s), K-tiles 0 .. STAGES - 1
-  load_scales(0);
-  if (E) load_scales(1);
+  // prologue (scales of the first group(s), K-tiles 0 .. STAGES - 1) and the K loop
+  auto run = [&]<bool LA>() __attribute__((always_inline)) {
+    constexpr int NL = LA ? 6 : 3;
+    load_scales(0);
+    if (E) load_scales(1);
 #pragma unroll
-  for (int t = 0; t < kStages; t++) load_tile(t, t);
-  wait_vmcnt<6 * (STAGES - 1)>();
-  barrier();
-  read_tile.template operator()<0>(0);
-  read_scales(0);
-  wait_lds_reads();
-  take_scales();
-  wait_vmcnt<6 * (STAGES - 2)>();
-  barrier();  // K-tile 1 is in place, and every wave has K-tile 0 in registers: its slot is free
-  for (int k = 0; k < nkt; k += 4) {
-    step.template operator()<0>(k);
-    step.template operator()<1>(k + 1);
-    step.template operator()<2>(k + 2);
-    step.template operator()<3>(k + 3);
+    for (int t = 0; t < kStages; t++) load_tile.template operator()<LA>(t, t);
+    wait_vmcnt<NL * (STAGES - 1)>();
+    barrier();
+    read_tile.template operator()<0>(0);
+    read_scales(0);
+    wait_lds_reads();
+    take_scales();
+    wait_vmcnt<NL * (STAGES - 2)>();
+    barrier();  // K-tile 1 is in place, and every wave has K-tile 0 in registers: its slot is free
+    for (int k = 0; k < nkt; k += 4) {
+      step.template operator()<0, LA>(k);
+      step.template operator()<1, LA>(k + 1);
+      step.template operator()<2, LA>(k + 2);
+      step.template operator()<3, LA>(k + 3);
+    }
+  };
+  if constexpr (WN == 2) {
+    run.template operator()<true>();
+  } else {
+    if (loads_a) run.template operator()<true>();
+    else run.template operator()<false>();
   }
   wait_vmcnt<0>();  // no direct load may still be on its way into LDS when the workgroup gives the memory back
 
@@ -267,7 +297,7 @@ __global__ __launch_bounds__(NW * 64, STAGES <= 3 ? 2 : 1) void gemm_block_kerne
   // (v_permlane32_swap), so that every lane owns 8 consecutive outputs and stores them as 16 bytes.
   const int N = args.N, N2 = N * (int)sizeof(OutT);
   const bool edge = rows_a != kBM || rows_b != kBN;
-  const __amdgpu_buffer_rsrc_t rC = make_rsrc((OutT*)args.C + (size_t)pm * kBM * N + (size_t)pn * kBN,
+  const __amdgpu_buffer_rsrc_t rC = make_rsrc((OutT*)args.C + (size_t)share * args.M * N + (size_t)pm * kBM * N + (size_t)pn * kBN,
                                               (uint32_t)((rows_a - 1) * N + rows_b) * (uint32_t)sizeof(OutT));
   const int row_l = wm * 64 + r32;
   if constexpr (sizeof(OutT) == 2) {
@@ -336,13 +366,20 @@ int cu_count_of_device() {
 template <int FA, int FB>
 hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, hipStream_t s) {
   const int cus = cu_count_of_device();
-  if (stages == 0) stages = (long)tiles * 8 <= (long)cus * 5 || (g.K >= 8192 && tiles < cus) ? 6 : 3;
+  const bool f32 = g.f32out || a.nsplit > 1;  // shares leave fp32 partial sums
+  const int grid = tiles * a.nsplit;
+  if (g.tile_cols == 256) {  // tiles of 128 x 256, eight waves, four slots
+    if (f32) gemm_block_kernel<FA, FB, OutF32, 4, 4><<<grid, 512, 0, s>>>(a);
+    else gemm_block_kernel<FA, FB, OutBf16, 4, 4><<<grid, 512, 0, s>>>(a);
+    return hipGetLastError();
+  }
+  if (stages == 0) stages = (long)grid * 8 <= (long)cus * 5 || ((g.K >= 8192 || a.nsplit > 1) && grid < cus) ? 6 : 3;
   if (stages == 6) {
-    if (g.f32out) gemm_block_kernel<FA, FB, OutF32, 6><<<tiles, NW * 64, 0, s>>>(a);
-    else gemm_block_kernel<FA, FB, OutBf16, 6><<<tiles, NW * 64, 0, s>>>(a);
+    if (f32) gemm_block_kernel<FA, FB, OutF32, 6, 2><<<grid, 256, 0, s>>>(a);
+    else gemm_block_kernel<FA, FB, OutBf16, 6, 2><<<grid, 256, 0, s>>>(a);
   } else {
-    if (g.f32out) gemm_block_kernel<FA, FB, OutF32, 3><<<tiles, NW * 64, 0, s>>>(a);
-    else gemm_block_kernel<FA, FB, OutBf16, 3><<<tiles, NW * 64, 0, s>>>(a);
+    if (f32) gemm_block_kernel<FA, FB, OutF32, 3, 2><<<grid, 256, 0, s>>>(a);
+    else gemm_block_kernel<FA, FB, OutBf16, 3, 2><<<grid, 256, 0, s>>>(a);
   }
   return hipGetLastError();
 }
@@ -355,7 +392,7 @@ bool gemm_block_supports(const GemmArgs& g) {
   return g.M > 0 && g.N > 0 && g.K >= 512 && g.N % 8 == 0 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) &&
          (long)128 * g.N * 4 < (1L << 31) && (long)((g.M + 127) / 128) <= 65535 && (long)((g.N + 127) / 128) <= 32767 &&
          (long)((g.M + 127) / 128) * ((g.N + 127) / 128) < (1L << 31) && ((uintptr_t)g.C % 16) == 0 && operands_aligned16(g) && !g.fmt_c &&
-         !epilogue_any(g.ep) && !g.ksplit && !g.no_alloc;
+         (!epilogue_any(g.ep) || g.ksplit > 1) && !g.no_alloc;
 }
 
 // Automatic choice, from a sweep of 64 - 2048 rows of A against fourteen (N, K) pairs on MI355X (us, the kernel chosen
@@ -368,36 +405,105 @@ bool gemm_block_supports(const GemmArgs& g) {
 // row-major: more than 256 rows and K <= 5120 0.87 - 0.93, tiles on three quarters of the CUs and K <= 16384
 // (512 x 6144 x 16384 85 -> 67), K <= 4096 against 12288 rows of B or more 0.84 - 0.92; otherwise level or behind.  More
 // tiles than CUs: level with the 8-wave kernel's 128 x 256 tiles up to 512 tiles, behind beyond; not chosen.
-// first: asked before the tiled kernel's K split is considered -- where the tiles fill more than half the CUs and K is at
-// most 16384 this kernel is ahead of the split as well (640 x 4096 x 14336 0.82, 384 x 6144 x 16384 0.76), and with K up to
+// first: asked before the tiled kernel's K split is considered -- where the tiles fill more than half the CUs, K is at
+// most 16384 and both operands are tile-major this kernel is ahead of the split as well (640 x 4096 x 14336 0.85,
+// 384 x 6144 x 16384 0.84; with a row-major operand 0.92 - 1.11: left to the split), and with K up to
 // 8192 from a quarter of the CUs on (192 x 8192 x 8192 30.7 -> 22.5, 1024 x 2048 x 8192 32 -> 23.5; not with many rows of
 // a row-major A: 512 x 2048 x 8192 24.3 -> 28.8); with fewer tiles or a longer K the split wins (256 x 8192 x 28672 1.38,
 // 256 x 6144 x 16384 1.02, 256 x 4096 x 14336 1.11).
 bool gemm_block_preferred(const GemmArgs& g, bool first) {
   if (!gemm_block_supports(g) || g.ablation || g.clock_stamps) return false;
   const int cus = cu_count_of_device();
-  const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + kBN - 1) / kBN);
+  const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
   const int nkt = g.K / kBK;
   if (cus <= 0 || tiles > cus) return false;
   // tiles on more than half the CUs (three quarters with a row-major B), K up to 16384
   const bool fills = nkt <= 128 && (g.layout_b ? tiles * 16 >= (long)cus * 9 : tiles * 4 >= (long)cus * 3);
   // ... or on a quarter of them, K up to 8192 (a row-major A: up to 256 rows of it)
   const bool quarter = nkt <= 64 && tiles * 4 >= cus && g.layout_b && (g.layout_a || g.M <= 256);
-  if (first && !fills && !quarter) return false;
+  if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
   const bool wide_short = nkt <= 32 && g.N >= 12288;
-  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || wide_short;
+  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && g.M > 64);
   if (g.layout_a) return g.M > 128 || nkt <= 64;
   return g.M > 128 || nkt <= 16 || wide_short;
 }
 
+// The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
+// 128 x 256 ones, K up to 16384.  Measured (us, the 8-wave tiled kernel's choice -> this): 640 x 8192 x 8192 42.1 -> 37.5,
+// 1024 x 8192 x 8192 48.7 -> 45.3, 2048 x 4096 x 4096 27.7 -> 26.3; with a row-major A level (1024 x 8192 x 8192 50.3 / 50.7), with
+// more tiles than CUs behind (1536 x 8192 x 8192 62.5 -> 72.6).
+bool gemm_block_wide_preferred(const GemmArgs& g) {
+  if (!gemm_block_supports(g) || g.ablation || g.clock_stamps || !g.layout_a || !g.layout_b) return false;
+  const int cus = cu_count_of_device();
+  const long rows = (g.M + kBM - 1) / kBM, tiles = rows * ((g.N + 127) / 128), wide = rows * ((g.N + 255) / 256);
+  return cus > 0 && tiles > cus && wide <= cus && g.K <= 16384;
+}
+
+// K split of this kernel's 128 x 128 tiles: shares per output tile (1 = none) and the workspace they need.
+// want: 0 = where it pays (below), 1 = never, -1 = wherever the shape allows it, n > 1 = n shares if the shape allows it.
+// A share gets a whole number of groups of four K-tiles and at least 16 K-tiles (8 where that would leave most CUs
+// idle); the shares of all tiles together do not outnumber the CUs.  Where it pays (sweep of 48 - 512 rows x nine (N, K) pairs x three layout pairs on MI355X, us, the
+// choice before -> this, each timed twice in alternation): K from 8192 on (5120 with both operands tile-major; shorter,
+// two launches lose), at most half as many tiles as CUs, more than three eighths of them only for K = 14336 .. 16384
+// (with K = 8192 an unsplit launch of that many tiles is as fast, with K = 28672 the tiled kernel's split is:
+// 256 x 8192 x 28672 63.7 against 69.1), e.g. both operands tile-major 64 x 8192 x 28672 50 -> 40,
+// 128 x 8192 x 28672 62 -> 48 (the tiled kernel's split before), 128 x 4096 x 14336 23.8 -> 17.9, 256 x 8192 x 16384 50 -> 44.5,
+// 64 x 8192 x 8192 20.9 -> 16.1, 384 x 2048 x 8192 26.3 -> 17.5; A row-major (more than 32 rows of it: fewer are the skinny
+// kernel's), B tile-major: 64 x 8192 x 28672 46.8 -> 42.4, 96 x 8192 x 16384 40.7 -> 30.9, 192 x 4096 x 14336 33.1 -> 24.9; a
+// row-major operand: only up to a quarter as many tiles as CUs (256 x 2048 x 8192 23.3 -> 18.7, 128 x 4096 x 14336 27.9 -> 23.7;
+// beyond, level with or behind the tiled kernel's split: 128 x 12288 x 14336 47.5 against 50.8).
+int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
+  if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps) return 1;
+  GemmArgs plain = g;
+  plain.ep = Epilogue{};  // the reduction applies the epilogue
+  if (!gemm_block_supports(plain)) return 1;
+  const int cus = cu_count_of_device();
+  const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
+  const int nkt = g.K / kBK, groups = nkt / 4;
+  if (cus < 8 || tiles * 2 > cus) return 1;
+  if (want == 0) {
+    if (nkt < 64 && !(g.layout_a && g.layout_b && nkt >= 40)) return 1;  // two launches for a K this short lose (96 x 8192 x 2048: 11 -> 14 us)
+    if (tiles * 8 > (long)cus * 3 && (nkt < 112 || nkt > 128)) return 1;
+    if (!(g.layout_a && g.layout_b) && tiles * 4 > cus) return 1;
+    if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64))) return 1;  // the skinny kernel's (level at 33 - 64 rows and K = 8192)
+  }
+  // the most shares that leave each at least 16 K-tiles; if those are fewer workgroups than three eighths of the CUs, at
+  // least 8 K-tiles (64 x 1024 x 16384: 16 shares of 8 K-tiles 14.9 us, unsplit 20.4; 256 x 2048 x 8192: 4 shares of 16
+  // K-tiles 16.7, 8 of 8 18.2)
+  int best = 1;
+  for (int min_tiles = 16; min_tiles >= 8 && best <= 1; min_tiles -= 8) {
+    for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
+      if (groups % sh == 0 && nkt / sh >= min_tiles && tiles * sh <= cus) {
+        best = sh;
+        break;
+      }
+      if (want > 1) break;
+    }
+    if (want == 0 && best > 1 && tiles * best * 8 < (long)cus * 3) best = 1;  // too few workgroups: try shorter shares
+  }
+  if (best <= 1) return 1;
+  // K beyond 16384 and shares on fewer than three quarters of the CUs: the tiled kernel's split streams B faster
+  // (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7)
+  if (want == 0 && nkt > 128 && tiles * best * 4 < (long)cus * 3) return 1;
+  *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
+  return best;
+}
+
+// g.ksplit > 1 (with g.ks_part): the K range of every output tile split between that many workgroups, then
+// ksplit_reduce_kernel (gemm_tiled.hip), which also applies a fused epilogue.  The caller has checked that K / ksplit is a
+// whole number of groups of four K-tiles.
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s) {
-  BlockArgs a{g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, (g.M + kBM - 1) / kBM, (g.N + kBN - 1) / kBN, g.layout_a, g.layout_b,
-              g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1};
+  const int bn = g.tile_cols == 256 ? 256 : 128, nsplit = g.ksplit > 1 ? g.ksplit : 1;
+  BlockArgs a{g.A, g.B, g.As, g.Bs, nsplit > 1 ? (void*)g.ks_part : g.C, g.M, g.N, g.K, (g.M + kBM - 1) / kBM, (g.N + bn - 1) / bn, g.layout_a, g.layout_b,
+              g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, nsplit};
   const int tiles = a.tiles_m * a.tiles_n, stages = g.tile_rows == 3 || g.tile_rows == 6 ? g.tile_rows : 0;
-  if (g.fmt_a == 2 && g.fmt_b == 2) return launch<2, 2>(g, a, tiles, stages, s);
-  if (g.fmt_a == 2 && g.fmt_b == 3) return launch<2, 3>(g, a, tiles, stages, s);
-  if (g.fmt_a == 3 && g.fmt_b == 2) return launch<3, 2>(g, a, tiles, stages, s);
-  return launch<3, 3>(g, a, tiles, stages, s);
+  hipError_t e;
+  if (g.fmt_a == 2 && g.fmt_b == 2) e = launch<2, 2>(g, a, tiles, stages, s);
+  else if (g.fmt_a == 2 && g.fmt_b == 3) e = launch<2, 3>(g, a, tiles, stages, s);
+  else if (g.fmt_a == 3 && g.fmt_b == 2) e = launch<3, 2>(g, a, tiles, stages, s);
+  else e = launch<3, 3>(g, a, tiles, stages, s);
+  if (e == hipSuccess && nsplit > 1) e = launch_ksplit_reduce(g, s);
+  return e;
 }
 
 }  // namespace mxfp6

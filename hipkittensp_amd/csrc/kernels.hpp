@@ -43,7 +43,10 @@ bool gemm_tiled4_supports(const GemmArgs& g);  // the 4-wave variant of the tile
 hipError_t launch_gemm_tiled4(const GemmArgs& g, hipStream_t s);
 bool gemm_block_supports(const GemmArgs& g);  // 128 x 128 tiles, four waves in step (a few hundred to a few thousand rows of A)
 bool gemm_block_preferred(const GemmArgs& g, bool first);  // by shape; first: even before the tiled kernel's K split is considered
+bool gemm_block_wide_preferred(const GemmArgs& g);  // its 128 x 256 tiles (eight waves) beat the 8-wave tiled kernel's
+int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes);  // K split of the block kernel for this problem: shares per tile (1 = none)
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s);
+hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s);  // sums g.ksplit partial matrices at g.ks_part into g.C, with the epilogue
 bool gemm_mid_supports(const GemmArgs& g);
 bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
 double tiled_estimate_us(const GemmArgs& g, int rows, int cols = 256);  // estimated time of the tiled kernel with tiles of rows x cols

@@ -47,6 +47,7 @@ KERNEL_SKINNY_64 = 19  # skinny kernel with 64 rows of B per workgroup (two tile
 KERNEL_SKINNY_64_SPLIT = (20, 21)  # the same with the K range split between 2 / 4 workgroups
 KERNEL_BLOCK = 22  # 128 x 128 tiles, four waves in step: one barrier per K-tile, fragments double-buffered in registers
 KERNEL_BLOCK_3SLOTS, KERNEL_BLOCK_6SLOTS = 23, 24  # the same with its operand ring forced to three / six slots
+KERNEL_BLOCK_WIDE = 26  # the block kernel with tiles of 128 x 256 and eight waves
 KERNEL_TILED_4WAVE = 18  # the 4-wave interleaved schedule of the tiled kernel (measurement: never chosen automatically)
 
 
@@ -287,14 +288,20 @@ def k_split_plan(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, shares: int
 
 
 CHOICE_TILED_K_SPLIT = 25  # kernel_choice(): the tiled kernel with its K split between workgroups
+CHOICE_BLOCK_K_SPLIT = 27  # kernel_choice(): the block kernel with its K split between workgroups
 
 
 def kernel_choice(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, layout_b: int = LAYOUT_ROW) -> int:
-    """The kernel (KERNEL_* code, or CHOICE_TILED_K_SPLIT) the automatic path takes for this shape; launches nothing."""
+    """The kernel (KERNEL_* code, or CHOICE_TILED_K_SPLIT / CHOICE_BLOCK_K_SPLIT) the automatic path takes for this shape; launches nothing."""
     n = _lib.lib().mxfp6_probe_choice(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1)
     if n < 0:
         _lib.check(n, "kernel_choice")
     return n
+
+
+def set_block_kernel(enable: bool) -> bool:
+    """Measurement: keep the block kernel out of (False) or in (True, the default) the automatic choice; returns the previous setting."""
+    return bool(_lib.lib().mxfp6_probe_block(int(bool(enable))))
 
 
 def set_kernel(which: int) -> int:

@@ -120,7 +120,9 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *   22  block kernel: output tiles of 128 x 128, four waves in step with the operand fragments double-buffered in
  *       registers, one barrier per K-tile (needs N % 8 == 0, K % 512 == 0, no fused epilogue); chosen automatically where
  *       its tiles do not outnumber the CUs and K is of moderate length (a few hundred rows of A);
- *       23 / 24: with an operand ring of three slots (two workgroups per CU) / six slots (one)
+ *       23 / 24: with an operand ring of three slots (two workgroups per CU) / six slots (one); 26: with tiles of
+ *       128 x 256 and eight waves.  22 - 24 split K between workgroups by the thread's mxfp6_probe_ksplit setting
+ *       (0: where the library's rule for this kernel says so; the same per-stream workspace as the tiled kernel's split)
  * No counterpart in the reference, whose shapes are compile-time constants per binary
  * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
  */
@@ -343,9 +345,14 @@ int mxfp6_probe_ksplit(int shares);
  * on them). */
 int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int *tile_rows);
 
+/* Measurement switch, per calling thread: 0 keeps the block kernel (mxfp6_set_kernel 22 - 27) out of the automatic choice,
+ * so that the same call can be timed with and without it; returns the previous setting.  Default 1. */
+int mxfp6_probe_block(int enable);
+
 /* The kernel the automatic path takes for a problem of this shape on the current device (e2m3 x e2m3, bf16 output, no fused
- * epilogue, 16-byte aligned tensors): a code of mxfp6_set_kernel (1 generic, 2 tiled, 3 skinny, 4 mid-M, 22 block), or 25
- * for the tiled kernel with its K split between workgroups; negative = error code.  layouts as in
+ * epilogue, 16-byte aligned tensors): a code of mxfp6_set_kernel (1 generic, 2 tiled, 3 skinny, 4 mid-M, 22 block, 26
+ * block with 128 x 256 tiles), or 25 / 27 for the tiled / the block kernel with its K split between workgroups; negative =
+ * error code.  layouts as in
  * mxfp6_probe_ksplit_plan.  Reads the thread's mxfp6_probe_ksplit setting; launches nothing. */
 int mxfp6_probe_choice(int M, int N, int K, int layouts);
 

@@ -145,7 +145,7 @@ def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
 @pytest.mark.parametrize("M,N,K", [(128, 128, 512), (256, 384, 1024), (512, 256, 2560), (300, 264, 1536), (129, 8, 512), (100, 1000, 1024), (33, 520, 2048),
                                    (1, 128, 512), (640, 1024, 4096)])  # edge tiles too; K in whole groups of four K-tiles
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
-@pytest.mark.parametrize("kernel", [23, 24])  # ring of three slots (two workgroups per CU) and of six (one)
+@pytest.mark.parametrize("kernel", [23, 24, 26])  # ring of three slots (two workgroups per CU), of six (one); tiles of 128 x 256
 def test_block_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
     ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M * 5 + N + K, kind_a="laplace" if fa == 3 else "normal", kind_b="weights")
     ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
@@ -153,7 +153,7 @@ def test_block_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
     check(got, ref, fa, fb, ap, asc, bp, bsc)
     cb = gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=kernel)
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
-    assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=22), got)   # ring depth chosen by the library: same bits
+    assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=22), got)   # ring depth chosen by the library, 128 x 128 tiles: same bits
 
 
 @pytest.mark.parametrize("M,N,K,la,lb", [(256, 8192, 2048, 1, 1), (192, 4096, 4096, 0, 1), (512, 3072, 3072, 0, 0), (1024, 2048, 8192, 1, 1), (96, 16384, 1024, 0, 1),
@@ -186,19 +186,67 @@ def test_block_kernel_is_chosen_and_matches_the_tiled_kernel(hk, M, N, K, la, lb
     check(outs[22][rows], o.gemm_ref(ap[rows], bp, asc[rows], bsc, acc=np.float64), 2, 2)
 
 
+@pytest.mark.parametrize("M,N,K,shares", [(128, 256, 4096, 2), (128, 512, 8192, 4), (100, 264, 4096, 2), (256, 512, 8192, 8), (64, 1024, 16384, 0), (192, 2048, 8192, 0)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
+def test_block_kernel_k_split(hk, M, N, K, shares, fa, fb):
+    """The block kernel with the K range of every output tile split between several workgroups: fp32 partial matrices in
+    the stream's workspace, summed in share order by the tiled kernel's reduction.  Forced share counts on the forced
+    kernel, and shapes on which the automatic path chooses this split itself.  Against the fp64 oracle; bf16 output = RNE
+    of the fp32 output; a second call gives the same bits; tile-major operands give the same bits as row-major ones; a
+    fused epilogue is applied by the reduction."""
+    tk = hk.tk_kernel
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M + N + K + shares, kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    kernel = 22 if shares else 0
+    if not shares:
+        assert tk.kernel_choice(M, N, K) == tk.CHOICE_BLOCK_K_SPLIT
+    prev = tk.set_k_split(shares)
+    try:
+        got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel)
+        check(got, ref, fa, fb, ap, asc, bp, bsc)
+        assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=kernel), got)
+        assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=kernel), o.f32_to_bf16_bits(got))
+        if N % 32 == 0:
+            C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            pk = tk.set_kernel(kernel)
+            try:
+                hk.dispatch_micro(dev(ap), hk.tile_operand(dev(bp)), dev(asc), hk.tile_scales(dev(bsc), K), C, fa, fb, layout_b=1)
+                torch.cuda.synchronize()
+            finally:
+                tk.set_kernel(pk)
+            if shares:
+                assert np.array_equal(C.cpu().numpy(), got)
+            else:
+                check(C.cpu().numpy(), ref, fa, fb, ap, asc, bp, bsc)  # the automatic path may take another split for another layout
+        if not shares:
+            bias = torch.linspace(-1, 1, N, device="cuda")
+            C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            hk.dispatch_micro(dev(ap), dev(bp), dev(asc), dev(bsc), C, fa, fb, bias=bias, activation="relu")
+            torch.cuda.synchronize()
+            want = np.maximum(got + bias.cpu().numpy()[None, :], 0)
+            assert np.allclose(C.cpu().numpy(), want, rtol=1e-6, atol=1e-6 * np.abs(got).max())
+    finally:
+        tk.set_k_split(prev)
+
+
 def test_kernel_choice_by_shape(hk):
     """The automatic choice over the library's kernels, as mxfp6_probe_choice reports it (A row-major unless stated)."""
     tk = hk.tk_kernel
     assert tk.kernel_choice(8192, 8192, 8192) == tk.KERNEL_TILED
     assert tk.kernel_choice(16, 8192, 28672) == tk.KERNEL_SKINNY and tk.kernel_choice(64, 8192, 8192, 0, 1) == tk.KERNEL_SKINNY
-    assert tk.kernel_choice(256, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT
+    assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT
+    assert tk.kernel_choice(256, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT    # K this long and 128 tiles of 128 x 128: the tiled kernel's split streams B faster
+    assert tk.kernel_choice(256, 8192, 16384, 1, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 4096, 14336, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT
+    assert tk.kernel_choice(96, 8192, 2048, 1, 1) != tk.CHOICE_BLOCK_K_SPLIT      # two launches for a K this short lose
+    assert tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(32, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY
     assert tk.kernel_choice(256, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(512, 4096, 4096, 0, 1) == tk.KERNEL_BLOCK
-    assert tk.kernel_choice(2048, 8192, 8192, 1, 1) == tk.KERNEL_TILED      # more 128 x 128 tiles than CUs
+    assert tk.kernel_choice(2048, 8192, 8192, 1, 1) == tk.KERNEL_TILED      # more 128 x 256 tiles than CUs
+    assert tk.kernel_choice(1024, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK_WIDE and tk.kernel_choice(1024, 8192, 8192, 0, 1) == tk.KERNEL_TILED
     assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_TILED  # K % 512
     assert tk.kernel_choice(40, 36, 96) == tk.KERNEL_GENERIC
     prev = tk.set_k_split(1)
     try:
-        assert tk.kernel_choice(256, 8192, 28672, 1, 1) != tk.CHOICE_TILED_K_SPLIT
+        assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY   # no split
     finally:
         tk.set_k_split(prev)
 
@@ -485,7 +533,7 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
     assert np.array_equal(hk.tile_scales(ts, K, untile=True).cpu().numpy(), sr)
 
 
-@pytest.mark.parametrize("kernel,M,N,K", [(23, 256, 512, 1024), (24, 320, 544, 1536), (1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
+@pytest.mark.parametrize("kernel,M,N,K", [(23, 256, 512, 1024), (24, 320, 544, 1536), (26, 256, 1024, 1024), (1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
                                           (18, 256, 512, 640), (18, 320, 544, 1152), (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
