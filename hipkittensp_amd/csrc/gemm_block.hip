@@ -425,7 +425,10 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   const bool wide_short = nkt <= 32 && g.N >= 12288;
   if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && g.M > 64);
   if (g.layout_a) return g.M > 128 || nkt <= 64;
-  return g.M > 128 || nkt <= 16 || wide_short;
+  // A row-major, B tile-major, few rows: the skinny kernel's, except a short K (above) and a B of 20480 .. 32767 rows
+  // (its tiles on five eighths of the CUs or more, one CU at least left over): 32 x 20480 x 8192 38.3 -> 30.7 us,
+  // 16 x 28672 x 8192 37.9 -> 33.6, 32 x 28672 x 16384 74.6 -> 66.3; 16384 rows 21 -> 26, 32768 rows level
+  return g.M > 128 || nkt <= 16 || wide_short || (tiles * 8 >= (long)cus * 5 && tiles < cus && nkt <= 128);
 }
 
 // The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
@@ -463,8 +466,15 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   if (cus < 8 || tiles * 2 > cus) return 1;
   if (want == 0) {
     if (nkt < 64 && !(g.layout_a && g.layout_b && nkt >= 40)) return 1;  // two launches for a K this short lose (96 x 8192 x 2048: 11 -> 14 us)
-    if (tiles * 8 > (long)cus * 3 && (nkt < 112 || nkt > 128)) return 1;
-    if (!(g.layout_a && g.layout_b) && tiles * 4 > cus) return 1;
+    const bool both = g.layout_a && g.layout_b;
+    if (tiles * 8 > (long)cus * 3) {  // more than three eighths as many tiles as CUs
+      // both tile-major: only K = 14336 .. 16384 (at 8192 the unsplit launch is as fast: 256 x 8192 x 8192 22.9 us against
+      // 26.5; at 28672 the tiled kernel's split is); a row-major operand: only K = 8192 (192 x 8192 x 8192, A row-major:
+      // 26.9 -> 22.8, both row-major 29.9 -> 25.3; 256 x 8192 x 16384 49.3 -> 51.6)
+      if (both ? (nkt < 112 || nkt > 128) : nkt > 64) return 1;
+    } else if (!both && tiles * 4 > cus && nkt > 64) {
+      return 1;  // a row-major operand and more than a quarter as many tiles as CUs: likewise only K = 8192
+    }
     if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64))) return 1;  // the skinny kernel's (level at 33 - 64 rows and K = 8192)
   }
   // the most shares that leave each at least 16 K-tiles; if those are fewer workgroups than three eighths of the CUs, at
