@@ -423,12 +423,12 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   const bool quarter = nkt <= 64 && tiles * 4 >= cus && g.layout_b && (g.layout_a || g.M <= 256);
   if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
   const bool wide_short = nkt <= 32 && g.N >= 12288;
-  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && g.M > 64);
+  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5)));
   if (g.layout_a) return g.M > 128 || nkt <= 64;
   // A row-major, B tile-major, few rows: the skinny kernel's, except a short K (above) and a B of 20480 .. 32767 rows
   // (its tiles on five eighths of the CUs or more, one CU at least left over): 32 x 20480 x 8192 38.3 -> 30.7 us,
   // 16 x 28672 x 8192 37.9 -> 33.6, 32 x 28672 x 16384 74.6 -> 66.3; 16384 rows 21 -> 26, 32768 rows level
-  return g.M > 128 || nkt <= 16 || wide_short || (tiles * 8 >= (long)cus * 5 && tiles < cus && nkt <= 128);
+  return g.M > 128 || nkt <= 16 || (wide_short && g.M > 32) || (tiles * 8 >= (long)cus * 5 && tiles < cus && nkt <= 128);
 }
 
 // The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
@@ -475,7 +475,9 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
     } else if (!both && tiles * 4 > cus && nkt > 64) {
       return 1;  // a row-major operand and more than a quarter as many tiles as CUs: likewise only K = 8192
     }
-    if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64))) return 1;  // the skinny kernel's (level at 33 - 64 rows and K = 8192)
+    // the skinny kernel's (level at 33 - 64 rows and K = 8192 while N is one of its whole rounds: 64 x 8192 x 8192 16.1 us
+    // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
+    if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)))) return 1;
   }
   // the most shares that leave each at least 16 K-tiles; if those are fewer workgroups than three eighths of the CUs, at
   // least 8 K-tiles (64 x 1024 x 16384: 16 shares of 8 K-tiles 14.9 us, unsplit 20.4; 256 x 2048 x 8192: 4 shares of 16
