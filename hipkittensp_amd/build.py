@@ -43,7 +43,7 @@ def _compile(unit) -> str:
 def build(verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     # the units that take longest first
-    order = sorted(UNITS, key=lambda u: (not u[1].startswith("gemm_tiled_fmt"), u[1] not in ("gemm_skinny", "gemm_mid")))
+    order = sorted(UNITS, key=lambda u: (u[1] != "gemm_block", not u[1].startswith("gemm_tiled_fmt"), u[1] not in ("gemm_skinny", "gemm_mid")))
     with cf.ThreadPoolExecutor(max_workers=min(8, len(order))) as ex:
         objs = list(ex.map(_compile, order))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]

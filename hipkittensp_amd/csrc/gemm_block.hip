@@ -12,7 +12,8 @@
 //
 // Same operand formats, LDS image, lane mapping and raster as the tiled kernel (common.hpp, gemm_tiled.hip): row-major
 // or tile-major operands and scales, any M and N (edge tiles: rows past M or N lie beyond the end of their buffer
-// resource and read as zeros, stores are predicated), K % 512 == 0, bf16 or fp32 output, no fused epilogue.
+// resource and read as zeros, stores are predicated), K % 512 == 0, bf16 or fp32 output, fused scales / bias / activation
+// (separate instantiations).
 //   ring: three slots of 24 KB (A's 128 rows x 96 bytes, then B's); K-tile k lives in slot k % 3
 //   scales: the 16 bytes a row has for four K-tiles, two buffers of (128 + 128) rows x 16 bytes, group g in buffer g % 2
 //   step k: loads of K-tile k+3 into the slot K-tile k has left (its fragments are in registers since step k-1), LDS
@@ -52,6 +53,7 @@ struct BlockArgs {
   void* C;
   int M, N, K, tiles_m, tiles_n, layout_a, layout_b, group_m, xcd_remap;
   int nsplit;  // workgroups that share an output tile, each over K / nsplit (a whole number of groups of four K-tiles); 1 = no split
+  Epilogue ep;  // FUSED instantiations: scales / bias / activation on the accumulators before the output rounding
 };
 
 // STAGES: ring slots, 3 (80 KB of LDS, two workgroups per CU) to 6 (152 KB, one).  Loads run STAGES K-tiles ahead of the
@@ -59,7 +61,8 @@ struct BlockArgs {
 // that they are older than every load a step's wait leaves in flight.
 // WN: waves side by side along N, 2 (tile of 128 x 128, four waves) or 4 (128 x 256, eight waves: waves 0-3 load A's tile
 // and half of B's, six loads per K-tile, waves 4-7 the other half of B's, three loads).
-template <int FA, int FB, typename Out, int STAGES, int WN>
+// FUSED: the epilogue applies args.ep (a separate instantiation, so that unfused calls carry none of it).
+template <int FA, int FB, typename Out, int STAGES, int WN, bool FUSED>
 __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_block_kernel(const BlockArgs args) {
   typedef typename Out::type OutT;
   static_assert(STAGES >= 3 && STAGES <= 6 && (WN == 2 || WN == 4), "ring depth, tile width");
@@ -297,6 +300,44 @@ __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_bl
   // (v_permlane32_swap), so that every lane owns 8 consecutive outputs and stores them as 16 bytes.
   const int N = args.N, N2 = N * (int)sizeof(OutT);
   const bool edge = rows_a != kBM || rows_b != kBN;
+  if constexpr (FUSED) {
+    // y = act(acc * row_scale[m] * col_scale[n] + bias[n]) in fp32.  Per 32 x 32 tile a lane owns row 32 i + lane % 32 of its
+    // wave's rows and columns 8 q + 4 h .. + 3 for q = 0 .. 3; N % 8 == 0, so a run of four is inside or outside N as a whole
+    const void* bias = args.ep.bias;
+    const float *row_scale = args.ep.row_scale, *col_scale = args.ep.col_scale;
+    const int act = args.ep.act, bias_bf16 = args.ep.bias_bf16;
+    const long m0 = (long)pm * kBM + wm * 64 + r32, n0 = (long)pn * kBN + wn * 64 + 4 * h;
+    float rs[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) rs[i] = row_scale && m0 + i * 32 < args.M ? row_scale[m0 + i * 32] : 1.f;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      if (bias || row_scale || col_scale) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const long n = n0 + j * 32 + q * 8;
+          v4f cs = {1.f, 1.f, 1.f, 1.f}, bi = {0.f, 0.f, 0.f, 0.f};
+          if (n < N) {
+            if (col_scale) cs = *reinterpret_cast<const v4f*>(col_scale + n);
+            if (bias && bias_bf16) {
+              const u32x2 b2 = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(bias) + n);
+              bi = v4f{__uint_as_float(b2[0] << 16), __uint_as_float(b2[0] & 0xffff0000u), __uint_as_float(b2[1] << 16), __uint_as_float(b2[1] & 0xffff0000u)};
+            } else if (bias) {
+              bi = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(bias) + n);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[i][j][4 * q + e] = fmaf(acc[i][j][4 * q + e] * rs[i], cs[e], bi[e]);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[i][j][e] = epilogue_act(acc[i][j][e], act);
+    }
+  }
   const __amdgpu_buffer_rsrc_t rC = make_rsrc((OutT*)args.C + (size_t)share * args.M * N + (size_t)pm * kBM * N + (size_t)pn * kBN,
                                               (uint32_t)((rows_a - 1) * N + rows_b) * (uint32_t)sizeof(OutT));
   const int row_l = wm * 64 + r32;
@@ -363,25 +404,31 @@ int cu_count_of_device() {
 // other's work (256 tiles: 1024 x 4096 x 4096 18.6 against 20.0, 512 x 8192 x 2048 11.9 against 13.6, 2048 x 2048 x 8192
 // 28.8 against 31.2) -- except with K from 8192 on while a CU is left over (512 x 6144 x 16384: six slots 46.0 against
 // 51.9, 64 x 28672 x 8192: 34.9 against 38.2).  stages = 3 or 6 forces one (measurement).
-template <int FA, int FB>
+template <int FA, int FB, bool FUSED>
 hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, hipStream_t s) {
   const int cus = cu_count_of_device();
   const bool f32 = g.f32out || a.nsplit > 1;  // shares leave fp32 partial sums
   const int grid = tiles * a.nsplit;
   if (g.tile_cols == 256) {  // tiles of 128 x 256, eight waves, four slots
-    if (f32) gemm_block_kernel<FA, FB, OutF32, 4, 4><<<grid, 512, 0, s>>>(a);
-    else gemm_block_kernel<FA, FB, OutBf16, 4, 4><<<grid, 512, 0, s>>>(a);
+    if (f32) gemm_block_kernel<FA, FB, OutF32, 4, 4, FUSED><<<grid, 512, 0, s>>>(a);
+    else gemm_block_kernel<FA, FB, OutBf16, 4, 4, FUSED><<<grid, 512, 0, s>>>(a);
     return hipGetLastError();
   }
   if (stages == 0) stages = (long)grid * 8 <= (long)cus * 5 || ((g.K >= 8192 || a.nsplit > 1) && grid < cus) ? 6 : 3;
   if (stages == 6) {
-    if (f32) gemm_block_kernel<FA, FB, OutF32, 6, 2><<<grid, 256, 0, s>>>(a);
-    else gemm_block_kernel<FA, FB, OutBf16, 6, 2><<<grid, 256, 0, s>>>(a);
+    if (f32) gemm_block_kernel<FA, FB, OutF32, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
+    else gemm_block_kernel<FA, FB, OutBf16, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
   } else {
-    if (f32) gemm_block_kernel<FA, FB, OutF32, 3, 2><<<grid, 256, 0, s>>>(a);
-    else gemm_block_kernel<FA, FB, OutBf16, 3, 2><<<grid, 256, 0, s>>>(a);
+    if (f32) gemm_block_kernel<FA, FB, OutF32, 3, 2, FUSED><<<grid, 256, 0, s>>>(a);
+    else gemm_block_kernel<FA, FB, OutBf16, 3, 2, FUSED><<<grid, 256, 0, s>>>(a);
   }
   return hipGetLastError();
+}
+template <int FA, int FB>
+hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, hipStream_t s) {
+  // a split leaves the epilogue to the reduction
+  if (a.nsplit == 1 && epilogue_any(g.ep)) return launch<FA, FB, true>(g, a, tiles, stages, s);
+  return launch<FA, FB, false>(g, a, tiles, stages, s);
 }
 
 }  // namespace
@@ -392,7 +439,7 @@ bool gemm_block_supports(const GemmArgs& g) {
   return g.M > 0 && g.N > 0 && g.K >= 512 && g.N % 8 == 0 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) &&
          (long)128 * g.N * 4 < (1L << 31) && (long)((g.M + 127) / 128) <= 65535 && (long)((g.N + 127) / 128) <= 32767 &&
          (long)((g.M + 127) / 128) * ((g.N + 127) / 128) < (1L << 31) && ((uintptr_t)g.C % 16) == 0 && operands_aligned16(g) && !g.fmt_c &&
-         (!epilogue_any(g.ep) || g.ksplit > 1) && !g.no_alloc;
+         !g.no_alloc;
 }
 
 // Automatic choice, from a sweep of 64 - 2048 rows of A against fourteen (N, K) pairs on MI355X (us, the kernel chosen
@@ -457,9 +504,7 @@ bool gemm_block_wide_preferred(const GemmArgs& g) {
 // beyond, level with or behind the tiled kernel's split: 128 x 12288 x 14336 47.5 against 50.8).
 int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps) return 1;
-  GemmArgs plain = g;
-  plain.ep = Epilogue{};  // the reduction applies the epilogue
-  if (!gemm_block_supports(plain)) return 1;
+  if (!gemm_block_supports(g)) return 1;
   const int cus = cu_count_of_device();
   const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
   const int nkt = g.K / kBK, groups = nkt / 4;
@@ -507,7 +552,7 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s) {
   const int bn = g.tile_cols == 256 ? 256 : 128, nsplit = g.ksplit > 1 ? g.ksplit : 1;
   BlockArgs a{g.A, g.B, g.As, g.Bs, nsplit > 1 ? (void*)g.ks_part : g.C, g.M, g.N, g.K, (g.M + kBM - 1) / kBM, (g.N + bn - 1) / bn, g.layout_a, g.layout_b,
-              g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, nsplit};
+              g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, nsplit, g.ep};
   const int tiles = a.tiles_m * a.tiles_n, stages = g.tile_rows == 3 || g.tile_rows == 6 ? g.tile_rows : 0;
   hipError_t e;
   if (g.fmt_a == 2 && g.fmt_b == 2) e = launch<2, 2>(g, a, tiles, stages, s);

@@ -705,7 +705,7 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
 # ------------------------------------------------------------------ fused epilogue
 @pytest.mark.parametrize("kernel,M,N,K", [(1, 70, 40, 96), (3, 16, 96, 1024), (3, 32, 100, 512), (4, 64, 72, 1024), (4, 200, 136, 2048),
                                           (5, 300, 264, 640), (6, 300, 264, 640), (5, 1024, 4104, 512), (6, 2304, 8200, 512),
-                                          (17, 300, 264, 640), (17, 1024, 4104, 512)])
+                                          (17, 300, 264, 640), (17, 1024, 4104, 512), (23, 300, 264, 1024), (24, 200, 136, 2048), (26, 300, 520, 1024)])
 @pytest.mark.parametrize("activation", [None, "relu", "gelu", "silu"])
 def test_fused_epilogue_every_kernel(hk, kernel, M, N, K, activation):
     """act(acc * row_scale * col_scale + bias) fused into each kernel's epilogue (the last two shapes have more tiles than
