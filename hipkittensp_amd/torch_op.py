@@ -67,6 +67,10 @@ class MXFP6Linear(torch.nn.Module):
         self.register_buffer("weight_scale", scales)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        xp, xs = tk_kernel.quantize((x if x.dtype == torch.bfloat16 else x.to(torch.float32)).contiguous(), self.fmt_x)
-        return mxfp6_gemm(xp, self.weight_packed, xs, self.weight_scale, self.fmt_x, self.fmt_w, tk_kernel.LAYOUT_ROW, self.layout_w,
+        # the input tile-major too from 64 rows on (a whole number of 32-row tiles): the tiled and block kernels then need
+        # no re-layout and load whole cache lines; fewer rows stay row-major for the skinny kernel
+        rows = x.numel() // x.shape[-1]
+        layout_x = tk_kernel.LAYOUT_TILE if (rows >= 64 and rows % 32 == 0 and self.in_features % 128 == 0) else tk_kernel.LAYOUT_ROW
+        xp, xs = tk_kernel.quantize((x if x.dtype == torch.bfloat16 else x.to(torch.float32)).contiguous(), self.fmt_x, layout_x)
+        return mxfp6_gemm(xp, self.weight_packed, xs, self.weight_scale, self.fmt_x, self.fmt_w, layout_x, self.layout_w,
                           bias=self.bias, activation=self.activation)

@@ -852,6 +852,12 @@ def test_torch_op_and_linear_module(hk):
     y2 = lin2(dev(x)).float().cpu().numpy().reshape(48, 160)
     want = o.epilogue_ref(ref, bias=b, activation="silu")
     assert o.rel_err(y2, want) <= 2 ** -7
+    # from 64 rows on (a whole number of 32-row tiles) the input is quantised tile-major: same bytes regrouped, same result
+    x3 = o.make_source("normal", (4, 64, 1024), rng)
+    y3 = lin2(dev(x3)).float().cpu().numpy().reshape(256, 160)
+    xp3, xs3 = co.quantise(x3.reshape(256, 1024), 2)
+    want3 = o.epilogue_ref(o.gemm_ref(xp3, wp, xs3, ws, acc=np.float32), bias=b, activation="silu")
+    assert o.rel_err(y3, want3) <= 2 ** -7
 
 
 # ------------------------------------------------------------------ edge cases
