@@ -437,12 +437,22 @@ def test_skinny_k_split_chosen_by_shape_streams_and_capture(hk):
         torch.cuda.synchronize()
 
 
-def test_tiled_k_split_streams_and_capture(hk):
-    """The tiled kernel's K split on a shape where the automatic path chooses it (a few hundred rows of A, long K):
-    against the generic kernel; two streams at once, each with its own workspace of partial sums; under stream capture
-    on a stream that has its workspace already (captured with the split) and replayed with eager work in between."""
+@pytest.mark.parametrize("block", [True, False])
+def test_k_split_streams_and_capture(hk, block):
+    """A K split on a shape where the automatic path chooses one (a few hundred rows of A, long K) -- the block kernel's,
+    and with that kernel kept out of the choice the tiled kernel's: against the generic kernel; two streams at once, each
+    with its own workspace of partial sums; under stream capture on a stream that has its workspace already (captured
+    with the split) and replayed with eager work in between."""
     M, N, K = 192, 1024, 16384
-    assert hk.tk_kernel.k_split_plan(M, N, K)[0] > 1
+    prev_block = hk.tk_kernel.set_block_kernel(block)
+    try:
+        assert hk.tk_kernel.kernel_choice(M, N, K) == (hk.tk_kernel.CHOICE_BLOCK_K_SPLIT if block else hk.tk_kernel.CHOICE_TILED_K_SPLIT)
+        _k_split_streams_and_capture(hk, M, N, K)
+    finally:
+        hk.tk_kernel.set_block_kernel(prev_block)
+
+
+def _k_split_streams_and_capture(hk, M, N, K):
     g = torch.Generator(device="cuda"); g.manual_seed(9)
     a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
     b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2)
