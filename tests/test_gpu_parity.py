@@ -452,6 +452,31 @@ def test_k_split_streams_and_capture(hk, block):
         hk.tk_kernel.set_block_kernel(prev_block)
 
 
+def test_capture_on_a_stream_without_workspace_runs_unsplit(hk):
+    """A shape the automatic path would split, captured on a stream that has never launched one: the library may not
+    allocate during capture, so the graph holds the unsplit launch; every replay gives the eager (split) result to
+    fp32 rounding of the sums, and nothing is left allocated by the capture."""
+    M, N, K = 192, 1024, 16384
+    assert hk.tk_kernel.kernel_choice(M, N, K) == hk.tk_kernel.CHOICE_BLOCK_K_SPLIT
+    g = torch.Generator(device="cuda"); g.manual_seed(10)
+    a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+    b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2)
+    eager = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    hk.dispatch_micro(a, b, asc, bsc, eager)
+    torch.cuda.synchronize()
+    fresh = torch.cuda.Stream()
+    Cg = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    fresh.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=fresh):
+        hk.dispatch_micro(a, b, asc, bsc, Cg)
+    for rep in range(2):
+        Cg.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert o.rel_err(Cg.cpu().numpy(), eager.cpu().numpy()) <= TOL_TIGHT, f"replay {rep}"
+
+
 def _k_split_streams_and_capture(hk, M, N, K):
     g = torch.Generator(device="cuda"); g.manual_seed(9)
     a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
