@@ -2,8 +2,8 @@
 // kernel selection.  Nothing here synchronises the device.  Allocations, all from the stream-ordered allocator on the
 // caller's stream and all kept per (device, stream) until mxfp6_release_workspaces(): the workspace of the re-layout
 // pre-pass (relayout_then_tiled; mxfp6_set_relayout(0) switches it off), the fp32 workspace of mxfp6_gemm_fused_fp6
-// on shapes the tiled kernel does not run, the partial sums of the tiled kernel's K split (plan_ksplit), and the K-split
-// workspace of the skinny kernel (gemm_skinny.hip).  mxfp6_gemm_noalloc allocates nothing.
+// on shapes the tiled kernel does not run, the partial sums of the tiled and the block kernel's K split (plan_ksplit,
+// plan_block_ksplit: one workspace, shared), and the K-split workspace of the skinny kernel (gemm_skinny.hip).  mxfp6_gemm_noalloc allocates nothing.
 #include "../../include/mxfp6_gemm.h"
 
 #include <map>

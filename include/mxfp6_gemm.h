@@ -27,8 +27,9 @@
  *   - mxfp6_gemm_fused_fp6 on shapes the LDS-tiled kernel does not run: 4 M N bytes;
  *   - the gemm entry points on decode shapes whose K range is split between workgroups (M <= 32, N <= 2048,
  *     K >= 24576): 2 MB;
- *   - the gemm entry points on problems of few output tiles and long K (a few hundred rows of A, K >= 8192; see
- *     mxfp6_probe_ksplit), where the LDS-tiled kernel splits K between workgroups: shares * 4 M N bytes, at most 64 MB.
+ *   - the gemm entry points on problems of few output tiles and long K (up to a few hundred rows of A, K >= 5120; see
+ *     mxfp6_probe_ksplit), where the LDS-tiled kernel or the block kernel splits K between workgroups: shares * 4 M N
+ *     bytes, at most 64 MB (one workspace for both kernels).
  * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K splits are left out
  * (same results up to the order of fp32 sums, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
  * hipErrorStreamCaptureUnsupported where it would need a new one.  mxfp6_gemm_noalloc never allocates.
@@ -324,7 +325,8 @@ int mxfp6_probe_tiled_ablation(int mask);
 int mxfp6_probe_raster(int group_m, int xcd_remap);
 
 /*
- * K split of the LDS-tiled kernel (per calling thread, measurement and tests; returns the previous setting).  Problems of
+ * K split of the LDS-tiled kernel and of the block kernel (per calling thread, measurement and tests; returns the previous
+ * setting; 1 switches both off, 0 lets each kernel's own rule decide, -1 / n apply to whichever of the two runs).  Problems of
  * few output tiles and long K (a few hundred rows of A against a wide weight matrix) run with several workgroups per
  * output tile, each over a part of K: the shares leave their fp32 sums in this stream's workspace (shares * M * N * 4
  * bytes, hipMallocAsync on the caller's stream at first use, kept until mxfp6_release_workspaces(); on a stream that is
@@ -335,7 +337,9 @@ int mxfp6_probe_raster(int group_m, int xcd_remap);
  * row-major A stay with the skinny kernel, except 33 - 64 rows against tile-major weights with K >= 24576 or N above 8192
  * and no multiple of it), 1 = never,
  * -1 = wherever the shape allows it, n > 1 = n workgroups per output tile where the shape allows it (K a multiple of 512 n,
- * at least 8 K-tiles of 128 per share, at most half as many output tiles as CUs), else unsplit.
+ * at least 8 K-tiles of 128 per share, at most half as many output tiles as CUs), else unsplit.  The block kernel's own
+ * rule (its 128 x 128 tiles on at most half the CUs, K >= 8192, or >= 5120 with both operands tile-major; asked before the
+ * tiled kernel's) is described with mxfp6_set_kernel 22 and reported by mxfp6_probe_choice (code 27).
  * No counterpart in the reference (its GEMMs are one workgroup per 256 x 256 tile, analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61).
  */
 int mxfp6_probe_ksplit(int shares);
