@@ -336,6 +336,50 @@ def test_forced_kernels_reject_shapes_they_cannot_take(hk):
     check(gemm(hk, ap, bp, asc, bsc, kernel=0), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64), 2, 2)  # automatic: generic
 
 
+# ------------------------------------------------------------------ automatic path over random shapes
+def test_automatic_path_random_shapes_against_the_generic_kernel(hk):
+    """Sixty seeded random shapes and layout pairs through the automatic choice, each against the generic kernel (which the
+    oracle tests pin) on the same bytes: whatever kernel, tile shape, ring depth or K split the rules pick, the fp32 result
+    agrees to the rounding of the sums.  The draw covers every kernel the choice can make."""
+    tk = hk.tk_kernel
+    rng = np.random.default_rng(2024)
+    seen = set()
+    for case in range(60):
+        kind = case % 6
+        if kind == 0:      # few rows, long K
+            M, N, K = int(rng.integers(1, 65)), int(rng.integers(1, 65)) * 128, int(rng.integers(4, 57)) * 512
+        elif kind == 1:    # a few hundred rows, K of moderate length
+            M, N, K = int(rng.integers(65, 769)), int(rng.integers(8, 65)) * 128, int(rng.integers(2, 17)) * 512
+        elif kind == 2:    # a few hundred rows, long K, narrow N
+            M, N, K = int(rng.integers(33, 513)), int(rng.integers(1, 33)) * 128, int(rng.integers(16, 57)) * 512
+        elif kind == 3:    # ragged everything (N % 8 == 0, K % 128 == 0)
+            M, N, K = int(rng.integers(1, 700)), int(rng.integers(1, 300)) * 8, int(rng.integers(1, 40)) * 128
+        elif kind == 4:    # many tiles
+            M, N, K = int(rng.integers(4, 17)) * 128, int(rng.integers(16, 33)) * 128, int(rng.integers(1, 9)) * 512
+        else:              # K % 32 only: the generic kernel's own
+            M, N, K = int(rng.integers(1, 200)), int(rng.integers(1, 200)), int(rng.integers(1, 30)) * 32
+        la = int(rng.integers(0, 2)) if M % 32 == 0 and K % 128 == 0 else 0
+        lb = int(rng.integers(0, 2)) if N % 32 == 0 and K % 128 == 0 else 0
+        seen.add(tk.kernel_choice(M, N, K, la, lb))
+        g = torch.Generator(device="cuda"); g.manual_seed(case)
+        a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2, la)
+        b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.05, 3 if case % 5 == 0 else 2, lb)
+        fb = 3 if case % 5 == 0 else 2
+        ref = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ar, asr = (hk.tile_operand(a, untile=True), hk.tile_scales(asc, K, untile=True)) if la else (a, asc)
+        br, bsr = (hk.tile_operand(b, untile=True), hk.tile_scales(bsc, K, untile=True)) if lb else (b, bsc)
+        prev = tk.set_kernel(1)
+        try:
+            hk.dispatch_micro(ar, br, asr, bsr, ref, 2, fb)
+        finally:
+            tk.set_kernel(prev)
+        hk.dispatch_micro(a, b, asc, bsc, got, 2, fb, layout_a=la, layout_b=lb)
+        torch.cuda.synchronize()
+        assert o.rel_err(got.cpu().numpy(), ref.cpu().numpy()) <= TOL_TIGHT, (case, M, N, K, la, lb)
+    assert {tk.KERNEL_GENERIC, tk.KERNEL_TILED, tk.KERNEL_SKINNY, tk.KERNEL_BLOCK, tk.CHOICE_BLOCK_K_SPLIT} <= seen, seen
+
+
 # ------------------------------------------------------------------ skinny kernel
 @pytest.mark.parametrize("M,N,K", [(16, 64, 512), (1, 32, 1024), (7, 100, 2048), (16, 512, 3584), (32, 96, 1536), (13, 33, 512 * 9), (17, 31, 512 * 13), (16, 1000, 512 * 20),
                                    (33, 40, 1024), (64, 96, 512 * 5), (48, 1000, 2048), (50, 31, 512 * 11),    # 33 - 64 rows of A: two accumulator tiles
