@@ -12,7 +12,7 @@
 //
 // Same operand formats, LDS image, lane mapping and raster as the tiled kernel (common.hpp, gemm_tiled.hip): row-major
 // or tile-major operands and scales, any M and N (edge tiles: rows past M or N lie beyond the end of their buffer
-// resource and read as zeros, stores are predicated), K % 512 == 0, bf16 or fp32 output, fused scales / bias / activation
+// resource and read as zeros, stores are predicated), K % 128 == 0, bf16 or fp32 output, fused scales / bias / activation
 // (separate instantiations).
 //   ring: three slots of 24 KB (A's 128 rows x 96 bytes, then B's); K-tile k lives in slot k % 3
 //   scales: the 16 bytes a row has for four K-tiles, two buffers of (128 + 128) rows x 16 bytes, group g in buffer g % 2
@@ -73,11 +73,11 @@ __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_bl
   __shared__ __attribute__((aligned(1024))) uint8_t smem[kLdsBytes];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
   const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
-  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt_all = K / kBK, nk4_all = nkt_all / 4;
+  const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt_all = K / kBK, nk4_all = (nkt_all + 3) / 4;  // tile-major scales: one 512-byte chunk per 32 rows and group of four K-tiles, the last one padded
   // K split: workgroup b takes share b / tiles of tile b % tiles, K-tiles [share, share + 1) * nkt, and leaves its fp32
   // sums in matrix `share` of args.C, then a workspace of nsplit matrices [M, N] (ksplit_reduce_kernel adds them up)
   const int ntiles = args.tiles_m * args.tiles_n, share = blockIdx.x / ntiles;
-  const int nkt = nkt_all / args.nsplit, nk4 = nkt / 4, kt0 = share * nkt;
+  const int nkt = nkt_all / args.nsplit, nk4 = (nkt + 3) / 4, kt0 = share * nkt;  // (a split leaves every share whole groups)
 
   const int tile = tile_order(blockIdx.x - share * ntiles, args.tiles_m, args.tiles_n, args.group_m, args.xcd_remap);
   if (tile < 0) return;  // never: the grid is the tile count times the shares
@@ -163,9 +163,11 @@ __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_bl
 #pragma unroll
     for (int n = 0; n < 6; n++) load_one.template operator()<LA>(t, slot, n);
   };
+  // (the group's offset goes into the per-lane offset, which the hardware checks against the end of the resource: with
+  // K % 512 != 0 the last group of a row-major row is shorter than 16 bytes, and the last row's must not read past the tensor)
   auto load_scales = [&](int grp) __attribute__((always_inline)) {
     const __amdgpu_buffer_rsrc_t rs = grp < nk4 ? rS : rZ;
-    dma16(rs, sdst + (grp & 1) * kScBuf, voff_s, grp * sstep);
+    dma16(rs, sdst + (grp & 1) * kScBuf, voff_s + grp * sstep, 0);
   };
   auto read_tile = [&]<int SET>(int slot) __attribute__((always_inline)) {
     const uint8_t* st = smem + slot * kSlot;
@@ -280,12 +282,17 @@ __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_bl
     take_scales();
     wait_vmcnt<NL * (STAGES - 2)>();
     barrier();  // K-tile 1 is in place, and every wave has K-tile 0 in registers: its slot is free
-    for (int k = 0; k < nkt; k += 4) {
+    int k = 0;
+    for (; k + 4 <= nkt; k += 4) {
       step.template operator()<0, LA>(k);
       step.template operator()<1, LA>(k + 1);
       step.template operator()<2, LA>(k + 2);
       step.template operator()<3, LA>(k + 3);
     }
+    // a last group of fewer than four K-tiles (K % 512 != 0): the same steps; their loads lie past the end and fetch nothing
+    if (k < nkt) step.template operator()<0, LA>(k);
+    if (k + 1 < nkt) step.template operator()<1, LA>(k + 1);
+    if (k + 2 < nkt) step.template operator()<2, LA>(k + 2);
   };
   if constexpr (WN == 2) {
     run.template operator()<true>();
@@ -434,9 +441,9 @@ hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, 
 }  // namespace
 
 bool gemm_block_supports(const GemmArgs& g) {
-  // N % 8 keeps every run of 8 bf16 outputs whole and aligned; K in whole groups of four K-tiles; 32-bit byte offsets
+  // N % 8 keeps every run of 8 bf16 outputs whole and aligned; K in whole K-tiles; 32-bit byte offsets
   // inside one tile's operand rows and inside one tile's rows of C
-  return g.M > 0 && g.N > 0 && g.K >= 512 && g.N % 8 == 0 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) &&
+  return g.M > 0 && g.N > 0 && g.K >= 128 && g.N % 8 == 0 && g.K % 128 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) &&
          (long)128 * g.N * 4 < (1L << 31) && (long)((g.M + 127) / 128) <= 65535 && (long)((g.N + 127) / 128) <= 32767 &&
          (long)((g.M + 127) / 128) * ((g.N + 127) / 128) < (1L << 31) && ((uintptr_t)g.C % 16) == 0 && operands_aligned16(g) && !g.fmt_c &&
          !g.no_alloc;
@@ -508,7 +515,7 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   const int cus = cu_count_of_device();
   const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
   const int nkt = g.K / kBK, groups = nkt / 4;
-  if (cus < 8 || tiles * 2 > cus) return 1;
+  if (cus < 8 || tiles * 2 > cus || nkt % 4 != 0) return 1;  // shares are whole groups of four K-tiles
   if (want == 0) {
     if (nkt < 64 && !(g.layout_a && g.layout_b && nkt >= 40)) return 1;  // two launches for a K this short lose (96 x 8192 x 2048: 11 -> 14 us)
     const bool both = g.layout_a && g.layout_b;

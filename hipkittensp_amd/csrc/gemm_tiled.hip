@@ -294,7 +294,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     }
     const int buf = (p0 + grp) & 1;
     const uint32_t dst = lds0 + kScaleBase + buf * kScaleBuf + swave * 1024;
-    dma16(rS, sc_a ? dst : dst + kScStage, voff_s, (INSIDE || grp < nk4 ? grp : grp - nk4) * sstep);
+    // the group's offset rides in the per-lane offset, which the hardware checks against the end of the resource (the
+    // scalar offset it does not): with K % 512 != 0 the last group of a row-major row is shorter than 16 bytes, and the
+    // last row's load must not read past the tensor
+    dma16(rS, sc_a ? dst : dst + kScStage, voff_s + (INSIDE || grp < nk4 ? grp : grp - nk4) * sstep, 0);
   };
   auto issue_one = [&]<bool INSIDE, int GRP>(int kk, int slot, int n) __attribute__((always_inline)) {
     constexpr int OPAg = GRP == 0 ? OPA : OPA1;

@@ -125,8 +125,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled4_kernel(const uint8_t* __r
 
   auto issue_scales = [&](int grp) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + kScaleBase + (grp & 1) * kScaleBuf + wave * 1024;
-    dma16(rSA, dst, voff_sa, grp * sstep_a);
-    dma16(rSB, dst + kScStage, voff_sb, grp * sstep_b);
+    // (the group's offset in the per-lane offset: that is the one the hardware checks against the end of the resource)
+    dma16(rSA, dst, voff_sa + grp * sstep_a, 0);
+    dma16(rSB, dst + kScStage, voff_sb + grp * sstep_b, 0);
   };
   auto issue_one = [&](int t, int slot, int n) __attribute__((always_inline)) {
     const uint32_t dst = lds0 + slot * kStage + wave * (OPS * 1024);

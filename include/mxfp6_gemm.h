@@ -119,7 +119,7 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *   18  the 4-wave interleaved schedule of the LDS-tiled kernel (one wave per SIMD with a 128 x 128 wave tile; shapes
  *       of kernel 2, no fused epilogue); never chosen automatically, kept to compare the two schedules
  *   22  block kernel: output tiles of 128 x 128, four waves in step with the operand fragments double-buffered in
- *       registers, one barrier per K-tile (needs N % 8 == 0, K % 512 == 0); chosen automatically where
+ *       registers, one barrier per K-tile (needs N % 8 == 0, K % 128 == 0); chosen automatically where
  *       its tiles do not outnumber the CUs and K is of moderate length (a few hundred rows of A);
  *       23 / 24: with an operand ring of three slots (two workgroups per CU) / six slots (one); 26: with tiles of
  *       128 x 256 and eight waves.  22 - 24 split K between workgroups by the thread's mxfp6_probe_ksplit setting

@@ -143,7 +143,7 @@ def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
 
 # ------------------------------------------------------------------ block kernel (128 x 128 tiles, four waves in step)
 @pytest.mark.parametrize("M,N,K", [(128, 128, 512), (256, 384, 1024), (512, 256, 2560), (300, 264, 1536), (129, 8, 512), (100, 1000, 1024), (33, 520, 2048),
-                                   (1, 128, 512), (640, 1024, 4096)])  # edge tiles too; K in whole groups of four K-tiles
+                                   (1, 128, 512), (640, 1024, 4096), (256, 256, 128), (300, 264, 640), (100, 520, 1152), (257, 8, 384)])  # edge tiles too; K % 512 != 0: a last group of fewer than four K-tiles
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
 @pytest.mark.parametrize("kernel", [23, 24, 26])  # ring of three slots (two workgroups per CU), of six (one); tiles of 128 x 256
 def test_block_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
@@ -242,7 +242,7 @@ def test_kernel_choice_by_shape(hk):
     assert tk.kernel_choice(256, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(512, 4096, 4096, 0, 1) == tk.KERNEL_BLOCK
     assert tk.kernel_choice(2048, 8192, 8192, 1, 1) == tk.KERNEL_TILED      # more 128 x 256 tiles than CUs
     assert tk.kernel_choice(1024, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK_WIDE and tk.kernel_choice(1024, 8192, 8192, 0, 1) == tk.KERNEL_TILED
-    assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_TILED  # K % 512
+    assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_BLOCK  # K % 512 != 0 is fine
     assert tk.kernel_choice(40, 36, 96) == tk.KERNEL_GENERIC
     prev = tk.set_k_split(1)
     try:
@@ -252,7 +252,7 @@ def test_kernel_choice_by_shape(hk):
 
 
 def test_block_kernel_rejects_what_it_cannot_take(hk):
-    ap, asc, bp, bsc = operands(128, 128, 384, 2, 2, seed=1)      # K % 512
+    ap, asc, bp, bsc = operands(128, 128, 96, 2, 2, seed=1)       # K % 128
     with pytest.raises(RuntimeError, match="bad shape"):
         gemm(hk, ap, bp, asc, bsc, kernel=22)
     ap, asc, bp, bsc = operands(128, 36, 512, 2, 2, seed=1)       # N % 8
