@@ -36,10 +36,10 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 PUBLISHED_FP6_8192 = 2861.52  # reference's published FP6 GEMM at 8192^3 on MI355X (analysis/fp6_gemm/mi355x_fp6_gemm.json:5)
 # Fabric bytes per launch (L2 fills + write-backs) from rocprofv3 FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the
 # factors calibrated on an elementwise kernel of known size in the same runs
-# (profiles/bench_gemm_tiled_8192_gemm_skinny_m16.md, taken on the current kernels): tiled 8192^3 = 614 900 + 131 082 KiB,
+# (profiles/bench_gemm_tiled_8192_gemm_skinny_m16.md, taken on the current kernels): tiled 8192^3 = 614 890 + 131 076 KiB,
 # skinny cfg3 = 187 110 + 256 KiB.  Both kernels move the same bytes on every launch of a shape (the counters repeat to four
 # digits over hundreds of launches), so the figure does not depend on the run.
-TILED_TRAFFIC_BYTES = (614900 + 131082) * 1024
+TILED_TRAFFIC_BYTES = (614890 + 131076) * 1024
 SKINNY_TRAFFIC_BYTES = (187110 + 256) * 1024
 
 
