@@ -34,6 +34,8 @@ sys.path.insert(0, ROOT)
 MFMA_PEAK_TFLOPS = 10066.0  # MI355X dense MXFP6: 256 CU x 4 SIMD x 4096 FLOP/clk x 2.4 GHz
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 PUBLISHED_FP6_8192 = 2861.52  # reference's published FP6 GEMM at 8192^3 on MI355X (analysis/fp6_gemm/mi355x_fp6_gemm.json:5)
+# the other square sizes of the same published table (analysis/fp6_gemm/mi355x_fp6_gemm.json:2-6), TFLOPS
+PUBLISHED_FP6_SQUARES = {1024: 74.9089, 2048: 470.161, 4096: 1865.47, 16384: 3122.13}
 # Fabric bytes per launch (L2 fills + write-backs) from rocprofv3 FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, the
 # factors calibrated on an elementwise kernel of known size in the same runs
 # (profiles/bench_gemm_tiled_8192_gemm_skinny_m16.md, taken on the current kernels): tiled 8192^3 = 614 890 + 131 076 KiB,
@@ -250,6 +252,32 @@ def cpu_baseline(inputs, M_sample, gpu_f32):
         "kind": "port",
         "sample": f"first {M_sample} of 8192 rows of A against all 8192 rows of B, K=8192, one pass (dequantise + fp32 matmul, {dt:.2f} s)",
     }
+
+
+def square_sizes(hk, torch, steps, warmup):
+    """The other square sizes of the reference's published FP6 table: the operator from row-major inputs (whatever the
+    library chooses, pre-pass included where it makes one) and on tile-major operands, back-to-back launches over
+    three input sets (two at 16384); TFLOPS and the ratio to the published figure."""
+    out = {"what": "M=N=K, e2m3 x e2m3, bf16 out: the operator on row-major inputs / on tile-major operands and scales; TFLOPS, and "
+                   "over the reference's published MI355X FP6 figure for the size (analysis/fp6_gemm/mi355x_fp6_gemm.json)"}
+    for S, ref in PUBLISHED_FP6_SQUARES.items():
+        ins = make_inputs(hk, torch, S, S, S, 2, 2, seed=10 + S // 1024, sets=2 if S > 8192 else 3)
+        C = torch.empty(S, S, dtype=torch.bfloat16, device="cuda")
+        pre = PREWARM_MS if S >= 4096 else 0.0
+        _, row_ms = timed_loop(hk, torch, ins, C, steps, warmup, 0, 0, prewarm_ms=pre)
+        tin = [(hk.tile_operand(ap), hk.tile_operand(bp), hk.tile_scales(asc, S), hk.tile_scales(bsc, S)) for ap, bp, asc, bsc in ins]
+        del ins
+        _, tile_ms = timed_loop(hk, torch, tin, C, steps, warmup, 1, 1, prewarm_ms=pre)
+        flops = 2.0 * S ** 3
+        out[str(S)] = {
+            "row_major_ms": row_ms, "row_major_tflops": flops / (row_ms * 1e-3) / 1e12, "row_major_vs_published": flops / (row_ms * 1e-3) / 1e12 / ref,
+            "tile_major_ms": tile_ms, "tile_major_tflops": flops / (tile_ms * 1e-3) / 1e12, "tile_major_vs_published": flops / (tile_ms * 1e-3) / 1e12 / ref,
+            "kernel_choice_row_major": hk.tk_kernel.kernel_choice(S, S, S, 0, 0), "kernel_choice_tile_major": hk.tk_kernel.kernel_choice(S, S, S, 1, 1),
+            "published_tflops": ref,
+        }
+        del tin, C
+        torch.cuda.empty_cache()
+    return out
 
 
 def dispatch_sweep(hk, torch, full):
@@ -506,8 +534,10 @@ def main():
             "launch_ms_mean": dtev_ms,
         }
     # ---- the quantiser (the step in front of the GEMM at inference time): 8192 x 8192 activations -> packed fp6 + E8M0,
-    # fp32 and bf16 sources, into preallocated outputs through the C ABI (no allocation inside the timed region)
     del dinputs
+    torch.cuda.empty_cache()
+    squares = square_sizes(hk, torch, args.steps, args.warmup) if args.layouts == "both" else None
+    # fp32 and bf16 sources, into preallocated outputs through the C ABI (no allocation inside the timed region)
     torch.cuda.empty_cache()
     from hipkittensp_amd import _lib
     L = _lib.lib()
@@ -585,6 +615,7 @@ def main():
         "cpu_baseline": cpu,
         "decode": decode,
         "quantize": quant,
+        "squares": squares,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(line))
