@@ -116,9 +116,63 @@ ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU = 0, 1, 2, 3
 _ACTS = {None: 0, "none": 0, "relu": 1, "gelu": 2, "silu": 3, 0: 0, 1: 1, 2: 2, 3: 3}
 
 
+_torch = None
+_fast = None  # (Tensor type, uint8, bfloat16, float32, raw-stream getter, current_device, the library's mxfp6_gemm_fused)
+
+
+def _fast_state():
+    global _torch, _fast
+    import torch
+
+    _torch = torch
+    get_raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if get_raw is None:
+        get_raw = lambda index: torch.cuda.current_stream(index).cuda_stream
+    _fast = (torch.Tensor, torch.uint8, torch.bfloat16, torch.float32, get_raw, torch.cuda.current_device, _lib.lib().mxfp6_gemm_fused)
+    return _fast
+
+
 def dispatch_micro(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, layout_a: int = LAYOUT_ROW,
                    layout_b: int = LAYOUT_ROW, bias=None, row_scale=None, col_scale=None, activation=None, C_scale=None,
                    fmt_c: int = E2M3) -> None:
+    """C = dq(A) @ dq(B).T (the full description is _dispatch_micro_checked's, which this is a short cut in front of).
+
+    The usual call -- five contiguous 2-D torch tensors of the right dtypes and shapes on the current GPU, no fused
+    epilogue -- is recognised here with one read of each tensor's metadata and goes straight to the library (a few
+    microseconds of host time, which is what a small GEMM's launch rate is bound by); everything else, including every
+    call that is wrong in some way, takes the checked path below, which handles the general cases and raises the
+    reference binding's errors."""
+    f = _fast or _fast_state()
+    T, u8 = f[0], f[1]
+    if (bias is None and row_scale is None and col_scale is None and activation is None and C_scale is None
+            and type(A) is T and type(B) is T and type(A_scale) is T and type(B_scale) is T and type(C) is T
+            and A.dtype is u8 and B.dtype is u8 and A_scale.dtype is u8 and B_scale.dtype is u8):
+        cd = C.dtype
+        sa, sb, sas, sbs, sc = A.shape, B.shape, A_scale.shape, B_scale.shape, C.shape
+        dev = C.get_device()
+        if ((cd is f[2] or cd is f[3]) and len(sa) == 2 and len(sb) == 2 and len(sas) == 2 and len(sbs) == 2 and len(sc) == 2
+                and dev >= 0 and dev == f[5]() and A.get_device() == dev and B.get_device() == dev
+                and A_scale.get_device() == dev and B_scale.get_device() == dev
+                and A.is_contiguous() and B.is_contiguous() and A_scale.is_contiguous() and B_scale.is_contiguous() and C.is_contiguous()
+                and (fmt_a == 2 or fmt_a == 3) and (fmt_b == 2 or fmt_b == 3) and (layout_a == 0 or layout_a == 1) and (layout_b == 0 or layout_b == 1)):
+            M, wa = sa
+            N = sb[0]
+            K = wa // 3 * 4
+            if (wa == sb[1] and wa % 24 == 0 and sc[0] == M and sc[1] == N and sas[0] == M and sbs[0] == N
+                    and sas[1] == (K // 32 if layout_a == 0 else (K + 511) // 512 * 16)
+                    and sbs[1] == (K // 32 if layout_b == 0 else (K + 511) // 512 * 16)
+                    and (layout_a == 0 or (M % 32 == 0 and K % 128 == 0)) and (layout_b == 0 or (N % 32 == 0 and K % 128 == 0))):
+                rc = f[6](A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C.data_ptr(), M, N, K,
+                          fmt_a, fmt_b, layout_a, layout_b, 1 if cd is f[3] else 0, 0, 0, 0, 0, 0, f[4](dev))
+                if rc:
+                    _lib.check(rc, "dispatch_micro")
+                return
+    _dispatch_micro_checked(A, B, A_scale, B_scale, C, fmt_a, fmt_b, layout_a, layout_b, bias, row_scale, col_scale, activation, C_scale, fmt_c)
+
+
+def _dispatch_micro_checked(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, layout_a: int = LAYOUT_ROW,
+                            layout_b: int = LAYOUT_ROW, bias=None, row_scale=None, col_scale=None, activation=None, C_scale=None,
+                            fmt_c: int = E2M3) -> None:
     """C = dq(A) @ dq(B).T; optionally fused, in fp32 before the output rounding:
     C = act(acc * row_scale[:, None] * col_scale[None, :] + bias[None, :]) with bias [N] float32 or bfloat16,
     row_scale [M] and col_scale [N] float32, activation one of None / "relu" / "gelu" / "silu".

@@ -965,6 +965,36 @@ def test_leading_dimensions_fold_into_rows(hk):
     assert o.rel_err(C.view(64, 32).cpu().numpy(), o.gemm_ref(ap, bp, asc, bsc, acc=np.float64)) <= TOL
 
 
+def test_short_cut_in_front_of_the_checked_path(hk):
+    """dispatch_micro recognises the plain call (2-D contiguous tensors on the current device, no epilogue) and skips
+    the per-argument checks: same bytes as the checked path on both layouts and both output types, and every call the
+    short cut does not recognise still arrives at the checked path's errors."""
+    tk = hk.tk_kernel
+    ap, asc, bp, bsc = operands(96, 160, 1024, 3, 2, seed=77)
+    A, B, As, Bs = dev(ap), dev(bp), dev(asc), dev(bsc)
+    At, Bt, Ast, Bst = tk.tile_operand(A), tk.tile_operand(B), tk.tile_scales(As, 1024), tk.tile_scales(Bs, 1024)
+    for dt in (torch.float32, torch.bfloat16):
+        for args, la, lb in (((A, B, As, Bs), 0, 0), ((At, Bt, Ast, Bst), 1, 1), ((A, Bt, As, Bst), 0, 1)):
+            C0 = torch.full((96, 160), float("nan"), dtype=dt, device="cuda")
+            C1 = torch.full((96, 160), float("nan"), dtype=dt, device="cuda")
+            hk.dispatch_micro(*args, C0, 3, 2, la, lb)
+            tk._dispatch_micro_checked(*args, C1, 3, 2, la, lb)
+            torch.cuda.synchronize()
+            assert torch.equal(C0, C1) and bool(torch.isfinite(C0.float()).all())
+    C = torch.empty(96, 160, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="A_scale"):
+        hk.dispatch_micro(A, B, As[:, :16].contiguous(), Bs, C, 3, 2)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hk.dispatch_micro(A, B, As, Bs, torch.empty(160, 96, dtype=torch.bfloat16, device="cuda").t(), 3, 2)
+    with pytest.raises(RuntimeError, match="tile-major operand needs"):
+        hk.dispatch_micro(A[:40].contiguous(), Bt, As[:40].contiguous(), Bst, C[:40].contiguous(), 3, 2, 1, 1)
+    with pytest.raises(RuntimeError, match="layout_a / layout_b"):
+        hk.dispatch_micro(A, B, As, Bs, C, 3, 2, 2, 0)
+    with pytest.raises(RuntimeError, match="C: expected dtype"):
+        hk.dispatch_micro(A, B, As, Bs, C.to(torch.float16), 3, 2)
+    torch.cuda.synchronize()
+
+
 # ------------------------------------------------------------------ quantiser: bit exact
 @pytest.mark.parametrize("fmt", [2, 3])
 @pytest.mark.parametrize("kind", ["normal", "weights", "weights_outliers", "laplace"])
