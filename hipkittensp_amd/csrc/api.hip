@@ -640,7 +640,7 @@ const char* mxfp6_strerror(int code) {
   return "mxfp6: unknown error code";
 }
 
-int mxfp6_abi_version(void) { return 119; }
+int mxfp6_abi_version(void) { return MXFP6_ABI_VERSION; }
 
 #pragma GCC visibility pop
 }  // extern "C"

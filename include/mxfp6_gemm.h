@@ -363,7 +363,9 @@ int mxfp6_probe_choice(int M, int N, int K, int layouts);
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);
 
-/* ABI version of this header: major * 100 + minor. */
+/* ABI version of this header, major * 100 + minor, and what the loaded library reports: a caller built against this
+ * header checks that the majors agree (entry points are only ever added within a major). */
+#define MXFP6_ABI_VERSION 119
 int mxfp6_abi_version(void);
 
 #ifdef __cplusplus
