@@ -365,8 +365,9 @@ def set_kernel(which: int) -> int:
 
 def dispatch_micro_noalloc(A, B, A_scale, B_scale, C, fmt_a: int = E2M3, fmt_b: int = E2M3, nsplit: int = 0) -> None:
     """dispatch_micro for callers that cannot allocate device memory (graph capture, tight serving loops): row-major
-    operands, bfloat16 C, no allocation of any kind behind the call.  nsplit = 0 picks kernel and K split like
-    dispatch_micro (bit-identical result); 1, 2, 4 or 8 fixes the K split of the skinny kernel (M <= 32, K % 512 == 0),
+    operands, bfloat16 C, no allocation of any kind behind the call.  nsplit = 0 picks the kernel dispatch_micro would
+    pick among those that need no workspace (bit-identical result on the decode shapes the skinny kernel takes; elsewhere
+    the same products, possibly added in another order); 1, 2, 4 or 8 fixes the K split of the skinny kernel (M <= 32, K % 512 == 0),
     whose partial tiles live in the library's static scratch memory (256 partial tiles: a RuntimeError says so when a
     split does not fit)."""
     import torch

@@ -269,8 +269,14 @@ int mxfp6_release_workspaces(void);
  * counterpart in the reference.  The re-layout pre-pass is left out, and the K split of decode shapes keeps its partial
  * tiles (4 KB per tile of C and split) and arrival counters in a static array of the library's device code: 1 MB + 1 KB
  * per GPU, held until the process ends, holding 256 partial tiles and 256 counters.
- *   nsplit = 0: kernel and split chosen as mxfp6_gemm chooses them (never more than 256 partial tiles) -- the result is
- *               bit-identical to mxfp6_gemm's;
+ *   nsplit = 0: the kernel mxfp6_gemm would choose among those that need no workspace (the skinny, mid-M, tiled and
+ *               generic kernels; the skinny kernel's K split as mxfp6_gemm chooses it, never more than 256 partial
+ *               tiles).  Where that is mxfp6_gemm's own choice -- the decode shapes it gives to the skinny kernel --
+ *               the result is bit-identical to mxfp6_gemm's, and so it is where mxfp6_gemm takes the pre-pass or
+ *               the block kernel unsplit (the sum along K runs in the same order); where mxfp6_gemm takes a K split
+ *               of the tiled or block kernel, or a kernel of another family for the shape, the same products are
+ *               added in another order: equal within the rounding of fp32 partial sums, and bit-identical whenever
+ *               those sums are exact;
  *   nsplit = 1, 2, 4, 8: the skinny kernel with K split between that many workgroups per tile of C (needs M <= 32,
  *               K % 512 == 0; MXFP6_EINVAL_SHAPE otherwise).  A tile of C is 16 columns for N <= 4096 and 32 beyond:
  *               ceil(N / 16 or 32) * nsplit must not exceed 256, else MXFP6_ESCRATCH and nothing is launched.
