@@ -498,8 +498,8 @@ bool gemm_block_wide_preferred(const GemmArgs& g) {
 
 // K split of this kernel's 128 x 128 tiles: shares per output tile (1 = none) and the workspace they need.
 // want: 0 = where it pays (below), 1 = never, -1 = wherever the shape allows it, n > 1 = n shares if the shape allows it.
-// A share gets a whole number of groups of four K-tiles and at least 16 K-tiles (8 where that would leave most CUs
-// idle); the shares of all tiles together do not outnumber the CUs.  Where it pays (sweep of 48 - 512 rows x nine (N, K) pairs x three layout pairs on MI355X, us, the
+// A share gets a whole number of groups of four K-tiles and at least 16 K-tiles (8 where no such split exists, and for
+// K = 8192 with few tiles); the shares of all tiles together do not outnumber the CUs.  Where it pays (sweep of 48 - 512 rows x nine (N, K) pairs x three layout pairs on MI355X, us, the
 // choice before -> this, each timed twice in alternation): K from 8192 on (5120 with both operands tile-major; shorter,
 // two launches lose), at most half as many tiles as CUs, more than three eighths of them only for K = 14336 .. 16384
 // (with K = 8192 an unsplit launch of that many tiles is as fast, with K = 28672 the tiled kernel's split is:
@@ -531,11 +531,16 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
     // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
     if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)))) return 1;
   }
-  // the most shares that leave each at least 16 K-tiles; if those are fewer workgroups than three eighths of the CUs, at
-  // least 8 K-tiles (64 x 1024 x 16384: 16 shares of 8 K-tiles 14.9 us, unsplit 20.4; 256 x 2048 x 8192: 4 shares of 16
-  // K-tiles 16.7, 8 of 8 18.2)
+  // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with 4 - 32 tiles a share
+  // of 16 K-tiles beats both shorter shares and every other kernel (us, 64 - 256 rows, what was chosen before -> this;
+  // each side timed twice in alternation): 128 x 512 x 16384 19.7 -> 15.7 (8 shares on 4 tiles = 32 workgroups),
+  // 64 x 512 x 28672 20.9 -> 15.3 (14 shares), 64 x 1024 x 28672 both row-major 30.0 -> 17.0, 128 x 1024 x 16384
+  // 18.1 -> 17.1 (8 shares instead of 16), 128 x 1024 x 14336 17.3 -> 16.4 (7 instead of 14).  K = 8192 with up to
+  // 12 tiles: shares of 8 K-tiles (128 x 512 x 8192: 8 shares 12.3, 4 shares 12.9, tiled kernel's split 16.8, skinny
+  // kernel 19.3; with 16 tiles and more 4 shares are level or ahead: 256 x 2048 x 8192 16.7 against 18.2).  With fewer
+  // than four tiles (not measured) as before: no split unless its workgroups are three eighths of the CUs or more.
   int best = 1;
-  for (int min_tiles = 16; min_tiles >= 8 && best <= 1; min_tiles -= 8) {
+  for (int min_tiles = want == 0 && nkt == 64 && tiles >= 4 && tiles <= 12 ? 8 : 16; min_tiles >= 8 && best <= 1; min_tiles -= 8) {
     for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
       if (groups % sh == 0 && nkt / sh >= min_tiles && tiles * sh <= cus) {
         best = sh;
@@ -543,12 +548,13 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
       }
       if (want > 1) break;
     }
-    if (want == 0 && best > 1 && tiles * best * 8 < (long)cus * 3) best = 1;  // too few workgroups: try shorter shares
+    if (want == 0 && best > 1 && tiles < 4 && tiles * best * 8 < (long)cus * 3) best = 1;  // too few workgroups: try shorter shares
   }
   if (best <= 1) return 1;
-  // K beyond 16384 and shares on fewer than three quarters of the CUs: the tiled kernel's split streams B faster
-  // (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7)
-  if (want == 0 && nkt > 128 && tiles * best * 4 < (long)cus * 3) return 1;
+  // K beyond 16384, more than 16 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
+  // streams B faster (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7; up
+  // to 16 tiles this kernel's: 128 x 2048 x 28672 23.4 against 26.0)
+  if (want == 0 && nkt > 128 && tiles > 16 && tiles * best * 4 < (long)cus * 3) return 1;
   *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
   return best;
 }

@@ -186,7 +186,8 @@ def test_block_kernel_is_chosen_and_matches_the_tiled_kernel(hk, M, N, K, la, lb
     check(outs[22][rows], o.gemm_ref(ap[rows], bp, asc[rows], bsc, acc=np.float64), 2, 2)
 
 
-@pytest.mark.parametrize("M,N,K,shares", [(128, 256, 4096, 2), (128, 512, 8192, 4), (100, 264, 4096, 2), (256, 512, 8192, 8), (64, 1024, 16384, 0), (192, 2048, 8192, 0)])
+@pytest.mark.parametrize("M,N,K,shares", [(128, 256, 4096, 2), (128, 512, 8192, 4), (100, 264, 4096, 2), (256, 512, 8192, 8), (64, 1024, 16384, 0), (192, 2048, 8192, 0),
+                                          (128, 512, 8192, 0), (96, 520, 28672, 0)])
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
 def test_block_kernel_k_split(hk, M, N, K, shares, fa, fb):
     """The block kernel with the K range of every output tile split between several workgroups: fp32 partial matrices in
@@ -244,6 +245,10 @@ def test_kernel_choice_by_shape(hk):
     assert tk.kernel_choice(1024, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK_WIDE and tk.kernel_choice(1024, 8192, 8192, 0, 1) == tk.KERNEL_TILED
     assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_BLOCK  # K % 512 != 0 is fine
     assert tk.kernel_choice(40, 36, 96) == tk.KERNEL_GENERIC
+    # few output tiles and a long K: this kernel's split however few workgroups it makes (4 tiles x 8 shares here), for every layout pair
+    for la, lb in ((0, 0), (0, 1), (1, 1)):
+        assert tk.kernel_choice(128, 512, 16384, la, lb) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 1024, 8192, la, lb) == tk.CHOICE_BLOCK_K_SPLIT
+    assert tk.kernel_choice(64, 1024, 28672) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 1024, 8192) == tk.KERNEL_SKINNY   # the skinny kernel's up to 64 rows at K = 8192
     prev = tk.set_k_split(1)
     try:
         assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY   # no split
