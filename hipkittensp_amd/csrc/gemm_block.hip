@@ -531,16 +531,20 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
     // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
     if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)))) return 1;
   }
-  // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with 4 - 32 tiles a share
-  // of 16 K-tiles beats both shorter shares and every other kernel (us, 64 - 256 rows, what was chosen before -> this;
-  // each side timed twice in alternation): 128 x 512 x 16384 19.7 -> 15.7 (8 shares on 4 tiles = 32 workgroups),
-  // 64 x 512 x 28672 20.9 -> 15.3 (14 shares), 64 x 1024 x 28672 both row-major 30.0 -> 17.0, 128 x 1024 x 16384
-  // 18.1 -> 17.1 (8 shares instead of 16), 128 x 1024 x 14336 17.3 -> 16.4 (7 instead of 14).  K = 8192 with up to
-  // 12 tiles: shares of 8 K-tiles (128 x 512 x 8192: 8 shares 12.3, 4 shares 12.9, tiled kernel's split 16.8, skinny
-  // kernel 19.3; with 16 tiles and more 4 shares are level or ahead: 256 x 2048 x 8192 16.7 against 18.2).  With fewer
-  // than four tiles (not measured) as before: no split unless its workgroups are three eighths of the CUs or more.
+  // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with up to 32 tiles such a
+  // split beats shorter shares and every other kernel (us, 64 - 256 rows, what was chosen before -> this; each side
+  // timed twice in alternation): 128 x 512 x 16384 19.7 -> 15.7 (8 shares on 4 tiles = 32 workgroups), 64 x 512 x 28672
+  // 20.9 -> 15.3 (14 shares), 64 x 1024 x 28672 both row-major 30.0 -> 17.0, 128 x 1024 x 16384 18.1 -> 17.1 (8 shares
+  // instead of 16), 128 x 1024 x 14336 17.3 -> 16.4 (7 instead of 14), 128 x 128 x 16384 (one tile, 8 workgroups)
+  // 16.7 -> 13.3, 64 x 256 x 28672 both row-major 30.5 -> 16.7.  K = 8192 with up to 12 tiles: shares of 8 K-tiles
+  // (128 x 512 x 8192: 8 shares 12.3, 4 shares 12.9, tiled kernel's split 16.8, skinny kernel 19.3; with 16 tiles and
+  // more 4 shares are level or ahead: 256 x 2048 x 8192 16.7 against 18.2).  K beyond 16384 with 12 tiles or more and a
+  // tile-major B: shares of at least 28 K-tiles (512 x 512 x 28672, 16 tiles: 8 shares 19.6, 14 shares 21.9;
+  // 128 x 2048 x 28672 22.0 / 23.2; with 8 tiles 14 shares are ahead: 128 x 1024 x 28672 19.0 against 21.0; with a
+  // row-major B as well: 128 x 2048 x 28672 24.5 against 25.6, 512 x 384 x 28672 21.9 against 25.4).
   int best = 1;
-  for (int min_tiles = want == 0 && nkt == 64 && tiles >= 4 && tiles <= 12 ? 8 : 16; min_tiles >= 8 && best <= 1; min_tiles -= 8) {
+  const int first = want != 0 ? 16 : nkt == 64 && tiles <= 12 ? 8 : nkt > 128 && tiles >= 12 && g.layout_b ? 28 : 16;
+  for (int min_tiles = first; min_tiles >= 8 && best <= 1; min_tiles = min_tiles > 16 ? 16 : min_tiles - 8) {
     for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
       if (groups % sh == 0 && nkt / sh >= min_tiles && tiles * sh <= cus) {
         best = sh;
@@ -548,13 +552,12 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
       }
       if (want > 1) break;
     }
-    if (want == 0 && best > 1 && tiles < 4 && tiles * best * 8 < (long)cus * 3) best = 1;  // too few workgroups: try shorter shares
   }
   if (best <= 1) return 1;
-  // K beyond 16384, more than 16 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
+  // K beyond 16384, more than 32 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
   // streams B faster (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7; up
-  // to 16 tiles this kernel's: 128 x 2048 x 28672 23.4 against 26.0)
-  if (want == 0 && nkt > 128 && tiles > 16 && tiles * best * 4 < (long)cus * 3) return 1;
+  // to 32 tiles this kernel's: 128 x 2048 x 28672 22.0 against 26.0, 128 x 4096 x 28672 30.4 against 34.1)
+  if (want == 0 && nkt > 128 && tiles > 32 && tiles * best * 4 < (long)cus * 3) return 1;
   *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
   return best;
 }
