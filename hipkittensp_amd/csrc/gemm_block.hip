@@ -410,7 +410,9 @@ int cu_count_of_device() {
 // 1024 x 2048 x 8192: 23.5 against 25.1); three slots beyond, where two workgroups may share a CU and one's waits are the
 // other's work (256 tiles: 1024 x 4096 x 4096 18.6 against 20.0, 512 x 8192 x 2048 11.9 against 13.6, 2048 x 2048 x 8192
 // 28.8 against 31.2) -- except with K from 8192 on while a CU is left over (512 x 6144 x 16384: six slots 46.0 against
-// 51.9, 64 x 28672 x 8192: 34.9 against 38.2).  stages = 3 or 6 forces one (measurement).
+// 51.9, 64 x 28672 x 8192: 34.9 against 38.2), and three slots for K up to 2048, where filling six takes a good part of
+// the 8 - 16 K-tiles there are (384 x 2048 x 1024: 6.3 against 7.2, 512 x 4096 x 2048: 10.2 against 11.1, 24 shapes of 384 -
+// 1024 rows x N = 2048 .. 6144 all 7 - 14 % ahead).  stages = 3 or 6 forces one (measurement).
 template <int FA, int FB, bool FUSED>
 hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, hipStream_t s) {
   const int cus = cu_count_of_device();
@@ -421,7 +423,7 @@ hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, 
     else gemm_block_kernel<FA, FB, OutBf16, 4, 4, FUSED><<<grid, 512, 0, s>>>(a);
     return hipGetLastError();
   }
-  if (stages == 0) stages = (long)grid * 8 <= (long)cus * 5 || ((g.K >= 8192 || a.nsplit > 1) && grid < cus) ? 6 : 3;
+  if (stages == 0) stages = ((long)grid * 8 <= (long)cus * 5 && g.K > 2048) || ((g.K >= 8192 || a.nsplit > 1) && grid < cus) ? 6 : 3;
   if (stages == 6) {
     if (f32) gemm_block_kernel<FA, FB, OutF32, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
     else gemm_block_kernel<FA, FB, OutBf16, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
@@ -470,7 +472,10 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   const int cus = cu_count_of_device();
   const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
   const int nkt = g.K / kBK;
-  if (cus <= 0 || tiles > cus) return false;
+  // (up to twice as many tiles as CUs for K up to 2048 with both operands tile-major: two workgroups share a CU, one round;
+  // us, the 128 x 256 tiles -> this: 4096 x 2048 x 1024 16.4 -> 12.9, 1024 x 8192 x 1024 17.1 -> 13.3, 2048 x 4096 x 2048 20.6 -> 18.9)
+  const bool short_k = nkt <= 16 && g.layout_a && g.layout_b;
+  if (cus <= 0 || tiles > (short_k ? 2 * cus : cus)) return false;
   // tiles on more than half the CUs (three quarters with a row-major B), K up to 16384
   const bool fills = nkt <= 128 && (g.layout_b ? tiles * 16 >= (long)cus * 9 : tiles * 4 >= (long)cus * 3);
   // ... or on a quarter of them, K up to 8192 (a row-major A: up to 256 rows of it)

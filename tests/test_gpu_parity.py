@@ -157,7 +157,7 @@ def test_block_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
 
 
 @pytest.mark.parametrize("M,N,K,la,lb", [(256, 8192, 2048, 1, 1), (192, 4096, 4096, 0, 1), (512, 3072, 3072, 0, 0), (1024, 2048, 8192, 1, 1), (96, 16384, 1024, 0, 1),
-                                         (384, 6144, 4096, 1, 0)])
+                                         (384, 6144, 4096, 1, 0), (2048, 4096, 1024, 1, 1)])  # the last: 512 tiles, two workgroups per CU
 def test_block_kernel_is_chosen_and_matches_the_tiled_kernel(hk, M, N, K, la, lb):
     """Shapes on which the automatic path takes the block kernel (its tiles do not outnumber the CUs, K of moderate length):
     the result is the forced block kernel's bit for bit (the two agree on the dispatch), equals the 8-wave tiled kernel's
@@ -242,6 +242,7 @@ def test_kernel_choice_by_shape(hk):
     assert tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(32, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY
     assert tk.kernel_choice(256, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(512, 4096, 4096, 0, 1) == tk.KERNEL_BLOCK
     assert tk.kernel_choice(2048, 8192, 8192, 1, 1) == tk.KERNEL_TILED      # more 128 x 256 tiles than CUs
+    assert tk.kernel_choice(4096, 2048, 1024, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(4096, 2048, 4096, 1, 1) == tk.KERNEL_BLOCK_WIDE  # K up to 2048: up to two 128 x 128 tiles per CU
     assert tk.kernel_choice(1024, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK_WIDE and tk.kernel_choice(1024, 8192, 8192, 0, 1) == tk.KERNEL_TILED
     assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_BLOCK  # K % 512 != 0 is fine
     assert tk.kernel_choice(40, 36, 96) == tk.KERNEL_GENERIC
