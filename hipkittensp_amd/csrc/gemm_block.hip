@@ -52,7 +52,7 @@ struct BlockArgs {
   const uint8_t *A, *B, *As, *Bs;
   void* C;
   int M, N, K, tiles_m, tiles_n, layout_a, layout_b, group_m, xcd_remap;
-  int nsplit;  // workgroups that share an output tile, each over K / nsplit (a whole number of groups of four K-tiles); 1 = no split
+  int nsplit;  // workgroups that share an output tile, each over the same number of whole groups of four K-tiles (the last one over what is left); 1 = no split
   Epilogue ep;  // FUSED instantiations: scales / bias / activation on the accumulators before the output rounding
 };
 
@@ -74,10 +74,12 @@ __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_bl
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
   const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
   const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt_all = K / kBK, nk4_all = (nkt_all + 3) / 4;  // tile-major scales: one 512-byte chunk per 32 rows and group of four K-tiles, the last one padded
-  // K split: workgroup b takes share b / tiles of tile b % tiles, K-tiles [share, share + 1) * nkt, and leaves its fp32
+  // K split: workgroup b takes share b / tiles of tile b % tiles -- the same number of whole groups of four K-tiles for
+  // every share, the last one what is left of K (at least one K-tile: the launcher sees to that) -- and leaves its fp32
   // sums in matrix `share` of args.C, then a workspace of nsplit matrices [M, N] (ksplit_reduce_kernel adds them up)
   const int ntiles = args.tiles_m * args.tiles_n, share = blockIdx.x / ntiles;
-  const int nkt = nkt_all / args.nsplit, nk4 = (nkt + 3) / 4, kt0 = share * nkt;  // (a split leaves every share whole groups)
+  const int share_groups = (nk4_all + args.nsplit - 1) / args.nsplit, kt0 = share * share_groups * 4;
+  const int nkt = min(nkt_all - kt0, share_groups * 4), nk4 = (nkt + 3) / 4;
 
   const int tile = tile_order(blockIdx.x - share * ntiles, args.tiles_m, args.tiles_n, args.group_m, args.xcd_remap);
   if (tile < 0) return;  // never: the grid is the tile count times the shares
@@ -484,10 +486,11 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   const bool wide_short = nkt <= 32 && g.N >= 12288;
   if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5)));
   if (g.layout_a) return g.M > 128 || nkt <= 64;
-  // A row-major, B tile-major, few rows: the skinny kernel's, except a short K (above) and a B of 20480 .. 32767 rows
+  // A row-major, B tile-major, few rows: the skinny kernel's (where it takes the shape: K % 512 == 0; 16 x 4096 x 11008
+  // otherwise went to the tiled kernel, 35 us against 26 here), except a short K (above) and a B of 20480 .. 32767 rows
   // (its tiles on five eighths of the CUs or more, one CU at least left over): 32 x 20480 x 8192 38.3 -> 30.7 us,
   // 16 x 28672 x 8192 37.9 -> 33.6, 32 x 28672 x 16384 74.6 -> 66.3; 16384 rows 21 -> 26, 32768 rows level
-  return g.M > 128 || nkt <= 16 || (wide_short && g.M > 32) || (tiles * 8 >= (long)cus * 5 && tiles < cus && nkt <= 128);
+  return g.M > 128 || nkt <= 16 || (wide_short && g.M > 32) || (tiles * 8 >= (long)cus * 5 && tiles < cus && nkt <= 128) || !gemm_skinny_supports(g);
 }
 
 // The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
@@ -503,8 +506,9 @@ bool gemm_block_wide_preferred(const GemmArgs& g) {
 
 // K split of this kernel's 128 x 128 tiles: shares per output tile (1 = none) and the workspace they need.
 // want: 0 = where it pays (below), 1 = never, -1 = wherever the shape allows it, n > 1 = n shares if the shape allows it.
-// A share gets a whole number of groups of four K-tiles and at least 16 K-tiles (8 where no such split exists, and for
-// K = 8192 with few tiles); the shares of all tiles together do not outnumber the CUs.  Where it pays (sweep of 48 - 512 rows x nine (N, K) pairs x three layout pairs on MI355X, us, the
+// Every share gets the same whole number of groups of four K-tiles, the last share what is left of K (so K need not be a
+// multiple of 512), and at least 16 K-tiles (8 where no such split exists, and for K = 8192 with few tiles); the shares of
+// all tiles together do not outnumber the CUs.  Where it pays (sweep of 48 - 512 rows x nine (N, K) pairs x three layout pairs on MI355X, us, the
 // choice before -> this, each timed twice in alternation): K from 8192 on (5120 with both operands tile-major; shorter,
 // two launches lose), at most half as many tiles as CUs, more than three eighths of them only for K = 14336 .. 16384
 // (with K = 8192 an unsplit launch of that many tiles is as fast, with K = 28672 the tiled kernel's split is:
@@ -519,22 +523,32 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   if (!gemm_block_supports(g)) return 1;
   const int cus = cu_count_of_device();
   const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
-  const int nkt = g.K / kBK, groups = nkt / 4;
-  if (cus < 8 || tiles * 2 > cus || nkt % 4 != 0) return 1;  // shares are whole groups of four K-tiles
+  const int nkt = g.K / kBK, groups = (nkt + 3) / 4;  // groups of four K-tiles, the last one short if K % 512 != 0
+  if (cus < 8 || tiles * 2 > cus) return 1;
   if (want == 0) {
     if (nkt < 64 && !(g.layout_a && g.layout_b && nkt >= 40)) return 1;  // two launches for a K this short lose (96 x 8192 x 2048: 11 -> 14 us)
     const bool both = g.layout_a && g.layout_b;
+    // whether the tiled kernel has a split for this K (a multiple of 512 whose groups of four K-tiles divide among shares:
+    // 18944 = 37 groups and 22016 = 43 do not)
+    int tiled_rows = 0;
+    size_t tiled_part = 0;
+    const bool tiled_splits = gemm_tiled_supports(g) && tiled_ksplit_plan(g, 0, &tiled_rows, &tiled_part) > 1;
     if (tiles * 8 > (long)cus * 3) {  // more than three eighths as many tiles as CUs
-      // both tile-major: only K = 14336 .. 16384 (at 8192 the unsplit launch is as fast: 256 x 8192 x 8192 22.9 us against
-      // 26.5; at 28672 the tiled kernel's split is); a row-major operand: only K = 8192 (192 x 8192 x 8192, A row-major:
-      // 26.9 -> 22.8, both row-major 29.9 -> 25.3; 256 x 8192 x 16384 49.3 -> 51.6)
-      if (both ? (nkt < 112 || nkt > 128) : nkt > 64) return 1;
-    } else if (!both && tiles * 4 > cus && nkt > 64) {
+      // both tile-major: only K = 12288 .. 16384 (at 8192 the unsplit launch is as fast: 256 x 8192 x 8192 22.9 us against
+      // 26.5; at 28672 the tiled kernel's split is as fast or faster); a row-major operand: only K = 8192 (192 x 8192 x 8192,
+      // A row-major: 26.9 -> 22.8, both row-major 29.9 -> 25.3; 256 x 8192 x 16384 49.3 -> 51.6: beyond, the tiled kernel's
+      // split).  Where the tiled kernel has no split for K, a long K is split here (two shares on 96 - 128
+      // tiles against the unsplit launch, 13 shapes of 256 - 1024 rows: K = 11008 with a row-major operand 0.73 - 0.89 of
+      // its time, K = 18944 and 22016 0.62 - 0.76, both tile-major 0.67 - 0.93; K = 11008 both tile-major 0.86 - 1.08: not split)
+      if (both ? (nkt < 96 || (nkt > 128 && tiled_splits)) : (nkt > 64 && tiled_splits)) return 1;
+    } else if (!both && tiles * 4 > cus && nkt > 64 && tiled_splits) {
       return 1;  // a row-major operand and more than a quarter as many tiles as CUs: likewise only K = 8192
     }
     // the skinny kernel's (level at 33 - 64 rows and K = 8192 while N is one of its whole rounds: 64 x 8192 x 8192 16.1 us
     // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
-    if (!g.layout_a && (g.M <= 32 || (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)))) return 1;
+    // (the skinny kernel needs K % 512 == 0: other K, e.g. 11008 or 18944, stay here for any number of rows --
+    // 16 x 4096 x 11008 on 32 tiles unsplit: 26 us, the tiled kernel 35)
+    if (!g.layout_a && gemm_skinny_supports(g) && (g.M <= 32 || (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)))) return 1;
   }
   // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with up to 32 tiles such a
   // split beats shorter shares and every other kernel (us, 64 - 256 rows, what was chosen before -> this; each side
@@ -551,7 +565,9 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   const int first = want != 0 ? 16 : nkt == 64 && tiles <= 12 ? 8 : nkt > 128 && tiles >= 12 && g.layout_b ? 28 : 16;
   for (int min_tiles = first; min_tiles >= 8 && best <= 1; min_tiles = min_tiles > 16 ? 16 : min_tiles - 8) {
     for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
-      if (groups % sh == 0 && nkt / sh >= min_tiles && tiles * sh <= cus) {
+      // every share the same number of whole groups, the last share what is left (at least one group)
+      const int per = (groups + sh - 1) / sh;
+      if ((sh - 1) * per < groups && per * 4 >= min_tiles && tiles * sh <= cus) {
         best = sh;
         break;
       }
@@ -568,8 +584,8 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
 }
 
 // g.ksplit > 1 (with g.ks_part): the K range of every output tile split between that many workgroups, then
-// ksplit_reduce_kernel (gemm_tiled.hip), which also applies a fused epilogue.  The caller has checked that K / ksplit is a
-// whole number of groups of four K-tiles.
+// ksplit_reduce_kernel (gemm_tiled.hip), which also applies a fused epilogue.  The caller has checked that the last share
+// is not empty (block_ksplit_plan).
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s) {
   const int bn = g.tile_cols == 256 ? 256 : 128, nsplit = g.ksplit > 1 ? g.ksplit : 1;
   BlockArgs a{g.A, g.B, g.As, g.Bs, nsplit > 1 ? (void*)g.ks_part : g.C, g.M, g.N, g.K, (g.M + kBM - 1) / kBM, (g.N + bn - 1) / bn, g.layout_a, g.layout_b,

@@ -187,7 +187,9 @@ def test_block_kernel_is_chosen_and_matches_the_tiled_kernel(hk, M, N, K, la, lb
 
 
 @pytest.mark.parametrize("M,N,K,shares", [(128, 256, 4096, 2), (128, 512, 8192, 4), (100, 264, 4096, 2), (256, 512, 8192, 8), (64, 1024, 16384, 0), (192, 2048, 8192, 0),
-                                          (128, 512, 8192, 0), (96, 520, 28672, 0), (100, 128, 16384, 0), (512, 512, 28672, 0)])
+                                          (128, 512, 8192, 0), (96, 520, 28672, 0), (100, 128, 16384, 0), (512, 512, 28672, 0),
+                                          # K % 512 != 0: the last share takes what is left of K, down to a single K-tile
+                                          (128, 256, 2816, 2), (100, 264, 4480, 3), (128, 384, 4224, 4), (16, 4096, 11008, 0), (256, 512, 11008, 0), (64, 1024, 18944, 0)])
 @pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2)])
 def test_block_kernel_k_split(hk, M, N, K, shares, fa, fb):
     """The block kernel with the K range of every output tile split between several workgroups: fp32 partial matrices in
@@ -250,6 +252,7 @@ def test_kernel_choice_by_shape(hk):
     for la, lb in ((0, 0), (0, 1), (1, 1)):
         assert tk.kernel_choice(128, 512, 16384, la, lb) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 1024, 8192, la, lb) == tk.CHOICE_BLOCK_K_SPLIT
     assert tk.kernel_choice(64, 1024, 28672) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 1024, 8192) == tk.KERNEL_SKINNY   # the skinny kernel's up to 64 rows at K = 8192
+    assert tk.kernel_choice(16, 4096, 11008, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT   # K % 512 != 0: not the skinny kernel's
     assert tk.kernel_choice(128, 128, 16384) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 384, 28672, 1, 1) == tk.CHOICE_BLOCK_K_SPLIT  # one and six tiles
     prev = tk.set_k_split(1)
     try:
