@@ -541,8 +541,12 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
       // tiles against the unsplit launch, 13 shapes of 256 - 1024 rows: K = 11008 with a row-major operand 0.73 - 0.89 of
       // its time, K = 18944 and 22016 0.62 - 0.76, both tile-major 0.67 - 0.93; K = 11008 both tile-major 0.86 - 1.08: not split)
       if (both ? (nkt < 96 || (nkt > 128 && tiled_splits)) : (nkt > 64 && tiled_splits)) return 1;
-    } else if (!both && tiles * 4 > cus && nkt > 64 && tiled_splits) {
-      return 1;  // a row-major operand and more than a quarter as many tiles as CUs: likewise only K = 8192
+    } else if (!both && tiles * 3 > cus && nkt > 64 && tiled_splits) {
+      // a row-major operand and more than a third as many tiles as CUs (two shares at most): likewise only K = 8192.  Up
+      // to a third, three shares beat the tiled kernel's split (us, 52 shapes of 128 - 768 rows, 65 - 85 tiles, K = 12288 ..
+      // 28672: 192 x 5120 x 16384 33.0 -> 27.6, both row-major 39.7 -> 31.3; 512 x 2560 x 28672 47.8 -> 43.1 / 67.4 -> 51.6;
+      // 128 x 10240 x 14336 43.0 -> 38.7; all between 0.77 and 0.95 of its time)
+      return 1;
     }
     // the skinny kernel's (level at 33 - 64 rows and K = 8192 while N is one of its whole rounds: 64 x 8192 x 8192 16.1 us
     // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
