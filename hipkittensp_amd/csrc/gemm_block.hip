@@ -483,14 +483,21 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // ... or on a quarter of them, K up to 8192 (a row-major A: up to 256 rows of it)
   const bool quarter = nkt <= 64 && tiles * 4 >= cus && g.layout_b && (g.layout_a || g.M <= 256);
   if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
-  const bool wide_short = nkt <= 32 && g.N >= 12288;
+  bool wide_short = nkt <= 32 && g.N >= 12288;
   if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5)));
   if (g.layout_a) return g.M > 128 || nkt <= 64;
   // A row-major, B tile-major, few rows: the skinny kernel's (where it takes the shape: K % 512 == 0; 16 x 4096 x 11008
   // otherwise went to the tiled kernel, 35 us against 26 here), except a short K (above) and a B of 20480 .. 32767 rows
-  // (its tiles on five eighths of the CUs or more, one CU at least left over): 32 x 20480 x 8192 38.3 -> 30.7 us,
-  // 16 x 28672 x 8192 37.9 -> 33.6, 32 x 28672 x 16384 74.6 -> 66.3; 16384 rows 21 -> 26, 32768 rows level
-  return g.M > 128 || nkt <= 16 || (wide_short && g.M > 32) || (tiles * 8 >= (long)cus * 5 && tiles < cus && nkt <= 128) || !gemm_skinny_supports(g);
+  // (its tiles on more than half the CUs, one CU at least left over: the skinny kernel's workgroups of 32 rows of B then
+  // need a third round that is mostly empty): 32 x 20480 x 8192 38.3 -> 30.7 us, 16 x 28672 x 8192 37.9 -> 33.6,
+  // 32 x 28672 x 16384 74.6 -> 66.3, 48 x 18944 x 5120 28.1 -> 16.1, 32 x 18944 x 8192 36.5 -> 29.0 (16 rows level);
+  // 16384 rows 21 -> 26, 32768 rows level.  K up to 2048: from 65 rows on, or with that many tiles (up to 64 rows the
+  // skinny kernel is 10 - 20 % ahead: 48 x 4096 x 2048 6.1 us against 7.8)
+  // (K = 5120 as well from 65 rows on: 96 x 14336 x 5120 20.9 us on the tiled kernel -> 18.9, 128 x 12288 x 5120 22.4 -> 20.4)
+  // (and from 10240 rows of B: 96 x 11008 x 3584 18.0 us on the skinny kernel -> 14.1, 128 x 11008 x 5120 22.1 on the tiled kernel -> 20.1)
+  wide_short = wide_short || (nkt <= 40 && g.M > 64 && g.N >= 10240);
+  const bool many_tiles = tiles * 2 > cus && tiles < cus && nkt <= 128;
+  return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
 }
 
 // The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
