@@ -485,7 +485,9 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
   bool wide_short = nkt <= 32 && g.N >= 12288;
   if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5)));
-  if (g.layout_a) return g.M > 128 || nkt <= 64;
+  // (A tile-major: neither the skinny nor the mid-M kernel takes it, and against the tiled kernel's 256-row tiles this one
+  // wins for any K once the splits have been asked: 32 x 14592 x 11904 47.2 us -> 35.4, 32 x 27008 x 21248 89.0 -> 75.4)
+  if (g.layout_a) return g.M > 128 || nkt <= 64 || !first;
   // A row-major, B tile-major, few rows: the skinny kernel's (where it takes the shape: K % 512 == 0; 16 x 4096 x 11008
   // otherwise went to the tiled kernel, 35 us against 26 here), except a short K (above) and a B of 20480 .. 32767 rows
   // (its tiles on more than half the CUs, one CU at least left over: the skinny kernel's workgroups of 32 rows of B then
@@ -532,14 +534,17 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
   const int nkt = g.K / kBK, groups = (nkt + 3) / 4;  // groups of four K-tiles, the last one short if K % 512 != 0
   if (cus < 8 || tiles * 2 > cus) return 1;
+  // whether the tiled kernel has a split for this K (a multiple of 512 whose groups of four K-tiles divide among shares:
+  // 18944 = 37 groups and 22016 = 43 do not)
+  int tiled_rows = 0;
+  size_t tiled_part = 0;
+  const bool tiled_splits = want == 0 && gemm_tiled_supports(g) && tiled_ksplit_plan(g, 0, &tiled_rows, &tiled_part) > 1;
   if (want == 0) {
-    if (nkt < 64 && !(g.layout_a && g.layout_b && nkt >= 40)) return 1;  // two launches for a K this short lose (96 x 8192 x 2048: 11 -> 14 us)
+    // two launches for a K below 5120 lose (96 x 8192 x 2048: 11 -> 14 us; 256 x 2048 x 4096 13.3 -> 13.9); from there on
+    // they pay (us, unsplit -> split: 256 x 2048 x 5120, A row-major 19.8 -> 16.9, both row-major 24.1 -> 18.2;
+    // 512 x 1024 x 7168 25.2 -> 17.1; 128 x 2048 x 5504, which the skinny kernel cannot take, 20.8 -> 14.9)
+    if (nkt < 40) return 1;
     const bool both = g.layout_a && g.layout_b;
-    // whether the tiled kernel has a split for this K (a multiple of 512 whose groups of four K-tiles divide among shares:
-    // 18944 = 37 groups and 22016 = 43 do not)
-    int tiled_rows = 0;
-    size_t tiled_part = 0;
-    const bool tiled_splits = gemm_tiled_supports(g) && tiled_ksplit_plan(g, 0, &tiled_rows, &tiled_part) > 1;
     if (tiles * 8 > (long)cus * 3) {  // more than three eighths as many tiles as CUs
       // both tile-major: only K = 12288 .. 16384 (at 8192 the unsplit launch is as fast: 256 x 8192 x 8192 22.9 us against
       // 26.5; at 28672 the tiled kernel's split is as fast or faster); a row-major operand: only K = 8192 (192 x 8192 x 8192,
@@ -547,8 +552,10 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
       // split).  Where the tiled kernel has no split for K, a long K is split here (two shares on 96 - 128
       // tiles against the unsplit launch, 13 shapes of 256 - 1024 rows: K = 11008 with a row-major operand 0.73 - 0.89 of
       // its time, K = 18944 and 22016 0.62 - 0.76, both tile-major 0.67 - 0.93; K = 11008 both tile-major 0.86 - 1.08: not split)
-      if (both ? (nkt < 96 || (nkt > 128 && tiled_splits)) : (nkt > 64 && tiled_splits)) return 1;
-    } else if (!both && tiles * 3 > cus && nkt > 64 && tiled_splits) {
+      // (a row-major operand, 96 - 128 tiles, two shares against the tiled kernel's split: K = 12288 0.73 - 0.81 of the unsplit
+      // time against 0.76 - 0.96, K = 14336 0.70 - 0.78 against 0.72 - 0.89, K = 16384 level, K = 28672 behind)
+      if (both ? (nkt < 96 || (nkt > 128 && tiled_splits)) : (nkt > 128 && tiled_splits)) return 1;
+    } else if (!both && tiles * 3 > cus && nkt > 128 && tiled_splits) {
       // a row-major operand and more than a third as many tiles as CUs (two shares at most): likewise only K = 8192.  Up
       // to a third, three shares beat the tiled kernel's split (us, 52 shapes of 128 - 768 rows, 65 - 85 tiles, K = 12288 ..
       // 28672: 192 x 5120 x 16384 33.0 -> 27.6, both row-major 39.7 -> 31.3; 512 x 2560 x 28672 47.8 -> 43.1 / 67.4 -> 51.6;
@@ -559,7 +566,20 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
     // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
     // (the skinny kernel needs K % 512 == 0: other K, e.g. 11008 or 18944, stay here for any number of rows --
     // 16 x 4096 x 11008 on 32 tiles unsplit: 26 us, the tiled kernel 35)
-    if (!g.layout_a && gemm_skinny_supports(g) && (g.M <= 32 || (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)))) return 1;
+    if (!g.layout_a && gemm_skinny_supports(g)) {
+      // up to 32 rows: the skinny kernel's, unless K is long and its last round of workgroups (32 rows of B each, 256 a
+      // round) is at most half full -- 16 x 8800 x 14848 (275 workgroups) 26.8 us -> 21.9, 32 x 9088 x 28672 61.6 -> 41.2,
+      // 8 x 10240 x 28672 49.6 -> 42.4, 16 x 8800 x 13824 24.7 -> 20.2; at K = 8192 it stays ahead (16 x 9088 x 8192 14.1
+      // against 15.1), with the last round three quarters full as well (16 x 14336 x 28672 59.0 against 57.0), and against
+      // row-major weights (1 x 11264 x 32256 58 against 76)
+      const long wgs = (g.N + 31) / 32;
+      const bool last_round_thin = wgs > 256 && wgs % 256 >= 1 && wgs % 256 <= 128;
+      if (g.M <= 32 && !(last_round_thin && nkt >= 96 && g.layout_b)) return 1;
+      if (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)) return 1;
+      // K below 8192: the skinny kernel's up to 96 rows (64 x 4096 x 6144 10.9 us against 12.9 split), up to 128 below 7168
+      // (128 x 2048 x 7680 18.4 -> 15.7, 128 x 2048 x 6144 level)
+      if (nkt < 64 && (g.M <= 96 || (g.M <= 128 && nkt < 56))) return 1;
+    }
   }
   // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with up to 32 tiles such a
   // split beats shorter shares and every other kernel (us, 64 - 256 rows, what was chosen before -> this; each side
@@ -589,7 +609,7 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   // K beyond 16384, more than 32 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
   // streams B faster (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7; up
   // to 32 tiles this kernel's: 128 x 2048 x 28672 22.0 against 26.0, 128 x 4096 x 28672 30.4 against 34.1)
-  if (want == 0 && nkt > 128 && tiles > 32 && tiles * best * 4 < (long)cus * 3) return 1;
+  if (want == 0 && nkt > 128 && tiles > 32 && tiles * best * 4 < (long)cus * 3 && tiled_splits) return 1;
   *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
   return best;
 }
