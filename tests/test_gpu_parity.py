@@ -253,6 +253,11 @@ def test_kernel_choice_by_shape(hk):
         assert tk.kernel_choice(128, 512, 16384, la, lb) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 1024, 8192, la, lb) == tk.CHOICE_BLOCK_K_SPLIT
     assert tk.kernel_choice(64, 1024, 28672) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 1024, 8192) == tk.KERNEL_SKINNY   # the skinny kernel's up to 64 rows at K = 8192
     assert tk.kernel_choice(16, 4096, 11008, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT   # K % 512 != 0: not the skinny kernel's
+    assert tk.kernel_choice(128, 2048, 5504, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 2048, 4096, 0, 1) != tk.CHOICE_BLOCK_K_SPLIT  # split from K = 5120 on
+    assert tk.kernel_choice(32, 14592, 11904, 1, 1) == tk.KERNEL_BLOCK          # A tile-major, few rows, no split for this K
+    # the skinny kernel's last round of workgroups (32 rows of B each, 256 a round) nearly empty, long K, tile-major weights
+    assert tk.kernel_choice(16, 8800, 14848, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(16, 8192, 14848, 0, 1) == tk.KERNEL_SKINNY
+    assert tk.kernel_choice(96, 23344, 8704) != tk.KERNEL_SKINNY                # K % 1024 != 0: the tiled kernel's, not the skinny kernel's
     assert tk.kernel_choice(128, 128, 16384) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 384, 28672, 1, 1) == tk.CHOICE_BLOCK_K_SPLIT  # one and six tiles
     prev = tk.set_k_split(1)
     try:
