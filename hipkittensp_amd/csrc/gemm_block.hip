@@ -411,8 +411,8 @@ int cu_count_of_device() {
 // on its CU anyway, and loads that run six K-tiles ahead cover the way from HBM (256 x 8192 x 8192: 23.0 us against 24.7,
 // 1024 x 2048 x 8192: 23.5 against 25.1); three slots beyond, where two workgroups may share a CU and one's waits are the
 // other's work (256 tiles: 1024 x 4096 x 4096 18.6 against 20.0, 512 x 8192 x 2048 11.9 against 13.6, 2048 x 2048 x 8192
-// 28.8 against 31.2) -- except with K from 8192 on while a CU is left over (512 x 6144 x 16384: six slots 46.0 against
-// 51.9, 64 x 28672 x 8192: 34.9 against 38.2), and three slots for K up to 2048, where filling six takes a good part of
+// 28.8 against 31.2) -- except with K from 6144 on while a CU is left over (512 x 6144 x 16384: six slots 46.0 against
+// 51.9, 64 x 28672 x 8192: 34.9 against 38.2, 1 x 27136 x 7680: 30.5 against 34.1; at K = 5120 three: 96 x 20480 x 5120 22.5 against 23.6), and three slots for K up to 2048, where filling six takes a good part of
 // the 8 - 16 K-tiles there are (384 x 2048 x 1024: 6.3 against 7.2, 512 x 4096 x 2048: 10.2 against 11.1, 24 shapes of 384 -
 // 1024 rows x N = 2048 .. 6144 all 7 - 14 % ahead).  stages = 3 or 6 forces one (measurement).
 template <int FA, int FB, bool FUSED>
@@ -425,7 +425,7 @@ hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, 
     else gemm_block_kernel<FA, FB, OutBf16, 4, 4, FUSED><<<grid, 512, 0, s>>>(a);
     return hipGetLastError();
   }
-  if (stages == 0) stages = ((long)grid * 8 <= (long)cus * 5 && g.K > 2048) || ((g.K >= 8192 || a.nsplit > 1) && grid < cus) ? 6 : 3;
+  if (stages == 0) stages = ((long)grid * 8 <= (long)cus * 5 && g.K > 2048) || ((g.K >= 6144 || a.nsplit > 1) && grid < cus) ? 6 : 3;
   if (stages == 6) {
     if (f32) gemm_block_kernel<FA, FB, OutF32, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
     else gemm_block_kernel<FA, FB, OutBf16, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
@@ -484,7 +484,9 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   const bool quarter = nkt <= 64 && tiles * 4 >= cus && g.layout_b && (g.layout_a || g.M <= 256);
   if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
   bool wide_short = nkt <= 32 && g.N >= 12288;
-  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5)));
+  // (B row-major as well from 32 rows on with tiles on more than half the CUs: 48 x 18816 x 4608 27.2 us on the skinny kernel -> 18.9)
+  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5))) ||
+                          (g.M >= 32 && tiles * 2 > cus && tiles < cus && nkt <= 128 && gemm_skinny_preferred(g));
   // (A tile-major: neither the skinny nor the mid-M kernel takes it, and against the tiled kernel's 256-row tiles this one
   // wins for any K once the splits have been asked: 32 x 14592 x 11904 47.2 us -> 35.4, 32 x 27008 x 21248 89.0 -> 75.4)
   if (g.layout_a) return g.M > 128 || nkt <= 64 || !first;
@@ -498,7 +500,8 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // (K = 5120 as well from 65 rows on: 96 x 14336 x 5120 20.9 us on the tiled kernel -> 18.9, 128 x 12288 x 5120 22.4 -> 20.4)
   // (and from 10240 rows of B: 96 x 11008 x 3584 18.0 us on the skinny kernel -> 14.1, 128 x 11008 x 5120 22.1 on the tiled kernel -> 20.1)
   wide_short = wide_short || (nkt <= 40 && g.M > 64 && g.N >= 10240);
-  const bool many_tiles = tiles * 2 > cus && tiles < cus && nkt <= 128;
+  // (up to 31 rows only from five eighths of the CUs on: 1 x 20736 x 6144 18.9 us on the skinny kernel, 25.0 here)
+  const bool many_tiles = (g.M >= 32 ? tiles * 2 > cus : tiles * 8 >= (long)cus * 5) && tiles < cus && nkt <= 128;
   return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
 }
 
@@ -554,8 +557,9 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
       // its time, K = 18944 and 22016 0.62 - 0.76, both tile-major 0.67 - 0.93; K = 11008 both tile-major 0.86 - 1.08: not split)
       // (a row-major operand, 96 - 128 tiles, two shares against the tiled kernel's split: K = 12288 0.73 - 0.81 of the unsplit
       // time against 0.76 - 0.96, K = 14336 0.70 - 0.78 against 0.72 - 0.89, K = 16384 level, K = 28672 behind)
-      if (both ? (nkt < 96 || (nkt > 128 && tiled_splits)) : (nkt > 128 && tiled_splits)) return 1;
-    } else if (!both && tiles * 3 > cus && nkt > 128 && tiled_splits) {
+      // (K = 19456, both tile-major, 121 tiles: two shares here 49.6 us, the tiled kernel's split 67.4: it takes over from K = 24576)
+      if (both ? (nkt < 96 || (nkt >= 192 && tiled_splits)) : (nkt >= 192 && tiled_splits)) return 1;
+    } else if (!both && tiles * 3 > cus && nkt >= 192 && tiled_splits) {
       // a row-major operand and more than a third as many tiles as CUs (two shares at most): likewise only K = 8192.  Up
       // to a third, three shares beat the tiled kernel's split (us, 52 shapes of 128 - 768 rows, 65 - 85 tiles, K = 12288 ..
       // 28672: 192 x 5120 x 16384 33.0 -> 27.6, both row-major 39.7 -> 31.3; 512 x 2560 x 28672 47.8 -> 43.1 / 67.4 -> 51.6;
@@ -568,17 +572,17 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
     // 16 x 4096 x 11008 on 32 tiles unsplit: 26 us, the tiled kernel 35)
     if (!g.layout_a && gemm_skinny_supports(g)) {
       // up to 32 rows: the skinny kernel's, unless K is long and its last round of workgroups (32 rows of B each, 256 a
-      // round) is at most half full -- 16 x 8800 x 14848 (275 workgroups) 26.8 us -> 21.9, 32 x 9088 x 28672 61.6 -> 41.2,
+      // round) is at most five eighths full -- 16 x 8800 x 14848 (275 workgroups) 26.8 us -> 21.9, 32 x 9088 x 28672 61.6 -> 41.2,
       // 8 x 10240 x 28672 49.6 -> 42.4, 16 x 8800 x 13824 24.7 -> 20.2; at K = 8192 it stays ahead (16 x 9088 x 8192 14.1
       // against 15.1), with the last round three quarters full as well (16 x 14336 x 28672 59.0 against 57.0), and against
       // row-major weights (1 x 11264 x 32256 58 against 76)
       const long wgs = (g.N + 31) / 32;
-      const bool last_round_thin = wgs > 256 && wgs % 256 >= 1 && wgs % 256 <= 128;
+      const bool last_round_thin = wgs > 256 && wgs % 256 >= 1 && wgs % 256 <= 160;
       if (g.M <= 32 && !(last_round_thin && nkt >= 96 && g.layout_b)) return 1;
       if (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)) return 1;
       // K below 8192: the skinny kernel's up to 96 rows (64 x 4096 x 6144 10.9 us against 12.9 split), up to 128 below 7168
       // (128 x 2048 x 7680 18.4 -> 15.7, 128 x 2048 x 6144 level)
-      if (nkt < 64 && (g.M <= 96 || (g.M <= 128 && nkt < 56))) return 1;
+      if (nkt < 64 && gemm_skinny_preferred(g) && (g.M <= 96 || (g.M <= 128 && nkt < 56))) return 1;  // (where it would be chosen: 96 x 9344 x 7680 goes to the tiled kernel otherwise, 32.5 us against 21.1 split)
     }
   }
   // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with up to 32 tiles such a
@@ -606,10 +610,10 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
     }
   }
   if (best <= 1) return 1;
-  // K beyond 16384, more than 32 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
+  // K from 24576 on, more than 32 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
   // streams B faster (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7; up
   // to 32 tiles this kernel's: 128 x 2048 x 28672 22.0 against 26.0, 128 x 4096 x 28672 30.4 against 34.1)
-  if (want == 0 && nkt > 128 && tiles > 32 && tiles * best * 4 < (long)cus * 3 && tiled_splits) return 1;
+  if (want == 0 && nkt >= 192 && tiles > 32 && tiles * best * 4 < (long)cus * 3 && tiled_splits) return 1;
   *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
   return best;
 }

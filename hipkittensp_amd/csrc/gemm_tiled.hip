@@ -835,8 +835,9 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
 // (the last three for measurement).  Returns the shares per tile (1: no split) and the tile height and workspace size
 // that go with them.
 // Where it pays (measured on MI355X against the best unsplit kernel over 360 shapes, M = 8 .. 2048, N = 1024 .. 57344,
-// tile-major and row-major B), in output tiles of 256 x 256: with K >= 14336 up to 64 tiles (128 beyond K = 16384:
-// 256 x 17920 x 23040 159 -> 114 us, 160 x 16768 x 17408 138 -> 110, 192 x 26880 x 21504 183 -> 155):
+// tile-major and row-major B), in output tiles of 256 x 256: with K >= 12288 up to 64 tiles (128 from K = 24576 on, and
+// for up to 256 rows of A: 256 x 17920 x 23040 159 -> 114 us, 160 x 16768 x 17408 138 -> 110, 160 x 18304 x 13824 81 -> 60;
+// with 2048 rows it loses: 2048 x 5120 x 16384 122 -> 134):
 // 0.45 - 0.9 of the unsplit time, e.g. 256 x 8192 x 28672 108 -> 63 us, 128 x 4096 x 14336 46 -> 24 us, 1024 x 1024 x 16384
 // 60 -> 34 us; with 8192 <= K < 14336 up to 32 tiles where the skinny kernel is not an option (more than 128 rows of A, or
 // a tile-major A): 256 x 2048 x 8192 28.5 -> 21 us, 768 x 2048 x 8192 33 -> 27 us; and up to 64 tiles for 65 - 128 rows of A
@@ -849,7 +850,7 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
   if (cus < 8) return 1;
   if (want == 0) {
     const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const bool pays = nkt >= 112 ? (tiles256 <= 64 || (nkt > 128 && tiles256 <= 128))
+    const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (g.M <= 256 || nkt >= 192)))
                                  : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
                                                  // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
                                                  (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192));
@@ -858,7 +859,7 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
       // up to 64 rows of a row-major A are the skinny kernel's, except more than 32 against tile-major weights with a
       // very long K, or a long K and a width that leaves the skinny kernel's last round of workgroups part empty
       const bool ragged = g.N > 8192 && g.N % 8192 != 0;
-      if (!(g.M > 32 && g.layout_b && tiles256 <= (nkt >= 192 ? 128 : 64) && (nkt >= 192 || ragged))) return 1;
+      if (!(g.M > 32 && g.layout_b && tiles256 <= 128 && (nkt >= 192 || ragged))) return 1;
     }
   }
   int best = 1, best_rows = 0;
