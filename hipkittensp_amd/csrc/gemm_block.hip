@@ -485,8 +485,11 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
   bool wide_short = nkt <= 32 && g.N >= 12288;
   // (B row-major as well from 32 rows on with tiles on more than half the CUs: 48 x 18816 x 4608 27.2 us on the skinny kernel -> 18.9)
-  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5))) ||
-                          (g.M >= 32 && tiles * 2 > cus && tiles < cus && nkt <= 128 && gemm_skinny_preferred(g));
+  // (K up to 2048 wherever the skinny kernel does not come first: 160 x 9216 x 1536 10.1 us on the tiled kernel -> 8.9,
+  // 96 x 4840 x 1792 9.9 -> 8.1, 24 x 12032 x 768 6.9 -> 6.1)
+  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (nkt <= 16 && (g.M > 128 || !gemm_skinny_preferred(g))) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5))) ||
+                          // (up to K = 10240: 48 x 23280 x 9216 53.9 us on the skinny kernel -> 51.9, 64 x 22784 x 10752 60.9 -> 62.8, 64 x 16640 x 16384 82.2 -> 89.3)
+                          (g.M >= 32 && tiles * 2 > cus && tiles < cus && nkt <= 80 && gemm_skinny_preferred(g));
   // (A tile-major: neither the skinny nor the mid-M kernel takes it, and against the tiled kernel's 256-row tiles this one
   // wins for any K once the splits have been asked: 32 x 14592 x 11904 47.2 us -> 35.4, 32 x 27008 x 21248 89.0 -> 75.4)
   if (g.layout_a) return g.M > 128 || nkt <= 64 || !first;
@@ -501,7 +504,12 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // (and from 10240 rows of B: 96 x 11008 x 3584 18.0 us on the skinny kernel -> 14.1, 128 x 11008 x 5120 22.1 on the tiled kernel -> 20.1)
   wide_short = wide_short || (nkt <= 40 && g.M > 64 && g.N >= 10240);
   // (up to 31 rows only from five eighths of the CUs on: 1 x 20736 x 6144 18.9 us on the skinny kernel, 25.0 here)
-  const bool many_tiles = (g.M >= 32 ? tiles * 2 > cus : tiles * 8 >= (long)cus * 5) && tiles < cus && nkt <= 128;
+  // (from 32 rows on a tile for every CU as well: 48 x 32768 x 12288 63.6 us on the tiled kernel, 70.6 on the skinny kernel -> 58.7)
+  // (K beyond 16384: from 32 rows on as well, 32 x 16640 x 28672 102 us on the skinny kernel -> 91.7; with fewer rows
+  // only up to K = 20480 with tiles on thirteen sixteenths of the CUs, 16 x 27392 x 19456 81.6 -> 70.9, 8 x 27904 x 18944
+  // 76.2 -> 69.9; 16 x 23808 x 19968 level, 8 x 16640 x 28672 76.4 -> 79.6)
+  const bool many_tiles = g.M >= 32 ? tiles * 2 > cus && tiles <= cus && nkt <= 256
+                                    : tiles * 8 >= (long)cus * 5 && tiles < cus && (nkt <= 128 || (nkt <= 160 && tiles * 16 >= (long)cus * 13));
   return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
 }
 
