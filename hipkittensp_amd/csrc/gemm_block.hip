@@ -484,12 +484,20 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   const bool quarter = nkt <= 64 && tiles * 4 >= cus && g.layout_b && (g.layout_a || g.M <= 256);
   if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
   bool wide_short = nkt <= 32 && g.N >= 12288;
-  // (B row-major as well from 32 rows on with tiles on more than half the CUs: 48 x 18816 x 4608 27.2 us on the skinny kernel -> 18.9)
-  // (K up to 2048 wherever the skinny kernel does not come first: 160 x 9216 x 1536 10.1 us on the tiled kernel -> 8.9,
-  // 96 x 4840 x 1792 9.9 -> 8.1, 24 x 12032 x 768 6.9 -> 6.1)
-  if (!g.layout_b) return (g.M > 256 && nkt <= 40) || (nkt <= 16 && (g.M > 128 || !gemm_skinny_preferred(g))) || (g.M > 128 && fills) || (wide_short && (g.M > 64 || (g.M >= 32 && tiles * 8 >= (long)cus * 5))) ||
-                          // (up to K = 10240: 48 x 23280 x 9216 53.9 us on the skinny kernel -> 51.9, 64 x 22784 x 10752 60.9 -> 62.8, 64 x 16640 x 16384 82.2 -> 89.3)
-                          (g.M >= 32 && tiles * 2 > cus && tiles < cus && nkt <= 80 && gemm_skinny_preferred(g));
+  if (!g.layout_b) {
+    // more than 256 rows up to K = 5120, more than 128 where the tiles fill the CUs
+    if ((g.M > 256 && nkt <= 40) || (g.M > 128 && fills)) return true;
+    // K up to 2048 wherever the skinny kernel does not come first: 160 x 9216 x 1536 10.1 us on the tiled kernel -> 8.9,
+    // 96 x 4840 x 1792 9.9 -> 8.1, 24 x 12032 x 768 6.9 -> 6.1
+    if (nkt <= 16 && (g.M > 128 || !gemm_skinny_preferred(g))) return true;
+    // K up to 4096 against 12288 rows of B or more: from 65 rows on, from 24 with tiles on five eighths of the CUs
+    // (24 x 28672 x 4096 21.1 us on the skinny kernel -> 18.5, 16 rows level)
+    if (wide_short && (g.M > 64 || (g.M >= 24 && tiles * 8 >= (long)cus * 5))) return true;
+    // from 32 rows on with tiles on more than half the CUs, up to K = 10240 (48 x 18816 x 4608 27.2 us on the skinny kernel
+    // -> 18.9, 48 x 23280 x 9216 53.9 -> 51.9; beyond, 64 x 22784 x 10752 60.9 -> 62.8, 64 x 16640 x 16384 82.2 -> 89.3);
+    // 32 rows, the skinny kernel's largest single row group, only up to K = 7168 (32 x 24576 x 8192 38.9 -> 43.3)
+    return g.M >= 32 && tiles * 2 > cus && tiles < cus && nkt <= (g.M > 32 ? 80 : 56) && gemm_skinny_preferred(g);
+  }
   // (A tile-major: neither the skinny nor the mid-M kernel takes it, and against the tiled kernel's 256-row tiles this one
   // wins for any K once the splits have been asked: 32 x 14592 x 11904 47.2 us -> 35.4, 32 x 27008 x 21248 89.0 -> 75.4)
   if (g.layout_a) return g.M > 128 || nkt <= 64 || !first;

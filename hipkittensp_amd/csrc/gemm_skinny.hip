@@ -309,7 +309,9 @@ bool gemm_wide_n_prefers_tiled(const GemmArgs& g) {
   const long tiles = (g.N + 255) / 256;
   if (g.M <= 16) return g.layout_b && tiles >= 256 && g.K <= 4096;
   if (g.layout_b) return tiles >= 160 || (tiles >= 96 && g.M >= 24);
-  return g.M > 64 ? tiles >= 96 : g.M > 32 && (tiles >= 224 || (tiles >= 96 && g.K <= 4096));
+  // (24 - 32 rows with K <= 4096 from N = 98304 on: 32 x 128256 x 4096 105 -> 94, 24 x 128256 x 4096 99 -> 91)
+  if (g.M <= 32) return g.M >= 24 && tiles >= 384 && g.K <= 4096;
+  return g.M > 64 ? tiles >= 96 : tiles >= 224 || (tiles >= 96 && g.K <= 4096);
 }
 
 bool gemm_skinny_preferred(const GemmArgs& g) {
