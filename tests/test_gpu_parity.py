@@ -259,6 +259,16 @@ def test_kernel_choice_by_shape(hk):
     assert tk.kernel_choice(16, 8800, 14848, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(16, 8192, 14848, 0, 1) == tk.KERNEL_SKINNY
     assert tk.kernel_choice(96, 23344, 8704) != tk.KERNEL_SKINNY                # K % 1024 != 0: the tiled kernel's, not the skinny kernel's
     assert tk.kernel_choice(128, 128, 16384) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 384, 28672, 1, 1) == tk.CHOICE_BLOCK_K_SPLIT  # one and six tiles
+    # few rows against wide weights: the block kernel with a tile for every CU, and beyond K = 16384 where its tiles fill the CUs
+    assert tk.kernel_choice(48, 32768, 12288, 0, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(32, 16640, 28672, 0, 1) == tk.KERNEL_BLOCK
+    assert tk.kernel_choice(16, 27392, 19456, 0, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(16, 23808, 19968, 0, 1) == tk.KERNEL_SKINNY
+    # B row-major: a short K wherever the skinny kernel does not come first, 24 rows at K = 4096, 32 rows only up to K = 7168
+    assert tk.kernel_choice(160, 9216, 1536, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(24, 28672, 4096, 0, 0) == tk.KERNEL_BLOCK
+    assert tk.kernel_choice(32, 24576, 8192, 0, 0) == tk.KERNEL_SKINNY and tk.kernel_choice(48, 24576, 8192, 0, 0) == tk.KERNEL_BLOCK
+    # the tiled kernel's split: three shares a tile for 33 - 64 rows against a wide row-major B, 65 - 128 tiles with few rows or a row-major B
+    assert tk.kernel_choice(64, 16640, 12288, 0, 0) == tk.CHOICE_TILED_K_SPLIT and tk.k_split_plan(64, 16640, 12288, 0, 0, 0)[0] == 3
+    assert tk.kernel_choice(64, 24576, 12288, 0, 0) != tk.CHOICE_TILED_K_SPLIT   # two shares a tile: level, not split
+    assert tk.kernel_choice(160, 18304, 13824, 0, 1) == tk.CHOICE_TILED_K_SPLIT and tk.kernel_choice(384, 12928, 19456, 0, 0) == tk.CHOICE_TILED_K_SPLIT
     prev = tk.set_k_split(1)
     try:
         assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY   # no split
