@@ -412,7 +412,7 @@ int cu_count_of_device() {
 // 1024 x 2048 x 8192: 23.5 against 25.1); three slots beyond, where two workgroups may share a CU and one's waits are the
 // other's work (256 tiles: 1024 x 4096 x 4096 18.6 against 20.0, 512 x 8192 x 2048 11.9 against 13.6, 2048 x 2048 x 8192
 // 28.8 against 31.2) -- except with K from 6144 on while a CU is left over (512 x 6144 x 16384: six slots 46.0 against
-// 51.9, 64 x 28672 x 8192: 34.9 against 38.2, 1 x 27136 x 7680: 30.5 against 34.1; at K = 5120 three: 96 x 20480 x 5120 22.5 against 23.6), and three slots for K up to 2048, where filling six takes a good part of
+// 51.9, 64 x 28672 x 8192: 34.9 against 38.2, 1 x 27136 x 7680: 30.5 against 34.1; at K = 5120 three: 96 x 20480 x 5120 22.5 against 23.6; between the two six with one row of tiles, 1 x 25600 x 5632 21.2 against 24.6, 32 x 20608 x 5632 19.8 against 22.6, three with more, 512 x 7552 x 5504 23.9 against 24.9), and three slots for K up to 2048, where filling six takes a good part of
 // the 8 - 16 K-tiles there are (384 x 2048 x 1024: 6.3 against 7.2, 512 x 4096 x 2048: 10.2 against 11.1, 24 shapes of 384 -
 // 1024 rows x N = 2048 .. 6144 all 7 - 14 % ahead).  stages = 3 or 6 forces one (measurement).
 template <int FA, int FB, bool FUSED>
@@ -425,7 +425,7 @@ hipError_t launch(const GemmArgs& g, const BlockArgs& a, int tiles, int stages, 
     else gemm_block_kernel<FA, FB, OutBf16, 4, 4, FUSED><<<grid, 512, 0, s>>>(a);
     return hipGetLastError();
   }
-  if (stages == 0) stages = ((long)grid * 8 <= (long)cus * 5 && g.K > 2048) || ((g.K >= 6144 || a.nsplit > 1) && grid < cus) ? 6 : 3;
+  if (stages == 0) stages = ((long)grid * 8 <= (long)cus * 5 && g.K > 2048) || ((g.K >= 6144 || (g.K > 5120 && a.tiles_m == 1) || a.nsplit > 1) && grid < cus) ? 6 : 3;
   if (stages == 6) {
     if (f32) gemm_block_kernel<FA, FB, OutF32, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
     else gemm_block_kernel<FA, FB, OutBf16, 6, 2, FUSED><<<grid, 256, 0, s>>>(a);
@@ -493,6 +493,10 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
     // K up to 4096 against 12288 rows of B or more: from 65 rows on, from 24 with tiles on five eighths of the CUs
     // (24 x 28672 x 4096 21.1 us on the skinny kernel -> 18.5, 16 rows level)
     if (wide_short && (g.M > 64 || (g.M >= 24 && tiles * 8 >= (long)cus * 5))) return true;
+    // up to 64 rows with tiles on more than half the CUs and a K the skinny kernel cannot take (K % 512 != 0), against the
+    // tiled kernel: 8 x 21624 x 2688 13.3 us -> 11.4, 4 x 20224 x 13184 66.3 -> 60.2, 32 x 30976 x 7424 49.5 -> 44.3
+    // (96 - 128 rows the other way: 96 x 20736 x 12672 80.2 -> 83.9)
+    if (g.M <= 64 && tiles * 2 > cus && !gemm_skinny_supports(g)) return true;
     // from 32 rows on with tiles on more than half the CUs, up to K = 10240 (48 x 18816 x 4608 27.2 us on the skinny kernel
     // -> 18.9, 48 x 23280 x 9216 53.9 -> 51.9; beyond, 64 x 22784 x 10752 60.9 -> 62.8, 64 x 16640 x 16384 82.2 -> 89.3);
     // 32 rows, the skinny kernel's largest single row group, only up to K = 7168 (32 x 24576 x 8192 38.9 -> 43.3)
@@ -516,7 +520,8 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // (K beyond 16384: from 32 rows on as well, 32 x 16640 x 28672 102 us on the skinny kernel -> 91.7; with fewer rows
   // only up to K = 20480 with tiles on thirteen sixteenths of the CUs, 16 x 27392 x 19456 81.6 -> 70.9, 8 x 27904 x 18944
   // 76.2 -> 69.9; 16 x 23808 x 19968 level, 8 x 16640 x 28672 76.4 -> 79.6)
-  const bool many_tiles = g.M >= 32 ? tiles * 2 > cus && tiles <= cus && nkt <= 256
+  // (17 - 31 rows like 32, the skinny kernel handles them as 32: 24 x 19968 x 14848 57.9 us there -> 48.0)
+  const bool many_tiles = g.M > 16 ? tiles * 2 > cus && tiles <= cus && nkt <= 256
                                     : tiles * 8 >= (long)cus * 5 && tiles < cus && (nkt <= 128 || (nkt <= 160 && tiles * 16 >= (long)cus * 13));
   return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
 }

@@ -838,7 +838,9 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
 // tile-major and row-major B), in output tiles of 256 x 256: with K >= 12288 up to 64 tiles (128 from K = 24576 on, and
 // for up to 256 rows of A: 256 x 17920 x 23040 159 -> 114 us, 160 x 16768 x 17408 138 -> 110, 160 x 18304 x 13824 81 -> 60;
 // up to 1024 rows against a row-major B: 384 x 12928 x 19456 160 -> 121, 768 x 9216 x 17408 142 -> 127;
-// with 2048 rows it loses: 2048 x 5120 x 16384 122 -> 134):
+// with 2048 rows it loses: 2048 x 5120 x 16384 122 -> 134, and so it does with both operands tile-major beyond 104
+// tiles: 192 x 28672 x 12288 76.4 on the block kernel's 128 x 256 tiles -> 88.5; with a row-major A, which those tiles
+// do not take, it wins there as well, 160 x 28672 x 16384 116 -> 104, 160 x 27904 x 18432 130 -> 113):
 // 0.45 - 0.9 of the unsplit time, e.g. 256 x 8192 x 28672 108 -> 63 us, 128 x 4096 x 14336 46 -> 24 us, 1024 x 1024 x 16384
 // 60 -> 34 us; with 8192 <= K < 14336 up to 32 tiles where the skinny kernel is not an option (more than 128 rows of A, or
 // a tile-major A): 256 x 2048 x 8192 28.5 -> 21 us, 768 x 2048 x 8192 33 -> 27 us; and up to 64 tiles for 65 - 128 rows of A
@@ -852,19 +854,21 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
   int min_shares = 2;
   if (want == 0) {
     const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (g.M <= 256 || nkt >= 192 || (!g.layout_b && g.M <= 1024))))
+    const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (nkt >= 192 || (g.layout_b ? g.M <= 256 && (tiles256 <= 104 || !g.layout_a) : g.M <= 1024))))
                                  : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
                                                  // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
-                                                 (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192));
+                                                 (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192) ||
+                                                 // 33 - 64 rows against a wide row-major B, three shares a tile (below)
+                                                 (g.M > 32 && g.M <= 64 && !g.layout_a && !g.layout_b && g.N > 16384 && tiles256 * 3 <= cus));
     if (!pays) return 1;
     if (g.M <= 64 && !g.layout_a) {
       // up to 64 rows of a row-major A are the skinny kernel's, except more than 32 against tile-major weights with a
       // very long K, or a long K and a width that leaves the skinny kernel's last round of workgroups part empty
       // (with K < 24576 up to 104 tiles: beyond, two shares a tile lose to the block kernel's unsplit tiles,
       // 48 x 28672 x 12288 59.9 us -> 53.8; and against a row-major B of more than 16384 rows with three shares a tile or more:
-      // 64 x 16640 x 12288 64.9 us on the skinny kernel -> 53.3, 64 x 17024 x 21504 103 -> 84.5, two shares level)
+      // 64 x 16640 x 12288 64.9 us on the skinny kernel -> 53.3, 48 x 16640 x 9216 49.7 -> 39.4, 64 x 17024 x 21504 103 -> 84.5, two shares level)
       const bool ragged = g.N > 8192 && g.N % 8192 != 0 && tiles256 <= 104;
-      if (g.M > 32 && !g.layout_b && nkt >= 96 && g.N > 16384 && tiles256 * 3 <= cus) min_shares = 3;
+      if (g.M > 32 && !g.layout_b && nkt >= 64 && g.N > 16384 && tiles256 * 3 <= cus) min_shares = 3;
       else if (!(g.M > 32 && g.layout_b && tiles256 <= 128 && (nkt >= 192 || ragged))) return 1;
     }
   }
