@@ -380,7 +380,9 @@ def main():
     p.add_argument("--raster-sweep", action="store_true", help="only time the tiled kernel at 8192^3 (tile-major operands) over raster settings and print one JSON line")
     p.add_argument("--kernel", type=int, default=0, help="with --raster-sweep: kernel code to time as well (18 = the 4-wave schedule)")
     p.add_argument("--shape", type=int, nargs=3, metavar=("M", "N", "K"), default=None, help="with --raster-sweep: the problem shape (default 8192 8192 8192)")
-    p.add_argument("--sweep-settings", choices=["all", "default"], default="all", help="with --raster-sweep: all raster settings, or only the kernel's own (to compare schedules under a profiler)")
+    p.add_argument("--sweep-settings", choices=["all", "default", "ksplit-order"], default="all",
+                   help="with --raster-sweep: all raster settings, only the kernel's own (to compare schedules under a profiler), or the kernel's own and, as "
+                        "xcd_remap=2, a K split's workgroups in tile-by-tile order instead of share by share (for shapes that take a K split)")
     p.add_argument("--dispatch-sweep", choices=["small", "full"], default=None,
                    help="only compare the automatic kernel choice with every forced kernel / tile shape / K split over a grid of shapes and print one JSON line")
     p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the decode run with tile-major weights (used for profiling one layout of the skinny kernel)")
@@ -414,7 +416,7 @@ def main():
         kin = [(hk.tile_operand(ap), hk.tile_operand(bp), hk.tile_scales(asc, K), hk.tile_scales(bsc, K)) for ap, bp, asc, bsc in inputs]
         res = {}
         for rnd in range(2):  # two rounds over all settings: the second is reported (the first also warms the chip up)
-            for xcd in ((1, 0) if args.sweep_settings == "all" else (1,)):
+            for xcd in {"all": (1, 0), "default": (1,), "ksplit-order": (1, 2)}[args.sweep_settings]:
                 for gm in ((1, 2, 4, 8, 16, 32) if args.sweep_settings == "all" else (4,)):
                     assert L.mxfp6_probe_raster(gm, xcd) == 0
                     _, ms = timed_loop(hk, torch, kin, C, args.steps, args.warmup, 1, 1)

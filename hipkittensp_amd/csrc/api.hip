@@ -546,7 +546,7 @@ int mxfp6_probe_choice(int M, int N, int K, int layouts) {
 
 int mxfp6_probe_raster(int group_m, int xcd_remap) {
   if (group_m < 0 || group_m > 4096) return MXFP6_EINVAL_SHAPE;
-  g_raster_group_m = group_m, g_raster_no_xcd = xcd_remap ? 0 : 1;
+  g_raster_group_m = group_m, g_raster_no_xcd = xcd_remap == 2 ? 2 : xcd_remap ? 0 : 1;
   return MXFP6_OK;
 }
 

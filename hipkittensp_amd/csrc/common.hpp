@@ -125,6 +125,19 @@ __host__ __device__ __forceinline__ int tile_order(int bid, int tiles_m, int til
   return (first + in % gsz) | (in / gsz) << 16;
 }
 
+// K split between workgroups: position of workgroup `bid` (of `total` = tiles x shares) in share-major order, share s of
+// tile i at s * tiles + i.  The hardware deals workgroups to the eight XCDs round-robin; this hands XCD x the x-th
+// eighth of that order, so that with eight shares or more an XCD's workgroups all work on the same K range: they pull
+// that eighth of A and of B through the XCD's L2 once, where tile-by-tile order has every XCD fetch all of A for its
+// tiles (256 x 8192 x 28672, eight shares: 263 MB of L2 misses for 189 MB of operands; A alone is 5.5 MB against 4 MB
+// of L2).  With fewer shares an XCD gets part of one share's tiles, the same volume as before.  A bijection on
+// [0, total) when total % 8 == 0; the identity otherwise, with the remap switched off (xcd_remap 0) or with xcd_remap 2
+// (measurement: tile-by-tile order, XCDs dealt by tile_order).
+__host__ __device__ __forceinline__ bool ksplit_by_share(int total, int xcd_remap) { return xcd_remap == 1 && (total & 7) == 0; }
+__host__ __device__ __forceinline__ int ksplit_order(int bid, int total, int xcd_remap) {
+  return ksplit_by_share(total, xcd_remap) ? (bid & 7) * (total >> 3) + (bid >> 3) : bid;
+}
+
 // Byte offset, inside a tile-major operand, of byte `b` (0 .. 3K/4) of row `row`; nkt = K / 128.
 // Tiles are 32 rows x 96 bytes in the kernels' LDS image order (16-byte pieces, pairs swapped in
 // rows with bit 3 set).

@@ -74,14 +74,17 @@ __global__ __launch_bounds__(2 * WN * 64, STAGES <= 3 ? 2 : WN / 2) void gemm_bl
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MXFP6_LDS uint8_t*)smem;
   const int K = args.K, layout_a = args.layout_a, layout_b = args.layout_b;
   const int rowbytes = K / 4 * 3, sbytes = K / 32, nkt_all = K / kBK, nk4_all = (nkt_all + 3) / 4;  // tile-major scales: one 512-byte chunk per 32 rows and group of four K-tiles, the last one padded
-  // K split: workgroup b takes share b / tiles of tile b % tiles -- the same number of whole groups of four K-tiles for
-  // every share, the last one what is left of K (at least one K-tile: the launcher sees to that) -- and leaves its fp32
-  // sums in matrix `share` of args.C, then a workspace of nsplit matrices [M, N] (ksplit_reduce_kernel adds them up)
-  const int ntiles = args.tiles_m * args.tiles_n, share = blockIdx.x / ntiles;
+  // K split: workgroup b takes share l / tiles of tile l % tiles, l = ksplit_order(b) -- the same number of whole groups
+  // of four K-tiles for every share, the last one what is left of K (at least one K-tile: the launcher sees to that) --
+  // and leaves its fp32 sums in matrix `share` of args.C, then a workspace of nsplit matrices [M, N]
+  // (ksplit_reduce_kernel adds them up)
+  const int ntiles = args.tiles_m * args.tiles_n;
+  const bool by_share = args.nsplit > 1 && ksplit_by_share(ntiles * args.nsplit, args.xcd_remap);  // the XCDs are dealt by ksplit_order, not by tile_order
+  const int order = args.nsplit > 1 ? ksplit_order(blockIdx.x, ntiles * args.nsplit, args.xcd_remap) : blockIdx.x, share = order / ntiles;
   const int share_groups = (nk4_all + args.nsplit - 1) / args.nsplit, kt0 = share * share_groups * 4;
   const int nkt = min(nkt_all - kt0, share_groups * 4), nk4 = (nkt + 3) / 4;
 
-  const int tile = tile_order(blockIdx.x - share * ntiles, args.tiles_m, args.tiles_n, args.group_m, args.xcd_remap);
+  const int tile = tile_order(order - share * ntiles, args.tiles_m, args.tiles_n, args.group_m, by_share ? 0 : args.xcd_remap);
   if (tile < 0) return;  // never: the grid is the tile count times the shares
   const int pm = tile & 0xffff, pn = tile >> 16;
   const int rows_a = min(kBM, args.M - pm * kBM), rows_b = min(kBN, args.N - pn * kBN);
@@ -645,7 +648,7 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s) {
   const int bn = g.tile_cols == 256 ? 256 : 128, nsplit = g.ksplit > 1 ? g.ksplit : 1;
   BlockArgs a{g.A, g.B, g.As, g.Bs, nsplit > 1 ? (void*)g.ks_part : g.C, g.M, g.N, g.K, (g.M + kBM - 1) / kBM, (g.N + bn - 1) / bn, g.layout_a, g.layout_b,
-              g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, nsplit, g.ep};
+              g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap == 1 ? 0 : g.raster_no_xcd_remap == 2 ? 2 : 1, nsplit, g.ep};
   const int tiles = a.tiles_m * a.tiles_n, stages = g.tile_rows == 3 || g.tile_rows == 6 ? g.tile_rows : 0;
   hipError_t e;
   if (g.fmt_a == 2 && g.fmt_b == 2) e = launch<2, 2>(g, a, tiles, stages, s);

@@ -179,23 +179,32 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
   };
 
   // ---- workgroup -> output tiles: workgroup b works on tiles b, b + gridDim.x, ... of tile_order() (common.hpp)
-  // KSPLIT: workgroup b takes share b / tiles of tile b % tiles (shares of one tile start on the same XCD)
+  // KSPLIT: workgroup b takes share l / tiles of tile l % tiles, l = ksplit_order(b): share-major, an eighth of it per XCD
+  auto split_order_of = [&](int bid) __attribute__((always_inline)) {  // bid < tiles * nsplit
+    const auto g = fresh_args();
+    return ksplit_order(bid, g->tiles_m * g->tiles_n * g->nsplit, g->xcd_remap);
+  };
   auto tile_of = [&](int bid) __attribute__((always_inline)) {
     const auto g = fresh_args();
     if constexpr (KSPLIT) {
-      const int tiles = g->tiles_m * g->tiles_n;
-      return bid < tiles * g->nsplit ? tile_order(bid % tiles, g->tiles_m, g->tiles_n, g->group_m, g->xcd_remap) : -1;
+      const int tiles = g->tiles_m * g->tiles_n, total = tiles * g->nsplit;
+      if (bid >= total) return -1;
+      const bool by_share = ksplit_by_share(total, g->xcd_remap);  // the XCDs are dealt by ksplit_order, not by tile_order
+      return tile_order(split_order_of(bid) % tiles, g->tiles_m, g->tiles_n, g->group_m, by_share ? 0 : g->xcd_remap);
     }
     return tile_order(bid, g->tiles_m, g->tiles_n, g->group_m, g->xcd_remap);
   };
-  // first K-tile of workgroup-share bid (0 without the split)
-  auto ktile0_of = [&](int bid) __attribute__((always_inline)) {
+  // share of workgroup bid (a workgroup with a tile: bid < tiles * nsplit); 0 without the split
+  auto share_of = [&](int bid) __attribute__((always_inline)) {
     if constexpr (KSPLIT) {
       const auto g = fresh_args();
-      return bid / (g->tiles_m * g->tiles_n) * nkt;
+      const int tiles = g->tiles_m * g->tiles_n;
+      return bid < tiles * g->nsplit ? split_order_of(bid) / tiles : 0;
     }
     return 0;
   };
+  // first K-tile of workgroup-share bid (0 without the split)
+  auto ktile0_of = [&](int bid) __attribute__((always_inline)) { return share_of(bid) * nkt; };
   // Buffer resources of one output tile's operand rows (A and B) and of the scale rows this wave loads.  Edge
   // tiles: rows past M (or N) lie beyond the end of the resource and read as zeros.  tile < 0: resources of
   // length zero, loads through them fetch nothing.
@@ -615,7 +624,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     const int N = g->N, N2 = N * (int)sizeof(OutT);  // N2: bytes per row of C
     // the resource ends with the tile's last valid element
     OutT* cbase = (OutT*)g->C;
-    if constexpr (KSPLIT) cbase += (size_t)(bid_cur / (g->tiles_m * g->tiles_n)) * g->M * N;  // this share's matrix
+    if constexpr (KSPLIT) cbase += (size_t)share_of(bid_cur) * g->M * N;  // this share's matrix
     const __amdgpu_buffer_rsrc_t rC = make_rsrc(cbase + (size_t)(tile_cur & 0xffff) * kBM * N + (size_t)(tile_cur >> 16) * kBN,
                                                 (uint32_t)((rows_a - 1) * N + rows_b) * (uint32_t)sizeof(OutT));
     const int row_l = wm * (TM * 32) + r32;
@@ -918,7 +927,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const bool ksplit = g.ksplit > 1 && g.ks_part;
   const int shape = ksplit ? g.tile_rows | 256 << 16 : tiled_tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap ? 0 : 1, g.clock_stamps,
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap == 1 ? 0 : g.raster_no_xcd_remap == 2 ? 2 : 1, g.clock_stamps,
                         ksplit ? g.ksplit : 1};
   if (ksplit) {
     if constexpr (sizeof(typename Out::type) != 1) {

@@ -19,7 +19,7 @@ struct GemmArgs {
   Epilogue ep;                     // fused bias / scales / activation (all optional)
   uint8_t* C_scale = nullptr;      // fp6 output (tiled kernel): C is the packed operand [M, 3N/4], this its E8M0 bytes [M, N/32]
   int fmt_c = 0;                   // 2 / 3: format of the fp6 output; 0: bf16 / fp32 output
-  int raster_group_m = 0, raster_no_xcd_remap = 0;  // tiled kernel, measurement only: tile rows per raster group (0 = the default, 4), XCD remap off
+  int raster_group_m = 0, raster_no_xcd_remap = 0;  // tiled kernel, measurement only: tile rows per raster group (0 = the default, 4), XCD remap off (1), or on with a K split's workgroups in tile-by-tile order (2)
   int ablation = 0;  // tiled kernel, measurement only: leave out LDS reads (1), loads (2), MFMAs (4); results are then meaningless
   uint32_t* clock_stamps = nullptr;  // tiled kernel, measurement only: four words for workgroup 0's clock / real-time counters at start and end
   int no_alloc = 0;                // skinny kernel: the K split keeps its partial tiles in the library's static scratch array instead of an allocated workspace

@@ -315,7 +315,9 @@ int mxfp6_probe_tiled_clock(uint32_t *stamps);
  * The kernel uses group_m = 4 and xcd_remap = 1; mxfp6_probe_raster (per calling thread, measurement only; group_m = 0
  * restores the default) makes later launches use other values, for sweeps of the raster like the reference's
  * (analysis/paper_experiments/grid_micro/data_to_log.json; remap include/common/util.cuh:78-101).  A host-side pointer:
- * `order` holds tiles_m * tiles_n ints.
+ * `order` holds tiles_m * tiles_n ints.  Launches with a K split between workgroups order (tile, share) pairs share by
+ * share and hand each XCD an eighth of that order, so that an XCD's workgroups work on one K range of A and B;
+ * mxfp6_probe_raster(group_m, 2) keeps the tile remap but orders them tile by tile (measurement: the order before).
  */
 int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int *order);
 

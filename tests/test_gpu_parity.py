@@ -1167,6 +1167,27 @@ def test_measurement_probes_run_and_leave_results_alone(hk):
     assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("M,N,K,kernel,shares", [(256, 1024, 8192, 2, 8), (300, 520, 8192, 2, 4), (128, 1024, 8192, 22, 8), (200, 1032, 4096 + 128, 22, 3), (128, 384, 8192, 22, 8)])
+def test_k_split_order_of_workgroups_does_not_change_the_result(hk, M, N, K, kernel, shares):
+    """(tile, share) pairs share by share with an eighth of that order per XCD (the library's own), tile by tile, and with
+    no XCD remap at all: the same bits, and the oracle's values.  Workgroup counts that are multiples of eight take the
+    remap (32, 24, 64 and 24 here); the fourth shape's 18 tiles x 3 shares do not, and its K % 512 != 0 gives a shorter last share."""
+    tk, L = hk.tk_kernel, hk._lib.lib()
+    ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=M + K, kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, 2, 2, acc=np.float64)
+    prev = tk.set_k_split(shares)
+    got = {}
+    try:
+        for xcd in (1, 2, 0):
+            assert L.mxfp6_probe_raster(0, xcd) == 0
+            got[xcd] = gemm(hk, ap, bp, asc, bsc, kernel=kernel)
+    finally:
+        L.mxfp6_probe_raster(0, 1)
+        tk.set_k_split(prev)
+    check(got[1], ref, 2, 2, ap, asc, bp, bsc)
+    assert np.array_equal(got[1], got[2]) and np.array_equal(got[1], got[0])
+
+
 # ------------------------------------------------------------------ full-size configurations
 def _sampled_check(hk, ap, asc, bp, bsc, fa, fb, kernel, rng, ns=48, band=256):
     """Full-size check of one configuration: a whole band of `band` consecutive rows of the fp32 result (all N columns, so
