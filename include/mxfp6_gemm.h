@@ -373,7 +373,7 @@ const char *mxfp6_strerror(int code);
 
 /* ABI version of this header, major * 100 + minor, and what the loaded library reports: a caller built against this
  * header checks that the majors agree (entry points are only ever added within a major). */
-#define MXFP6_ABI_VERSION 119
+#define MXFP6_ABI_VERSION 120
 int mxfp6_abi_version(void);
 
 #ifdef __cplusplus

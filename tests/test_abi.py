@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert name in exported, f"{name} declared in the header but not exported"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 119
+    assert L.mxfp6_abi_version() == 120
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
