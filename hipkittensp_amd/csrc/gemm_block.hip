@@ -526,7 +526,8 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // (17 - 31 rows like 32, the skinny kernel handles them as 32: 24 x 19968 x 14848 57.9 us there -> 48.0)
   const bool many_tiles = g.M > 16 ? tiles * 2 > cus && tiles <= cus && nkt <= 256
                                     : tiles * 8 >= (long)cus * 5 && tiles < cus && (nkt <= 128 || (nkt <= 160 && tiles * 16 >= (long)cus * 13));
-  return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
+  // (K up to 1024 from 33 rows on: 64 x 10496 x 1024 7.4 us on the skinny kernel -> 5.9)
+  return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (nkt <= 8 && g.M > 32) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
 }
 
 // The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
@@ -602,7 +603,10 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
       // row-major weights (1 x 11264 x 32256 58 against 76)
       const long wgs = (g.N + 31) / 32;
       const bool last_round_thin = wgs > 256 && wgs % 256 >= 1 && wgs % 256 <= 160;
-      if (g.M <= 32 && !(last_round_thin && nkt >= 96 && g.layout_b)) return 1;
+      // (17 - 32 rows with K from 24576 on and more than one round of workgroups there: 32 x 14080 x 26112, last round
+      // seven tenths full, 64.4 us -> 55.5)
+      const bool long_k_32 = g.M > 16 && wgs > 256 && nkt >= 192;
+      if (g.M <= 32 && !(((last_round_thin && nkt >= 96) || long_k_32) && g.layout_b)) return 1;
       if (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)) return 1;
       // K below 8192: the skinny kernel's up to 96 rows (64 x 4096 x 6144 10.9 us against 12.9 split), up to 128 below 7168
       // (128 x 2048 x 7680 18.4 -> 15.7, 128 x 2048 x 6144 level)
