@@ -269,6 +269,14 @@ def test_kernel_choice_by_shape(hk):
     assert tk.kernel_choice(64, 16640, 12288, 0, 0) == tk.CHOICE_TILED_K_SPLIT and tk.k_split_plan(64, 16640, 12288, 0, 0, 0)[0] == 3
     assert tk.kernel_choice(64, 24576, 12288, 0, 0) != tk.CHOICE_TILED_K_SPLIT   # two shares a tile: level, not split
     assert tk.kernel_choice(160, 18304, 13824, 0, 1) == tk.CHOICE_TILED_K_SPLIT and tk.kernel_choice(384, 12928, 19456, 0, 0) == tk.CHOICE_TILED_K_SPLIT
+    # the mid-M kernel's estimate counts a thin last round of workgroups (268 of them here): not chosen
+    assert tk.kernel_choice(256, 8576, 10240, 0, 0) != tk.KERNEL_MID
+    # a K the skinny kernel cannot take against a row-major B, few rows, many tiles; 17 - 31 rows count as 32
+    assert tk.kernel_choice(8, 21624, 2688, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(24, 19968, 14848, 0, 1) == tk.KERNEL_BLOCK
+    # the tiled split beyond 104 tiles against a tile-major B: only with a row-major A (both tile-major, the 128 x 256 tiles win)
+    assert tk.kernel_choice(192, 28672, 12288, 1, 1) != tk.CHOICE_TILED_K_SPLIT and tk.kernel_choice(160, 28672, 16384, 0, 1) == tk.CHOICE_TILED_K_SPLIT
+    # 17 - 32 rows, a very long K, more than one round of the skinny kernel's workgroups; a very short K from 33 rows on
+    assert tk.kernel_choice(32, 14080, 26112, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 10496, 1024, 0, 1) == tk.KERNEL_BLOCK
     prev = tk.set_k_split(1)
     try:
         assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY   # no split
