@@ -844,7 +844,8 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
 // (the last three for measurement).  Returns the shares per tile (1: no split) and the tile height and workspace size
 // that go with them.
 // Where it pays (measured on MI355X against the best unsplit kernel over 360 shapes, M = 8 .. 2048, N = 1024 .. 57344,
-// tile-major and row-major B), in output tiles of 256 x 256: with K >= 12288 up to 64 tiles (128 from K = 24576 on, and
+// tile-major and row-major B), in output tiles of 256 x 256: with K >= 12288 up to 64 tiles (128 from K = 20480 on
+// -- 768 x 6912 x 20480 131 -> 118, 1536 x 4096 x 21504 127 -> 121 -- and
 // for up to 256 rows of A: 256 x 17920 x 23040 159 -> 114 us, 160 x 16768 x 17408 138 -> 110, 160 x 18304 x 13824 81 -> 60;
 // up to 1024 rows against a row-major B: 384 x 12928 x 19456 160 -> 121, 768 x 9216 x 17408 142 -> 127;
 // with 2048 rows it loses: 2048 x 5120 x 16384 122 -> 134, and so it does with both operands tile-major beyond 104
@@ -863,12 +864,18 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
   int min_shares = 2;
   if (want == 0) {
     const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (nkt >= 192 || (g.layout_b ? g.M <= 256 && (tiles256 <= 104 || !g.layout_a) : g.M <= 1024))))
+    // (K = 8192 .. 12287, a row-major B, more than 128 rows, 65 - 85 tiles -- more 128 x 128 tiles than CUs, so the block
+    // kernel is out -- and three shares a tile: 640 x 6800 x 10752 66.4 us -> 57.6, 768 x 6760 x 9216 60.3 -> 56.2; two
+    // shares lose, 768 x 6144 x 8192 51.6 -> 54.1, and so do three against a tile-major B, 512 x 10496 x 9216 49.3 -> 60.5)
+    const bool three_shares_mid_k = nkt >= 64 && nkt < 96 && !g.layout_b && g.M > 128 && tiles256 > 64 && tiles256 * 3 <= cus;
+    if (three_shares_mid_k) min_shares = 3;
+    const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (nkt >= 160 || (g.layout_b ? g.M <= 256 && (tiles256 <= 104 || !g.layout_a) : g.M <= 1024))))
                                  : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
                                                  // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
                                                  (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192) ||
                                                  // 33 - 64 rows against a wide row-major B, three shares a tile (below)
-                                                 (g.M > 32 && g.M <= 64 && !g.layout_a && !g.layout_b && g.N > 16384 && tiles256 * 3 <= cus));
+                                                 (g.M > 32 && g.M <= 64 && !g.layout_a && !g.layout_b && g.N > 16384 && tiles256 * 3 <= cus) ||
+                                                 three_shares_mid_k);
     if (!pays) return 1;
     if (g.M <= 64 && !g.layout_a) {
       // up to 64 rows of a row-major A are the skinny kernel's, except more than 32 against tile-major weights with a
