@@ -480,7 +480,11 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // (up to twice as many tiles as CUs for K up to 2048 with both operands tile-major: two workgroups share a CU, one round;
   // us, the 128 x 256 tiles -> this: 4096 x 2048 x 1024 16.4 -> 12.9, 1024 x 8192 x 1024 17.1 -> 13.3, 2048 x 4096 x 2048 20.6 -> 18.9)
   const bool short_k = nkt <= 16 && g.layout_a && g.layout_b;
-  if (cus <= 0 || tiles > (short_k ? 2 * cus : cus)) return false;
+  // (K up to 640 against a row-major B: any number of tiles -- the launch is prologue and epilogue, and two of these
+  // workgroups share a CU; us, tiled kernel -> this: 640 x 24192 x 640 23.9 -> 19.9, 2048 x 26624 x 640 68.4 -> 57.0,
+  // 768 x 5888 x 512 10.5 -> 9.3, 256 x 25216 x 512 11.8 -> 10.7)
+  const bool very_short_k = nkt <= 5 && !g.layout_b;
+  if (cus <= 0 || (!very_short_k && tiles > (short_k ? 2 * cus : cus))) return false;
   // tiles on more than half the CUs (three quarters with a row-major B), K up to 16384
   const bool fills = nkt <= 128 && (g.layout_b ? tiles * 16 >= (long)cus * 9 : tiles * 4 >= (long)cus * 3);
   // ... or on a quarter of them, K up to 8192 (a row-major A: up to 256 rows of it)
@@ -566,7 +570,11 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   // 18944 = 37 groups and 22016 = 43 do not)
   int tiled_rows = 0;
   size_t tiled_part = 0;
-  const bool tiled_splits = want == 0 && gemm_tiled_supports(g) && tiled_ksplit_plan(g, 0, &tiled_rows, &tiled_part) > 1;
+  // ... and its workgroups fill half the CUs at least: K = 31744 = 62 groups gives it two shares a tile only
+  // (320 x 4224 x 31744: 68 workgroups, 94.6 us, against 72.4 with two shares of this kernel's 99 tiles;
+  // 256 x 5888 x 29696, both tile-major: 86.2 against 59.5)
+  const int tiled_shares = want == 0 && gemm_tiled_supports(g) ? tiled_ksplit_plan(g, 0, &tiled_rows, &tiled_part) : 1;
+  const bool tiled_splits = tiled_shares > 1 && (long)((g.M + tiled_rows - 1) / tiled_rows) * ((g.N + 255) / 256) * tiled_shares * 2 >= cus;
   if (want == 0) {
     // two launches for a K below 5120 lose (96 x 8192 x 2048: 11 -> 14 us; 256 x 2048 x 4096 13.3 -> 13.9); from there on
     // they pay (us, unsplit -> split: 256 x 2048 x 5120, A row-major 19.8 -> 16.9, both row-major 24.1 -> 18.2;
@@ -625,7 +633,8 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   // 128 x 2048 x 28672 22.0 / 23.2; with 8 tiles 14 shares are ahead: 128 x 1024 x 28672 19.0 against 21.0; with a
   // row-major B as well: 128 x 2048 x 28672 24.5 against 25.6, 512 x 384 x 28672 21.9 against 25.4).
   int best = 1;
-  const int first = want != 0 ? 16 : nkt == 64 && tiles <= 12 ? 8 : nkt > 128 && tiles >= 12 && g.layout_b ? 28 : 16;
+  // (up to 64 rows the partial sums are small and shorter shares win: 48 x 2304 x 18304, 18 tiles, 5 shares 17.2 us, 9 shares 14.4)
+  const int first = want != 0 ? 16 : nkt == 64 && tiles <= 12 ? 8 : nkt > 128 && tiles >= 12 && g.layout_b && g.M > 64 ? 28 : 16;
   for (int min_tiles = first; min_tiles >= 8 && best <= 1; min_tiles = min_tiles > 16 ? 16 : min_tiles - 8) {
     for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
       // every share the same number of whole groups, the last share what is left (at least one group)
@@ -641,7 +650,8 @@ int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
   // K from 24576 on, more than 32 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
   // streams B faster (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7; up
   // to 32 tiles this kernel's: 128 x 2048 x 28672 22.0 against 26.0, 128 x 4096 x 28672 30.4 against 34.1)
-  if (want == 0 && nkt >= 192 && tiles > 32 && tiles * best * 4 < (long)cus * 3 && tiled_splits) return 1;
+  // (from K = 20480 on: 128 x 11008 x 23040, 86 tiles, two shares here 71.5 us, five shares of the tiled kernel's 43 tiles 56.9)
+  if (want == 0 && nkt >= 160 && tiles > 32 && tiles * best * 4 < (long)cus * 3 && tiled_splits) return 1;
   *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
   return best;
 }
