@@ -157,7 +157,8 @@ def test_block_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
 
 
 @pytest.mark.parametrize("M,N,K,la,lb", [(256, 8192, 2048, 1, 1), (192, 4096, 4096, 0, 1), (512, 3072, 3072, 0, 0), (1024, 2048, 8192, 1, 1), (96, 16384, 1024, 0, 1),
-                                         (384, 6144, 4096, 1, 0), (2048, 4096, 1024, 1, 1)])  # the last: 512 tiles, two workgroups per CU
+                                         (384, 6144, 4096, 1, 0), (2048, 4096, 1024, 1, 1),   # 512 tiles, two workgroups per CU
+                                         (640, 12808, 640, 0, 0), (24, 12032, 768, 0, 0)])    # a very short K against a row-major B: 505 tiles with a ragged last column; few rows
 def test_block_kernel_is_chosen_and_matches_the_tiled_kernel(hk, M, N, K, la, lb):
     """Shapes on which the automatic path takes the block kernel (its tiles do not outnumber the CUs, K of moderate length):
     the result is the forced block kernel's bit for bit (the two agree on the dispatch), equals the 8-wave tiled kernel's
@@ -275,6 +276,9 @@ def test_kernel_choice_by_shape(hk):
     assert tk.kernel_choice(8, 21624, 2688, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(24, 19968, 14848, 0, 1) == tk.KERNEL_BLOCK
     # the tiled split beyond 104 tiles against a tile-major B: only with a row-major A (both tile-major, the 128 x 256 tiles win)
     assert tk.kernel_choice(192, 28672, 12288, 1, 1) != tk.CHOICE_TILED_K_SPLIT and tk.kernel_choice(160, 28672, 16384, 0, 1) == tk.CHOICE_TILED_K_SPLIT
+    # a long K goes to the tiled split only where its workgroups fill half the CUs (K = 31744 leaves it two shares a tile)
+    assert tk.kernel_choice(320, 4224, 31744, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 11008, 23040, 0, 1) == tk.CHOICE_TILED_K_SPLIT
+    assert tk.kernel_choice(2048, 26624, 640, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(2048, 26624, 640, 0, 1) != tk.KERNEL_BLOCK   # K up to 640, B row-major: any number of tiles
     # 17 - 32 rows, a very long K, more than one round of the skinny kernel's workgroups; a very short K from 33 rows on
     assert tk.kernel_choice(32, 14080, 26112, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 10496, 1024, 0, 1) == tk.KERNEL_BLOCK
     prev = tk.set_k_split(1)
