@@ -483,7 +483,10 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
   // (K up to 640 against a row-major B: any number of tiles -- the launch is prologue and epilogue, and two of these
   // workgroups share a CU; us, tiled kernel -> this: 640 x 24192 x 640 23.9 -> 19.9, 2048 x 26624 x 640 68.4 -> 57.0,
   // 768 x 5888 x 512 10.5 -> 9.3, 256 x 25216 x 512 11.8 -> 10.7)
-  const bool very_short_k = nkt <= 5 && !g.layout_b;
+  // (not where the tiled kernel's 256 x 256 tiles make one round on three quarters of the CUs or more: 512 x 28928 x 512,
+  // 226 of them, 15.1 us there against 18.0 here)
+  const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
+  const bool very_short_k = nkt <= 5 && !g.layout_b && !(tiles256 <= cus && tiles256 * 4 >= (long)cus * 3);
   if (cus <= 0 || (!very_short_k && tiles > (short_k ? 2 * cus : cus))) return false;
   // tiles on more than half the CUs (three quarters with a row-major B), K up to 16384
   const bool fills = nkt <= 128 && (g.layout_b ? tiles * 16 >= (long)cus * 9 : tiles * 4 >= (long)cus * 3);
@@ -496,7 +499,8 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
     if ((g.M > 256 && nkt <= 40) || (g.M > 128 && fills)) return true;
     // K up to 2048 wherever the skinny kernel does not come first: 160 x 9216 x 1536 10.1 us on the tiled kernel -> 8.9,
     // 96 x 4840 x 1792 9.9 -> 8.1, 24 x 12032 x 768 6.9 -> 6.1
-    if (nkt <= 16 && (g.M > 128 || !gemm_skinny_preferred(g))) return true;
+    // (up to K = 3072 likewise: 96 x 2952 x 2432 11.5 -> 8.8, 96 x 21352 x 2304 14.1 -> 13.2, 96 x 18048 x 3072 16.4 -> 15.2)
+    if (nkt <= 24 && (g.M > 128 || !gemm_skinny_preferred(g))) return true;
     // K up to 4096 against 12288 rows of B or more: from 65 rows on, from 24 with tiles on five eighths of the CUs
     // (24 x 28672 x 4096 21.1 us on the skinny kernel -> 18.5, 16 rows level)
     if (wide_short && (g.M > 64 || (g.M >= 24 && tiles * 8 >= (long)cus * 5))) return true;

@@ -868,11 +868,12 @@ int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes
     // kernel is out -- and three shares a tile: 640 x 6800 x 10752 66.4 us -> 57.6, 768 x 6760 x 9216 60.3 -> 56.2; two
     // shares lose, 768 x 6144 x 8192 51.6 -> 54.1, and so do three against a tile-major B, 512 x 10496 x 9216 49.3 -> 60.5)
     const bool three_shares_mid_k = nkt >= 64 && nkt < 96 && !g.layout_b && g.M > 128 && tiles256 > 64 && tiles256 * 3 <= cus;
-    if (three_shares_mid_k) min_shares = 3;
+    if (three_shares_mid_k || (nkt < 96 && tiles256 > 64 && g.M > 64 && g.M <= 128)) min_shares = 3;
     const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (nkt >= 160 || (g.layout_b ? g.M <= 256 && (tiles256 <= 104 || !g.layout_a) : g.M <= 1024))))
                                  : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
                                                  // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
-                                                 (tiles256 <= 64 && g.M > 64 && g.M <= 128 && g.N > 8192) ||
+                                                 // (up to 85 tiles with three shares a tile: 96 x 19584 x 10752 55.3 us on the block kernel -> 44.8)
+                                                 (tiles256 * 3 <= cus && g.M > 64 && g.M <= 128 && g.N > 8192) ||
                                                  // 33 - 64 rows against a wide row-major B, three shares a tile (below)
                                                  (g.M > 32 && g.M <= 64 && !g.layout_a && !g.layout_b && g.N > 16384 && tiles256 * 3 <= cus) ||
                                                  three_shares_mid_k);
