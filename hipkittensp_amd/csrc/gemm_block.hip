@@ -500,14 +500,16 @@ bool gemm_block_preferred(const GemmArgs& g, bool first) {
     // K up to 2048 wherever the skinny kernel does not come first: 160 x 9216 x 1536 10.1 us on the tiled kernel -> 8.9,
     // 96 x 4840 x 1792 9.9 -> 8.1, 24 x 12032 x 768 6.9 -> 6.1
     // (up to K = 3072 likewise: 96 x 2952 x 2432 11.5 -> 8.8, 96 x 21352 x 2304 14.1 -> 13.2, 96 x 18048 x 3072 16.4 -> 15.2)
-    if (nkt <= 24 && (g.M > 128 || !gemm_skinny_preferred(g))) return true;
+    // (and K up to 1024 from 33 rows on, as against a tile-major B: 48 x 15872 x 512 6.8 us on the skinny kernel -> 6.0)
+    if ((nkt <= 24 && (g.M > 128 || !gemm_skinny_preferred(g))) || (nkt <= 8 && g.M > 32)) return true;
     // K up to 4096 against 12288 rows of B or more: from 65 rows on, from 24 with tiles on five eighths of the CUs
     // (24 x 28672 x 4096 21.1 us on the skinny kernel -> 18.5, 16 rows level)
     if (wide_short && (g.M > 64 || (g.M >= 24 && tiles * 8 >= (long)cus * 5))) return true;
-    // up to 64 rows with tiles on more than half the CUs and a K the skinny kernel cannot take (K % 512 != 0), against the
+    // up to 64 rows and a K the skinny kernel cannot take (K % 512 != 0), against the
     // tiled kernel: 8 x 21624 x 2688 13.3 us -> 11.4, 4 x 20224 x 13184 66.3 -> 60.2, 32 x 30976 x 7424 49.5 -> 44.3
     // (96 - 128 rows the other way: 96 x 20736 x 12672 80.2 -> 83.9)
-    if (g.M <= 64 && tiles * 2 > cus && !gemm_skinny_supports(g)) return true;
+    // (with few tiles as well: 24 x 6992 x 4864, 55 tiles, 19.3 -> 16.9)
+    if (g.M <= 64 && !gemm_skinny_supports(g)) return true;
     // from 32 rows on with tiles on more than half the CUs, up to K = 10240 (48 x 18816 x 4608 27.2 us on the skinny kernel
     // -> 18.9, 48 x 23280 x 9216 53.9 -> 51.9; beyond, 64 x 22784 x 10752 60.9 -> 62.8, 64 x 16640 x 16384 82.2 -> 89.3);
     // 32 rows, the skinny kernel's largest single row group, only up to K = 7168 (32 x 24576 x 8192 38.9 -> 43.3)
