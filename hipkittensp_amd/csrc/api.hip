@@ -27,43 +27,75 @@ thread_local int g_ksplit = 0;                                // mxfp6_probe_ksp
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
 // demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
+// A workspace that was handed out while its stream was being captured is recorded in a graph: it is `pinned`, and a
+// pinned block is never freed again -- when it must grow, or at mxfp6_release_workspaces(), it is retired (kept
+// allocated until the process ends), so that replays of the graph never write into memory somebody else owns.
 struct StreamWs {
   uint8_t* p = nullptr;
   size_t bytes = 0;
+  bool pinned = false;
+  uint64_t used = 0;  // g_sws_clock at the last use (least recently used entries make room when the table is full)
 };
 std::mutex g_sws_mutex;
 // Held while a call enqueues the kernels that write and then read a stream's workspace (pre-pass + GEMM, GEMM + quantiser):
 // two threads that launch into the same stream must not interleave those, or one's GEMM would read the other's copies.
 std::recursive_mutex g_sws_launch_mutex;
 std::map<std::tuple<int, hipStream_t, int>, StreamWs> g_sws;
+uint64_t g_sws_clock = 0;
 constexpr size_t kStreamWsMax = 128;
 
-// kind 0: pre-pass copies, kind 1: fp32 result of mxfp6_gemm_fused_fp6, kind 2: partial sums of the tiled kernel's K split.
-// nullptr: no workspace (capture, limit, out of memory).
-uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes) {
+bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // unknown: behave as if it were
+  }
+  return cap != hipStreamCaptureStatusNone;
+}
+
+// kind 0: pre-pass copies, kind 1: fp32 result of mxfp6_gemm_fused_fp6, kind 2: partial sums of a K split, kind 3: arrival
+// counters of the ring kernel's K split (zeroed when allocated; the kernels leave them zero).
+// nullptr: no workspace (capture without one, table full of pinned entries, out of memory).
+uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes, bool zeroed = false) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> lock(g_sws_mutex);
+  const bool capturing = stream_is_capturing(s);
   auto it = g_sws.find({dev, s, kind});
-  if (it != g_sws.end() && it->second.bytes >= bytes) return it->second.p;
-  // never allocate into a stream that is being captured: the caller replays the graph with its own memory plan
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return nullptr;
+  if (it != g_sws.end() && it->second.bytes >= bytes) {
+    it->second.used = ++g_sws_clock;
+    if (capturing) it->second.pinned = true;  // a graph now holds this pointer
+    return it->second.p;
   }
-  if (it == g_sws.end() && g_sws.size() >= kStreamWsMax) return nullptr;
+  // never allocate into a stream that is being captured: the caller replays the graph with its own memory plan
+  if (capturing) return nullptr;
+  if (it == g_sws.end() && g_sws.size() >= kStreamWsMax) {
+    // full: the least recently used workspace that no graph holds goes back to the allocator, in its own stream's order
+    auto victim = g_sws.end();
+    for (auto j = g_sws.begin(); j != g_sws.end(); ++j)
+      if (!j->second.pinned && (victim == g_sws.end() || j->second.used < victim->second.used)) victim = j;
+    if (victim == g_sws.end()) return nullptr;
+    int cur = dev;
+    (void)hipSetDevice(std::get<0>(victim->first));
+    if (hipFreeAsync(victim->second.p, std::get<1>(victim->first)) != hipSuccess) (void)hipGetLastError();  // a destroyed stream: the block is lost to the pool
+    (void)hipSetDevice(cur);
+    g_sws.erase(victim);
+  }
   uint8_t* p = nullptr;
   const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
   if (hipMallocAsync((void**)&p, want, s) != hipSuccess || !p) {
     (void)hipGetLastError();
     return nullptr;
   }
+  if (zeroed && mxfp6::launch_fill_zero(p, want, s) != hipSuccess) {
+    (void)hipFreeAsync(p, s);
+    return nullptr;
+  }
   if (it != g_sws.end()) {
-    (void)hipFreeAsync(it->second.p, s);
-    it->second = {p, want};
+    if (!it->second.pinned) (void)hipFreeAsync(it->second.p, s);  // a pinned block stays allocated: a graph may replay into it
+    it->second = {p, want, false, ++g_sws_clock};
   } else {
-    g_sws[{dev, s, kind}] = {p, want};
+    g_sws[{dev, s, kind}] = {p, want, false, ++g_sws_clock};
   }
   return p;
 }
@@ -89,6 +121,16 @@ void plan_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
   uint8_t* pp = stream_workspace(s, 2, part);
   if (!pp) return;
   g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp);
+}
+// The ring kernel's K split, likewise.
+void plan_ring_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
+  size_t part = 0, counters = 0;
+  const int shares = mxfp6::ring_ksplit_plan(g, g_ksplit, &part, &counters);
+  if (shares <= 1) return;
+  uint8_t* pp = stream_workspace(s, 2, part);
+  uint8_t* pc = pp ? stream_workspace(s, 3, counters * sizeof(int), true) : nullptr;
+  if (!pc) return;
+  g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp), g.ks_counters = reinterpret_cast<int*>(pc);
 }
 bool launch_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
   std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
@@ -144,6 +186,7 @@ hipError_t release_stream_workspaces() {
   (void)hipGetDevice(&cur);
   hipError_t first = hipSuccess;
   for (auto& kv : g_sws) {
+    if (kv.second.pinned) continue;  // recorded in a graph: stays allocated until the process ends
     (void)hipSetDevice(std::get<0>(kv.first));
     const hipError_t e = hipFreeAsync(kv.second.p, std::get<1>(kv.first));
     if (e != hipSuccess && first == hipSuccess) first = e;
@@ -275,6 +318,11 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (K != 0 && force == 18) {
     if (!mxfp6::gemm_tiled4_supports(g)) return MXFP6_EINVAL_SHAPE;
     e = mxfp6::launch_gemm_tiled4(g, s);
+  } else if (K != 0 && force == 28) {
+    if (!mxfp6::gemm_ring_supports(g)) return MXFP6_EINVAL_SHAPE;
+    std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
+    plan_ring_ksplit(g, s);
+    e = mxfp6::launch_gemm_ring(g, s);
   } else if (K != 0 && ((force >= 22 && force <= 24) || force == 26)) {
     if (!mxfp6::gemm_block_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.tile_rows = force == 23 ? 3 : force == 24 ? 6 : 0, g.tile_cols = force == 26 ? 256 : 0;
@@ -362,14 +410,7 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
   }
   std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);
   float* tmp = reinterpret_cast<float*>(stream_workspace(s, 1, (size_t)M * N * 4));
-  if (!tmp) {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-      (void)hipGetLastError();
-      return (int)hipErrorStreamCaptureUnsupported;
-    }
-    return (int)hipErrorOutOfMemory;
-  }
+  if (!tmp) return stream_is_capturing(s) ? (int)hipErrorStreamCaptureUnsupported : MXFP6_EWORKSPACE;
   rc = gemm_common(A, B, As, Bs, tmp, M, N, K, fmt_a, fmt_b, true, layout_a, layout_b, stream, ep);
   if (rc == MXFP6_OK) {
     const hipError_t e = mxfp6::launch_quantize(tmp, 0, (uint8_t*)C_packed, (uint8_t*)C_scale, M, N, fmt_c, MXFP6_LAYOUT_ROW, s);
@@ -407,7 +448,7 @@ int mxfp6_set_relayout(int on) {
 }
 
 int mxfp6_set_kernel(int which) {
-  if (which < 0 || which > 26 || which == 25) return MXFP6_EINVAL_KERNEL;
+  if (which < 0 || which > 28 || which == 25 || which == 27) return MXFP6_EINVAL_KERNEL;
   const int prev = g_force;
   g_force = which;
   return prev;
@@ -633,6 +674,7 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_EINVAL_EPILOGUE: return "mxfp6: activation must be 0 (none), 1 (relu), 2 (gelu) or 3 (silu)";
     case MXFP6_ESCRATCH: return "mxfp6: the K split of this call needs more than the static scratch memory holds (256 partial tiles: rows of C tiles times nsplit)";
     case MXFP6_EINVAL_KERNEL: return "mxfp6: unknown kernel code";
+    case MXFP6_EWORKSPACE: return "mxfp6: no workspace for this call (the allocator refused, or every workspace slot is held by a captured graph)";
     case MXFP6_EBLOB: return "mxfp6: not a tile-major operand blob this library reads (magic, version, format, layout or shape)";
     default: break;
   }

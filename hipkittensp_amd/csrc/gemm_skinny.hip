@@ -333,6 +333,7 @@ constexpr size_t kWsMax = 64;
 struct SplitWs {
   float* part = nullptr;
   int* cnt = nullptr;
+  bool pinned = false;  // handed out while its stream was being captured: a graph holds the pointers, the block is never freed
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, SplitWs> g_ws;
@@ -346,14 +347,15 @@ SplitWs split_workspace(hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return {};
   std::lock_guard<std::mutex> lock(g_ws_mutex);
-  auto it = g_ws.find({dev, s});
-  if (it != g_ws.end()) return it->second;
-  if (g_ws.size() >= kWsMax) return {};
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return {};
+  const bool capturing = hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+  if (capturing) (void)hipGetLastError();
+  auto it = g_ws.find({dev, s});
+  if (it != g_ws.end()) {
+    if (capturing) it->second.pinned = true;
+    return it->second;
   }
+  if (g_ws.size() >= kWsMax || capturing) return {};
   SplitWs w;
   uint8_t* base = nullptr;
   if (hipMallocAsync((void**)&base, (size_t)kWsSlots * 4096 + kWsTiles * sizeof(int), s) != hipSuccess || !base) {
@@ -402,6 +404,7 @@ hipError_t release_split_workspaces() {
   (void)hipGetDevice(&cur);
   hipError_t first = hipSuccess;
   for (auto& kv : g_ws) {
+    if (kv.second.pinned) continue;  // recorded in a graph: stays allocated until the process ends
     // stream-ordered: the memory goes back once the work queued on that stream so far has finished with it
     (void)hipSetDevice(kv.first.first);
     const hipError_t e = hipFreeAsync(kv.second.part, kv.first.second);

@@ -25,7 +25,8 @@ struct GemmArgs {
   int no_alloc = 0;                // skinny kernel: the K split keeps its partial tiles in the library's static scratch array instead of an allocated workspace
   int force_split = 0;             // skinny kernel, M <= 32: split K between this many workgroups (1, 2, 4, 8); 0 = by shape
   int ksplit = 0;                  // tiled kernel: workgroups that share an output tile (from tiled_ksplit_plan, which also gives tile_rows); needs ks_part
-  float* ks_part = nullptr;        // ... their partial sums: ksplit matrices [M, N] of floats
+  float* ks_part = nullptr;        // ... their partial sums: ksplit matrices [M, N] of floats (ring kernel: partial tiles)
+  int* ks_counters = nullptr;      // ring kernel's K split: one arrival counter per tile of C, zero between launches
 };
 
 // the LDS-staged kernels fetch operands and scales 16 bytes per lane: all four tensors must be 16-byte aligned
@@ -47,6 +48,9 @@ bool gemm_block_wide_preferred(const GemmArgs& g);  // its 128 x 256 tiles (eigh
 int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes);  // K split of the block kernel for this problem: shares per tile (1 = none)
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s);
 hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s);  // sums g.ksplit partial matrices at g.ks_part into g.C, with the epilogue
+bool gemm_ring_supports(const GemmArgs& g);  // batched decode: private streams of B per wave, A through a flag-guarded ring (no barrier per K-tile)
+int ring_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes, size_t* counters);  // its K split for this problem (want: 0 = by shape, 1 = none, n = n shares): shares (1 = none), bytes of partial tiles, arrival counters
+hipError_t launch_gemm_ring(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
 bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
 double tiled_estimate_us(const GemmArgs& g, int rows, int cols = 256);  // estimated time of the tiled kernel with tiles of rows x cols

@@ -48,6 +48,7 @@ KERNEL_SKINNY_64_SPLIT = (20, 21)  # the same with the K range split between 2 /
 KERNEL_BLOCK = 22  # 128 x 128 tiles, four waves in step: one barrier per K-tile, fragments double-buffered in registers
 KERNEL_BLOCK_3SLOTS, KERNEL_BLOCK_6SLOTS = 23, 24  # the same with its operand ring forced to three / six slots
 KERNEL_BLOCK_WIDE = 26  # the block kernel with tiles of 128 x 256 and eight waves
+KERNEL_RING = 28  # batched decode: a private stream of B per wave, A through a flag-guarded ring, no barrier per K-tile
 KERNEL_TILED_4WAVE = 18  # the 4-wave interleaved schedule of the tiled kernel (measurement: never chosen automatically)
 
 

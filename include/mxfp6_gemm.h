@@ -70,6 +70,7 @@ extern "C" {
 #define MXFP6_ESCRATCH (-8)     /* mxfp6_gemm_noalloc: the requested K split does not fit the static scratch memory */
 #define MXFP6_EINVAL_KERNEL (-9) /* mxfp6_set_kernel: unknown kernel code                        */
 #define MXFP6_EBLOB (-10)       /* not a tile-major operand blob of a version this library reads */
+#define MXFP6_EWORKSPACE (-11)  /* a call that cannot run without a workspace did not get one (allocator, or all slots held by graphs) */
 
 /* Activations of mxfp6_gemm_fused. */
 #define MXFP6_ACT_NONE 0

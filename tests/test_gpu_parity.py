@@ -141,6 +141,36 @@ def test_tiled_kernel_vs_oracle(hk, M, N, K, fa, fb, kernel):
     assert np.array_equal(cb, o.f32_to_bf16_bits(got))
 
 
+# ------------------------------------------------------------------ ring kernel (batched decode: private streams of B, flag-guarded ring of A)
+@pytest.mark.parametrize("M,N,K", [(1, 128, 512), (16, 256, 2048), (17, 1000, 1024), (32, 132, 3584), (33, 520, 2048), (64, 4096, 4096), (64, 8192, 8192),
+                                   (100, 264, 1536), (128, 384, 8192), (129, 132, 1024), (200, 520, 28672), (256, 1024, 4096), (300, 4, 512)])
+@pytest.mark.parametrize("fa,fb", [(2, 2), (3, 2), (2, 3), (3, 3)])
+def test_ring_kernel_vs_oracle(hk, M, N, K, fa, fb):
+    """One, two and four row-tiles of A per workgroup, several blocks of rows, ragged M and N, every K split the shape allows
+    (shares 1, the automatic number, 3): against the fp64 oracle; bf16 output = RNE of the fp32 output; the sum over the
+    shares is taken in share order whoever arrives last, so a call repeated gives the same bits."""
+    tk = hk.tk_kernel
+    ap, asc, bp, bsc = operands(M, N, K, fa, fb, seed=M * 7 + N + K, kind_a="laplace" if fa == 3 else "normal", kind_b="weights")
+    ref = o.gemm_ref(ap, bp, asc, bsc, fa, fb, acc=np.float64)
+    for shares in (1, 0, 3):
+        prev = tk.set_k_split(shares)
+        try:
+            got = gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=tk.KERNEL_RING)
+            check(got, ref, fa, fb, ap, asc, bp, bsc)
+            assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, out="bf16", kernel=tk.KERNEL_RING), o.f32_to_bf16_bits(got))
+            assert np.array_equal(gemm(hk, ap, bp, asc, bsc, fa, fb, kernel=tk.KERNEL_RING), got)
+        finally:
+            tk.set_k_split(prev)
+
+
+def test_ring_kernel_rejects_what_it_cannot_take(hk):
+    tk = hk.tk_kernel
+    for M, N, K in ((64, 128, 640), (64, 130, 1024), (64, 128, 256)):   # K % 512 != 0, N % 4 != 0, K < 512
+        ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=3)
+        with pytest.raises(RuntimeError):
+            gemm(hk, ap, bp, asc, bsc, kernel=tk.KERNEL_RING)
+
+
 # ------------------------------------------------------------------ block kernel (128 x 128 tiles, four waves in step)
 @pytest.mark.parametrize("M,N,K", [(128, 128, 512), (256, 384, 1024), (512, 256, 2560), (300, 264, 1536), (129, 8, 512), (100, 1000, 1024), (33, 520, 2048),
                                    (1, 128, 512), (640, 1024, 4096), (256, 256, 128), (300, 264, 640), (100, 520, 1152), (257, 8, 384)])  # edge tiles too; K % 512 != 0: a last group of fewer than four K-tiles
@@ -650,7 +680,7 @@ def test_tile_operand_matches_format_definition(hk, rows, K):
 
 
 @pytest.mark.parametrize("kernel,M,N,K", [(23, 256, 512, 1024), (24, 320, 544, 1536), (26, 256, 1024, 1024), (1, 64, 96, 256), (1, 32, 64, 1152), (2, 256, 512, 640), (2, 512, 256, 2048), (2, 288, 96, 384), (2, 320, 544, 1152),
-                                          (18, 256, 512, 640), (18, 320, 544, 1152), (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128)])
+                                          (18, 256, 512, 640), (18, 320, 544, 1152), (3, 16, 128, 1024), (3, 7, 64, 512), (3, 32, 96, 2560), (4, 64, 96, 2048), (4, 160, 64, 1024), (4, 64, 8320, 1024), (4, 192, 4160, 1024), (0, 32, 32, 128), (28, 32, 128, 1024), (28, 64, 544, 4096), (28, 160, 256, 2048)])
 @pytest.mark.parametrize("la,lb", [(0, 1), (1, 0), (1, 1)])
 def test_tile_major_operands_give_identical_results(hk, kernel, M, N, K, la, lb):
     if kernel in (3, 4) and la == 1:
@@ -821,7 +851,7 @@ def test_tiled_kernel_walk_matches_generic_kernel_bit_for_bit(hk, M, N, K, la, l
 # ------------------------------------------------------------------ fused epilogue
 @pytest.mark.parametrize("kernel,M,N,K", [(1, 70, 40, 96), (3, 16, 96, 1024), (3, 32, 100, 512), (4, 64, 72, 1024), (4, 200, 136, 2048),
                                           (5, 300, 264, 640), (6, 300, 264, 640), (5, 1024, 4104, 512), (6, 2304, 8200, 512),
-                                          (17, 300, 264, 640), (17, 1024, 4104, 512), (23, 300, 264, 1024), (24, 200, 136, 2048), (26, 300, 520, 1024)])
+                                          (17, 300, 264, 640), (17, 1024, 4104, 512), (23, 300, 264, 1024), (24, 200, 136, 2048), (26, 300, 520, 1024), (28, 48, 264, 1024), (28, 200, 136, 8192)])
 @pytest.mark.parametrize("activation", [None, "relu", "gelu", "silu"])
 def test_fused_epilogue_every_kernel(hk, kernel, M, N, K, activation):
     """act(acc * row_scale * col_scale + bias) fused into each kernel's epilogue (the last two shapes have more tiles than
@@ -943,6 +973,51 @@ def test_graph_capture_replays_match_eager(hk):
         assert torch.equal(Cg, eager[rep % 2]), f"replay {rep}"
         hk.dispatch_micro(a, b, asc, bsc, torch.empty_like(Cg))   # eager work between replays
         torch.cuda.synchronize()
+
+
+def test_graph_survives_a_regrown_and_a_released_workspace(hk):
+    """A graph that recorded a K split holds the stream's workspace pointer.  A larger eager split on the same stream makes
+    the library take a larger workspace, and mxfp6_release_workspaces() gives workspaces back: neither may free the block
+    the graph replays into (it stays allocated until the process ends), so every replay still reproduces the eager result."""
+    from hipkittensp_amd import _lib
+    tk = hk.tk_kernel
+    small, large = (128, 512, 8192), (256, 2048, 16384)
+    assert tk.kernel_choice(*small, 0, 1) in (tk.CHOICE_BLOCK_K_SPLIT, tk.CHOICE_TILED_K_SPLIT)
+    assert tk.kernel_choice(*large, 0, 1) in (tk.CHOICE_BLOCK_K_SPLIT, tk.CHOICE_TILED_K_SPLIT)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+
+    def make(M, N, K):
+        a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+        b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2, layout=1)
+        return a, b, asc, bsc
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        a, b, asc, bsc = make(*small)
+        eager = torch.empty(small[0], small[1], dtype=torch.bfloat16, device="cuda")
+        hk.dispatch_micro(a, b, asc, bsc, eager, layout_b=1)      # warm-up on the capture stream: the workspace exists
+        side.synchronize()
+        Cg = torch.zeros_like(eager)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            hk.dispatch_micro(a, b, asc, bsc, Cg, layout_b=1)
+        la, lb, las, lbs = make(*large)
+        Cl = torch.empty(large[0], large[1], dtype=torch.bfloat16, device="cuda")
+        for rep in range(3):
+            if rep == 1:
+                hk.dispatch_micro(la, lb, las, lbs, Cl, layout_b=1)   # a larger split: the stream's workspace grows
+            if rep == 2:
+                assert _lib.lib().mxfp6_release_workspaces() == 0
+                junk = [torch.full((1 << 22,), 7.0, device="cuda") for _ in range(8)]   # whatever the pool hands out next is overwritten
+            Cg.zero_()
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(Cg, eager), f"replay {rep}"
+            hk.dispatch_micro(la, lb, las, lbs, Cl, layout_b=1)
+            side.synchronize()
+        del junk
+    torch.cuda.synchronize()
 
 
 # ------------------------------------------------------------------ torch.library operator
