@@ -1,7 +1,12 @@
-"""Builds hipkittensp_amd/libmxfp6_gemm.so (gfx950 only) from csrc/*.hip with hipcc.
+"""Builds hipkittensp_amd/libmxfp6_gemm.so (gfx950 only) from csrc/*.hip with hipcc, and libmxfp6_probes.so beside it.
 
     python -m hipkittensp_amd.build            # rebuild everything
-The library is built in-tree; nothing is installed.  No GPU is needed to build.
+The libraries are built in-tree; nothing is installed.  No GPU is needed to build.
+
+libmxfp6_gemm.so is the operator (include/mxfp6_gemm.h).  libmxfp6_probes.so is the measurement build
+(include/mxfp6_probes.h): the same objects, except that the C ABI and the e2m3 x e2m3 instantiations of the LDS-tiled
+kernel are compiled a second time with -DMXFP6_PROBES (probe entry points, ablation builds, clock stamps) and the probe
+kernels (csrc/probes.hip) are added.  bench.py loads it for its ceilings and ablations; the operator never does.
 """
 from __future__ import annotations
 
@@ -14,12 +19,16 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmxfp6_gemm.so")
-SOURCES = ["api.hip", "gemm_generic.hip", "gemm_tiled.hip", "gemm_tiled4.hip", "gemm_block.hip", "gemm_mid.hip", "gemm_skinny.hip", "gemm_ring.hip", "quantize.hip", "probes.hip"]
+PROBES_LIB = os.path.join(HERE, "libmxfp6_probes.so")
+SOURCES = ["api.hip", "gemm_generic.hip", "gemm_tiled.hip", "gemm_tiled4.hip", "gemm_block.hip", "gemm_mid.hip", "gemm_skinny.hip", "gemm_ring.hip", "quantize.hip"]
 # (source, object name, extra flags).  gemm_tiled.hip gives five objects: its host-side part, and the kernel
 # instantiations of each pair of operand formats (the bulk of the build time; they compile side by side).
 UNITS = [(src, src.replace(".hip", ""), []) for src in SOURCES] + [
     ("gemm_tiled.hip", f"gemm_tiled_fmt{fmt}", [f"-DMXFP6_TILED_FMT={fmt}"]) for fmt in (22, 23, 32, 33)
 ]
+# what the measurement build compiles again (or in addition), with -DMXFP6_PROBES
+PROBE_UNITS = [("api.hip", "api_probes", ["-DMXFP6_PROBES"]), ("gemm_tiled.hip", "gemm_tiled_fmt22_probes", ["-DMXFP6_TILED_FMT=22", "-DMXFP6_PROBES"]),
+               ("probes.hip", "probes", ["-DMXFP6_PROBES"])]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-std=c++20", "-O3", "-fPIC", "-fvisibility=hidden",
@@ -43,15 +52,19 @@ def _compile(unit) -> str:
 def build(verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     # the units that take longest first
-    order = sorted(UNITS, key=lambda u: (u[1] != "gemm_block", not u[1].startswith("gemm_tiled_fmt"), u[1] not in ("gemm_skinny", "gemm_mid")))
+    order = sorted(UNITS + PROBE_UNITS, key=lambda u: (u[1] != "gemm_block", not u[1].startswith("gemm_tiled_fmt"), u[1] not in ("gemm_skinny", "gemm_mid")))
     with cf.ThreadPoolExecutor(max_workers=min(8, len(order))) as ex:
-        objs = list(ex.map(_compile, order))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode:
-        raise RuntimeError(f"link failed:\n{r.stderr}")
-    if verbose:
-        print(f"built {LIB}")
+        objs = dict(zip((u[1] for u in order), ex.map(_compile, order)))
+    product = [objs[u[1]] for u in UNITS]
+    swapped = {"api": "api_probes", "gemm_tiled_fmt22": "gemm_tiled_fmt22_probes"}
+    probes = [objs[swapped.get(u[1], u[1])] for u in UNITS] + [objs["probes"]]
+    for lib, members in ((LIB, product), (PROBES_LIB, probes)):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode:
+            raise RuntimeError(f"link failed:\n{r.stderr}")
+        if verbose:
+            print(f"built {lib}")
     return LIB
 
 

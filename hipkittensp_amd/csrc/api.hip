@@ -5,6 +5,9 @@
 // on shapes the tiled kernel does not run, the partial sums of the tiled and the block kernel's K split (plan_ksplit,
 // plan_block_ksplit: one workspace, shared), and the K-split workspace of the skinny kernel (gemm_skinny.hip).  mxfp6_gemm_noalloc allocates nothing.
 #include "../../include/mxfp6_gemm.h"
+#ifdef MXFP6_PROBES
+#include "../../include/mxfp6_probes.h"
+#endif
 
 #include <map>
 #include <mutex>
@@ -19,11 +22,16 @@ namespace {
 // other threads' calls run.
 thread_local int g_force = 0;
 thread_local int g_relayout = 1;
+thread_local int g_allow_e3m2_pair = 0;  // mxfp6_allow_e3m2_pair
+thread_local int g_ksplit = 0;  // mxfp6_set_k_split: 0 = where it pays, -1 = wherever possible, 1 = never, n = n shares per output tile
+#ifdef MXFP6_PROBES  // the measurement build (libmxfp6_probes.so, include/mxfp6_probes.h)
 thread_local uint32_t* g_clock_stamps = nullptr;  // mxfp6_probe_tiled_clock
 thread_local int g_raster_group_m = 0, g_raster_no_xcd = 0;  // mxfp6_probe_raster
 thread_local int g_ablation = 0;                              // mxfp6_probe_tiled_ablation
 thread_local int g_block = 1;                                 // mxfp6_probe_block: 0 keeps the block kernel out of the automatic choice
-thread_local int g_ksplit = 0;                                // mxfp6_probe_ksplit: 0 = where it pays, -1 = wherever possible, 1 = never, n = n shares per output tile
+#else
+constexpr int g_block = 1;
+#endif
 
 // Workspaces kept per (device, stream, kind): launches on one stream are ordered, so they can share one; it grows on
 // demand (old one returned to the allocator in stream order) and lives until mxfp6_release_workspaces().
@@ -123,14 +131,16 @@ void plan_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
   g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp);
 }
 // The ring kernel's K split, likewise.
-void plan_ring_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
+// returns false when the plan is a split whose workspace is not to be had (capture, allocator): then nothing is set
+bool plan_ring_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
   size_t part = 0, counters = 0;
   const int shares = mxfp6::ring_ksplit_plan(g, g_ksplit, &part, &counters);
-  if (shares <= 1) return;
+  if (shares <= 1) return true;
   uint8_t* pp = stream_workspace(s, 2, part);
   uint8_t* pc = pp ? stream_workspace(s, 3, counters * sizeof(int), true) : nullptr;
-  if (!pc) return;
+  if (!pc) return false;
   g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp), g.ks_counters = reinterpret_cast<int*>(pc);
+  return true;
 }
 bool launch_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
   std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
@@ -153,10 +163,13 @@ bool launch_tiled_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
 // The kernel the automatic path takes for a call, by shape, layouts and alignment alone (codes of mxfp6_set_kernel; the
 // tiled kernel with its K split: kChoiceTiledKsplit).  allow_ksplit = false: what it takes when the split's workspace is
 // not to be had (a stream that is being captured, the allocator's refusal).
-constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceMid = 4, kChoiceBlock = 22, kChoiceTiledKsplit = 25, kChoiceBlockWide = 26, kChoiceBlockKsplit = 27;
+constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceMid = 4, kChoiceBlock = 22, kChoiceTiledKsplit = 25, kChoiceBlockWide = 26, kChoiceBlockKsplit = 27, kChoiceRing = 28;
 int auto_choice(const mxfp6::GemmArgs& g, int force_split, bool allow_ksplit) {
   if (g.K == 0) return kChoiceGeneric;  // act(bias) everywhere: the generic kernel's K loop runs zero times
   const bool block = g_block && !force_split;  // the block kernel may be chosen
+  // weights streamed from HBM against a few dozen rows of A: private streams of B per wave (its K split needs no workspace to
+  // be correct: without one it runs unsplit, which the shapes it is chosen for would not survive, so only with one)
+  if (!force_split && allow_ksplit && g_ksplit != 1 && mxfp6::gemm_ring_preferred(g)) return kChoiceRing;
   // 128 x 128 tiles on at most half the CUs: the block kernel with its K split between workgroups
   if (block && allow_ksplit) {
     size_t part = 0;
@@ -216,17 +229,26 @@ int check_device() {
 // fewer rows.  The workspace is this stream's (stream_workspace: allocated once, kept).  Returns false when no
 // pre-pass pays or it cannot run (then the caller launches the row-major path).
 bool relayout_then_tiled(const mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
-  if (!g_relayout || g.no_alloc || g.layout_a || g.layout_b || g.K % 128) return false;
+  if (!g_relayout || g.no_alloc || (g.layout_a && g.layout_b) || g.K % 128) return false;
   const double tiles = (double)((g.M + 255) / 256) * ((g.N + 255) / 256);
   const double t_gemm_us = (tiles > 256 ? tiles / 256 : 1.0) * (g.K / 128) * 1.5;            // row-major tiled kernel
   auto cost_us = [&](int rows) { return (double)rows * g.K * 0.78125 * 2 / 4.9e6; };         // read + write at 4.9 TB/s
   // the operand with fewer rows first (it is the cheaper one to convert; the gain is the same)
   const bool a_first = g.M <= g.N;
   const int rows1 = a_first ? g.M : g.N, rows2 = a_first ? g.N : g.M;
-  // fixed costs: the allocation and the dependent launch in front of the GEMM (about 10 us measured on a 33 us GEMM), a
-  // second launch about 3 us
-  bool conv1 = rows1 % 32 == 0 && 0.15 * t_gemm_us > 10 + 1.5 * cost_us(rows1);
-  bool conv2 = rows2 % 32 == 0 && (conv1 ? 0.11 * t_gemm_us > 3 + 1.5 * cost_us(rows2) : 0.15 * t_gemm_us > 10 + 1.5 * cost_us(rows2));
+  bool conv1, conv2;
+  if (g.layout_a || g.layout_b) {
+    // one operand is tile-major already (prepared weights): the other one's copy is the second conversion of the two,
+    // worth about 11 % of the row-major GEMM, for one launch in front of it
+    const bool first_is_row = a_first ? !g.layout_a : !g.layout_b;
+    const int rows = first_is_row ? rows1 : rows2;
+    const bool conv = rows % 32 == 0 && 0.11 * t_gemm_us > 6 + cost_us(rows);
+    conv1 = first_is_row && conv, conv2 = !first_is_row && conv;
+  } else {
+    // fixed costs: the dependent launch in front of the GEMM (about 10 us measured on a 33 us GEMM), a second operand about 3 us
+    conv1 = rows1 % 32 == 0 && 0.15 * t_gemm_us > 10 + 1.5 * cost_us(rows1);
+    conv2 = rows2 % 32 == 0 && (conv1 ? 0.11 * t_gemm_us > 3 + 1.5 * cost_us(rows2) : 0.15 * t_gemm_us > 10 + 1.5 * cost_us(rows2));
+  }
   if (!conv1 && !conv2) return false;
   const bool conv_a = a_first ? conv1 : conv2, conv_b = a_first ? conv2 : conv1;
   auto bytes_of = [&](int rows) { return (((size_t)rows * (g.K / 4 * 3) + 255) & ~(size_t)255) + (((size_t)rows * ((g.K + 511) / 512) * 16 + 255) & ~(size_t)255); };
@@ -259,6 +281,9 @@ int check_gemm_args(const void* A, const void* B, const void* As, const void* Bs
   if (M < 0 || N < 0 || K < 0 || K % 32 != 0) return MXFP6_EINVAL_SHAPE;
   if ((fmt_a != MXFP6_FMT_E2M3 && fmt_a != MXFP6_FMT_E3M2) || (fmt_b != MXFP6_FMT_E2M3 && fmt_b != MXFP6_FMT_E3M2))
     return MXFP6_EINVAL_FMT;
+  // e3m2 on both sides is the one pair whose accumulators can miss the library's accuracy bar (the MFMA's own sum is
+  // inexact there): only for callers that have said they accept that
+  if (fmt_a == MXFP6_FMT_E3M2 && fmt_b == MXFP6_FMT_E3M2 && !g_allow_e3m2_pair) return MXFP6_EACCURACY;
   if ((layout_a != MXFP6_LAYOUT_ROW && layout_a != MXFP6_LAYOUT_TILE) || (layout_b != MXFP6_LAYOUT_ROW && layout_b != MXFP6_LAYOUT_TILE))
     return MXFP6_EINVAL_LAYOUT;
   if ((layout_a == MXFP6_LAYOUT_TILE && (M % 32 || K % 128)) || (layout_b == MXFP6_LAYOUT_TILE && (N % 32 || K % 128)))
@@ -293,9 +318,11 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C, M, N, K, fmt_a, fmt_b, f32out, layout_a, layout_b};
   g.ep = ep;
   g.no_alloc = no_alloc, g.force_split = force_split;
+#ifdef MXFP6_PROBES
   g.clock_stamps = g_clock_stamps;
   g.raster_group_m = g_raster_group_m, g.raster_no_xcd_remap = g_raster_no_xcd;
   g.ablation = g_ablation;
+#endif
   const int force = no_alloc ? 0 : g_force;  // the entry point that allocates nothing takes no override
   hipError_t e;
   if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
@@ -321,7 +348,7 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   } else if (K != 0 && force == 28) {
     if (!mxfp6::gemm_ring_supports(g)) return MXFP6_EINVAL_SHAPE;
     std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
-    plan_ring_ksplit(g, s);
+    (void)plan_ring_ksplit(g, s);  // without a workspace: unsplit
     e = mxfp6::launch_gemm_ring(g, s);
   } else if (K != 0 && ((force >= 22 && force <= 24) || force == 26)) {
     if (!mxfp6::gemm_block_supports(g)) return MXFP6_EINVAL_SHAPE;
@@ -334,6 +361,11 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     // the split needs this stream's workspace: without it, what the shape gets otherwise
     if (choice == kChoiceBlockKsplit && !launch_block_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
     if (choice == kChoiceTiledKsplit && !launch_tiled_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
+    if (choice == kChoiceRing) {
+      std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
+      if (plan_ring_ksplit(g, s)) e = mxfp6::launch_gemm_ring(g, s);
+      else choice = auto_choice(g, force_split, false);  // no workspace (capture, allocator): what the shape gets otherwise
+    }
     if (choice == kChoiceBlock) {
       e = mxfp6::launch_gemm_block(g, s);
     } else if (choice == kChoiceBlockWide) {
@@ -538,18 +570,39 @@ int mxfp6_blob_unpack(const void* blob, void* packed, void* scales, int rows, in
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
+int mxfp6_allow_e3m2_pair(int allow) {
+  const int prev = g_allow_e3m2_pair;
+  g_allow_e3m2_pair = allow ? 1 : 0;
+  return prev;
+}
+
+int mxfp6_set_k_split(int shares) {
+  if (shares < -1 || shares > 64) return MXFP6_EINVAL_SHAPE;
+  const int prev = g_ksplit;
+  g_ksplit = shares;
+  return prev;
+}
+
+int mxfp6_kernel_choice(int M, int N, int K, int layouts) {
+  if (M <= 0 || N <= 0 || K < 0 || K % 32) return MXFP6_EINVAL_SHAPE;
+  if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;
+  const int layout_a = layouts & 1, layout_b = layouts >> 1;
+  if ((layout_a && (M % 32 || K % 128)) || (layout_b && (N % 32 || K % 128))) return MXFP6_EINVAL_SHAPE;
+  const int rc = check_device();
+  if (rc) return rc;
+  // aligned stand-ins for the pointers: the choice looks at their alignment only
+  const uint8_t* p = reinterpret_cast<const uint8_t*>((uintptr_t)4096);
+  mxfp6::GemmArgs g{p, p, p, p, const_cast<uint8_t*>(p), M, N, K, 2, 2, false, layout_a, layout_b};
+  return auto_choice(g, 0, true);
+}
+
+#ifdef MXFP6_PROBES  // ---- measurement entry points (include/mxfp6_probes.h)
 int mxfp6_probe_tiled_ablation(int mask) {
   if (mask < 0 || mask > 6 || mask == 5) return MXFP6_EINVAL_SHAPE;
   g_ablation = mask;
   return MXFP6_OK;
 }
 
-int mxfp6_probe_ksplit(int shares) {
-  if (shares < -1 || shares > 64) return MXFP6_EINVAL_SHAPE;
-  const int prev = g_ksplit;
-  g_ksplit = shares;
-  return prev;
-}
 
 int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int* tile_rows) {
   if (M <= 0 || N <= 0 || K <= 0 || shares < -1 || shares > 64) return MXFP6_EINVAL_SHAPE;
@@ -572,18 +625,6 @@ int mxfp6_probe_block(int enable) {
   return prev;
 }
 
-int mxfp6_probe_choice(int M, int N, int K, int layouts) {
-  if (M <= 0 || N <= 0 || K < 0 || K % 32) return MXFP6_EINVAL_SHAPE;
-  if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;
-  const int layout_a = layouts & 1, layout_b = layouts >> 1;
-  if ((layout_a && (M % 32 || K % 128)) || (layout_b && (N % 32 || K % 128))) return MXFP6_EINVAL_SHAPE;
-  const int rc = check_device();
-  if (rc) return rc;
-  // aligned stand-ins for the pointers: the choice looks at their alignment only
-  const uint8_t* p = reinterpret_cast<const uint8_t*>((uintptr_t)4096);
-  mxfp6::GemmArgs g{p, p, p, p, const_cast<uint8_t*>(p), M, N, K, 2, 2, false, layout_a, layout_b};
-  return auto_choice(g, 0, true);
-}
 
 int mxfp6_probe_raster(int group_m, int xcd_remap) {
   if (group_m < 0 || group_m > 4096) return MXFP6_EINVAL_SHAPE;
@@ -630,6 +671,8 @@ int mxfp6_probe_stream(const void* buf, size_t bytes, int workgroups, int waves,
   return e == hipSuccess ? MXFP6_OK : (int)e;
 }
 
+#endif  // MXFP6_PROBES
+
 int mxfp6_release_workspaces(void) {
   const hipError_t a = release_stream_workspaces();
   const hipError_t b = mxfp6::release_split_workspaces();
@@ -675,6 +718,7 @@ const char* mxfp6_strerror(int code) {
     case MXFP6_ESCRATCH: return "mxfp6: the K split of this call needs more than the static scratch memory holds (256 partial tiles: rows of C tiles times nsplit)";
     case MXFP6_EINVAL_KERNEL: return "mxfp6: unknown kernel code";
     case MXFP6_EWORKSPACE: return "mxfp6: no workspace for this call (the allocator refused, or every workspace slot is held by a captured graph)";
+    case MXFP6_EACCURACY: return "mxfp6: e3m2 x e3m2 can exceed the 2e-3 accuracy bar (up to 1e-4 of sum |a||b| per output); call mxfp6_allow_e3m2_pair(1) to accept that";
     case MXFP6_EBLOB: return "mxfp6: not a tile-major operand blob this library reads (magic, version, format, layout or shape)";
     default: break;
   }

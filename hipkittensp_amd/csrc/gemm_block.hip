@@ -20,6 +20,7 @@
 //           reads of K-tile k+1, MFMAs of K-tile k, wait for the LDS reads and for every load older than this step's,
 //           barrier.  A load has two steps to land.
 #include "kernels.hpp"
+#include "loader.hpp"
 
 namespace mxfp6 {
 namespace {
@@ -29,24 +30,6 @@ constexpr int kATile = kBM * 96;  // bytes of A's tile in a ring slot
 constexpr int kScA = kBM * 16;    // bytes of A's scales for four K-tiles
 constexpr int kGroupM = 8;        // tile rows per raster group
 
-// one direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff, the hardware writes them at LDS
-// address lds_base + 16 * lane; the VMEM counter is managed by hand (wait_vmcnt)
-__device__ __forceinline__ void dma16(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void barrier() {
-  __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_barrier" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
 
 struct BlockArgs {
   const uint8_t *A, *B, *As, *Bs;

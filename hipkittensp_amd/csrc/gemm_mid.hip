@@ -22,6 +22,7 @@
 // analysis/bf16_gemm/mi325x/kernel_8192.cpp:24-32).
 #include "common.hpp"
 #include "kernels.hpp"
+#include "loader.hpp"
 
 namespace mxfp6 {
 
@@ -30,12 +31,6 @@ namespace {
 constexpr int kBSlot = 24576;  // bytes of one B slot: BN rows x GB K-tiles
 constexpr int kASlots = 3;
 
-__device__ __forceinline__ void dma16_md(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory");
-}
 // wait until at most n of this wave's loads are outstanding (n is one of the sums that occur: see the callers)
 #define MXFP6_MID_WAIT(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
 __device__ __forceinline__ void wait_loads_md(int n) {
@@ -147,10 +142,10 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
     for (int i = 0; i < kScJobs; i++) {
       if (a_wave && (i & 3) == wave) {
         if (i < TMW) {
-          dma16_md(rAs, dst + i * 1024, i * 32 * sbytes + voff_srow, __builtin_amdgcn_readfirstlane(sg * 32));
+          dma16(rAs, dst + i * 1024, i * 32 * sbytes + voff_srow, __builtin_amdgcn_readfirstlane(sg * 32));
         } else {
           const int q = i - TMW;
-          dma16_md(rBs, dst + BM * 32 + q * 1024, layout_b ? q * nk4 * 512 + lane * 16 : q * 32 * sbytes + voff_srow,
+          dma16(rBs, dst + BM * 32 + q * 1024, layout_b ? q * nk4 * 512 + lane * 16 : q * 32 * sbytes + voff_srow,
                    __builtin_amdgcn_readfirstlane(sg * sstep_b));
         }
       }
@@ -160,13 +155,13 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint8_t* __restrict
     const uint32_t dst = lds0 + (j % kASlots) * kASlot + lw * (NA * 1024);
     const int so = __builtin_amdgcn_readfirstlane(j * GA * 96);
 #pragma unroll
-    for (int i = 0; i < NA; i++) dma16_md(rA, dst + i * 1024, voff_ld[i], so);
+    for (int i = 0; i < NA; i++) dma16(rA, dst + i * 1024, voff_ld[i], so);
   };
   auto issue_b = [&](int b) __attribute__((always_inline)) {  // B slot b: K-tiles GB b .. GB b + GB-1 (B-waves)
     const uint32_t dst = lds0 + kBRing + (b % KB) * kBSlot + lw * (NB * 1024);
     const int so = __builtin_amdgcn_readfirstlane(b * bstep);
 #pragma unroll
-    for (int i = 0; i < NB; i++) dma16_md(rB, dst + i * 1024, voff_ld[i], so);
+    for (int i = 0; i < NB; i++) dma16(rB, dst + i * 1024, voff_ld[i], so);
   };
 
   v16f acc;

@@ -32,6 +32,7 @@
 #include <utility>
 #include "common.hpp"
 #include "kernels.hpp"
+#include "loader.hpp"
 
 // Scratch memory of mxfp6_gemm_noalloc: kScratchSlots partial tiles of 4 KB (one per (tile, split) pair of a K split) followed by
 // kScratchTiles arrival counters.  In host code this name is only a handle for hipGetSymbolAddress; kernels get the device
@@ -40,18 +41,6 @@ constexpr int kScratchSlots = 256, kScratchTiles = 256;
 static __device__ __align__(256) unsigned char scratch[kScratchSlots * 4096 + kScratchTiles * 4];
 
 namespace mxfp6 {
-
-namespace {
-
-__device__ __forceinline__ void dma16_sk(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory");
-}
-__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-}  // namespace
 
 // AR = rows of A staged (16, 32 or 64: one or two 32-row accumulator tiles per wave); NW = waves per workgroup;
 // BR = rows of B per workgroup (32; 16 so that a narrow N still gives every CU a workgroup: the MFMA's other 16
@@ -153,19 +142,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     const int sg = KT == 4 ? chunk : chunk >> 1;  // the scales come in groups of four K-tiles
     const int sosb = __builtin_amdgcn_readfirstlane(layout_b ? sg * 512 : sg * 16);
     const uint32_t pb = __builtin_amdgcn_readfirstlane(par);
-    dma16_sk(rBs, buf + kScOff + pb * 1024, voff_bs, sosb);
+    dma16(rBs, buf + kScOff + pb * 1024, voff_bs, sosb);
     const int sob = __builtin_amdgcn_readfirstlane(layout_b ? chunk * (KT * 3072) : chunk * kRow);
 #pragma unroll
-    for (int i = 0; i < NBL; i++) dma16_sk(rB, buf + pb * kBBuf + i * 1024, voff_b[i], sob);
+    for (int i = 0; i < NBL; i++) dma16(rB, buf + pb * kBBuf + i * 1024, voff_b[i], sob);
   };
   auto issue_a = [&](int chunk) __attribute__((always_inline)) {
     const int sg = KT == 4 ? chunk : chunk >> 1;
     const int sos = __builtin_amdgcn_readfirstlane(sg * 16);
 #pragma unroll
-    for (int i = 0; i < NAS; i++) dma16_sk(rAs, buf + kAScOff + i * 1024, voff_as + i * 64 * sbytes, sos);
+    for (int i = 0; i < NAS; i++) dma16(rAs, buf + kAScOff + i * 1024, voff_as + i * 64 * sbytes, sos);
     const int so = __builtin_amdgcn_readfirstlane(chunk * kRow);
 #pragma unroll
-    for (int i = 0; i < NAL; i++) dma16_sk(rA, buf + kAOff + i * 1024, voff_a[i], so);
+    for (int i = 0; i < NAL; i++) dma16(rA, buf + kAOff + i * 1024, voff_a[i], so);
   };
 
   v16f acc[TT];
@@ -182,7 +171,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
     if (DB == 2 && mine > 1) issue_b(c0 + wave + NW, 1);
     for (int j = 0; j < mine; j++) {
       if (DB == 2 && j + 1 < mine) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NBL + 1) : "memory");
-      else wait_all_loads();
+      else wait_vmcnt<0>();
       const int par = DB == 2 ? j & 1 : 0;
       const uint8_t* bufb = bufp + par * kBBuf;
       v4i sc_b[TB], sc_a[TA];
@@ -254,7 +243,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const uint8_t* __r
       for (int w = 0; w < NW; w++) t += part[w * (TT * 1024) + idx];
       __hip_atomic_store(mine_ws + idx, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    wait_all_loads();  // stores count there too: the partial tile has arrived before the counter moves
+    wait_vmcnt<0>();  // stores count there too: the partial tile has arrived before the counter moves
     __syncthreads();
     int* flag = reinterpret_cast<int*>(smem + NW * TT * 16 * 64 * 4);  // behind the partial tiles
     if (tid == 0) *flag = __hip_atomic_fetch_add(ws_cnt + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1;

@@ -54,6 +54,7 @@
 // instantiations are what takes the time to compile, and four objects compile side by side.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "loader.hpp"
 
 namespace mxfp6 {
 
@@ -104,26 +105,8 @@ struct Shape {
   static_assert(kLdsBytes <= 163840, "LDS budget");
 };
 
-// One direct-to-LDS load: every lane fetches 16 bytes at rsrc.base + voff + soff and the hardware
-// writes them at LDS address lds_base + 16 * lane.  Issued from inline assembly so that the VMEM
-// counter is managed by hand: the ring keeps two K-tiles in flight across barriers, which the
-// compiler's automatic waits would serialise.  M0 is used by nothing else in this kernel.
-__device__ __forceinline__ void dma16(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void barrier() {
-  __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_barrier" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
+// (dma16, wait_vmcnt, wait_lds_reads, barrier: loader.hpp.  The ring keeps two K-tiles in flight across barriers, which
+// the compiler's automatic waits would serialise: hence the loads from inline assembly and the VMEM counter by hand.)
 
 // The kernel's arguments, passed as one struct: a workgroup that walks through several output tiles reads
 // them again from the kernel-argument segment whenever it moves on, instead of keeping all of them in
@@ -136,14 +119,16 @@ struct TiledArgs {
   uint8_t* C_scale;  // fp6 output only
   int fmt_c;
   int group_m, xcd_remap;  // raster: tile rows per group (kGroupM unless a measurement overrides it), XCD remap on / off
-  uint32_t* stamps;  // measurement only (else null): workgroup 0 leaves its shader-clock and real-time counters here at start and end
   int nsplit;        // KSPLIT: workgroups that share an output tile, each over K / nsplit (1 otherwise)
+#ifdef MXFP6_PROBES
+  uint32_t* stamps;  // measurement build only (else null): workgroup 0 leaves its shader-clock and real-time counters here at start and end
+#endif
 };
 
 // FUSED: the epilogue applies scales / bias / activation (args.ep).  A separate instantiation, because branches
 // around updates of all accumulators make the compiler copy them at every output tile, taken or not (3-4 % of an
 // unfused 8192^3 GEMM).
-// ABL (measurement only, results are then meaningless): bit 0 leaves out the LDS reads of the operands after the first
+// ABL (measurement build only, -DMXFP6_PROBES; results are then meaningless): bit 0 leaves out the LDS reads of the operands after the first
 // K-tile of an output tile, bit 1 the direct loads after the prologue, bit 2 the MFMAs after the first K-tile of an output
 // tile.  What the remaining parts of the kernel take, in time and in shader clocks, is how bench.py splits the kernel's
 // time between the matrix cores, the LDS reads and the loads.
@@ -697,6 +682,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
     }
   };
 
+#ifdef MXFP6_PROBES
   auto clock_stamp = [&](int where) __attribute__((always_inline)) {
     const auto g = fresh_args();
     uint32_t* st = g->stamps;
@@ -706,6 +692,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
       st[2 * where] = (uint32_t)t, st[2 * where + 1] = (uint32_t)r;
     }
   };
+#else
+  auto clock_stamp = [](int) __attribute__((always_inline)) {};
+#endif
   clock_stamp(0);
   // prologue: scales of the first four K-tiles, K-tiles 0 .. D-1 and, for group 1, the loads of tile D
   // that its compute cluster of "step -1" would have issued; tile 0 must have landed everywhere
@@ -935,8 +924,11 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const bool ksplit = g.ksplit > 1 && g.ks_part;
   const int shape = ksplit ? g.tile_rows | 256 << 16 : tiled_tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
-  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap == 1 ? 0 : g.raster_no_xcd_remap == 2 ? 2 : 1, g.clock_stamps,
-                        ksplit ? g.ksplit : 1};
+  const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap == 1 ? 0 : g.raster_no_xcd_remap == 2 ? 2 : 1, ksplit ? g.ksplit : 1
+#ifdef MXFP6_PROBES
+                        , g.clock_stamps
+#endif
+  };
   if (ksplit) {
     if constexpr (sizeof(typename Out::type) != 1) {
       if ((bm != 128 && bm != 256) || g.K % (4 * kBK * g.ksplit) != 0 || g.K / kBK / g.ksplit < kMinShareTiles || (size_t)g.M * g.N % 4) return hipErrorInvalidValue;
@@ -959,6 +951,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     if (bn == 128) gemm_tiled_kernel<FA, FB, Out, 2, 1, true><<<grid, NW * 64, 0, s>>>(ta);
     else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
     else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
+#ifdef MXFP6_PROBES
   } else if (g.ablation > 0 && g.ablation < 8) {
     // measurement instantiations: e2m3 x e2m3, bf16 output, 256 x 256 tiles only
     if constexpr (FA == 2 && FB == 2 && sizeof(typename Out::type) == 2) {
@@ -974,6 +967,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     } else {
       return hipErrorInvalidValue;
     }
+#endif
   } else {
     if (bn == 128) gemm_tiled_kernel<FA, FB, Out, 2, 1, false><<<grid, NW * 64, 0, s>>>(ta);
     else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, false><<<grid, NW * 64, 0, s>>>(ta);

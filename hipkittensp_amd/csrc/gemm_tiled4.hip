@@ -14,6 +14,7 @@
 // LDS for the store; no fused epilogue.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "loader.hpp"
 
 namespace mxfp6 {
 namespace t4 {
@@ -32,22 +33,6 @@ constexpr int SCL = 2;        // scale direct loads per wave per batch that carr
 constexpr int NMMA = 2 * TM * TN;
 static_assert(kLdsBytes <= 163840, "LDS budget");
 
-__device__ __forceinline__ void dma16(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void barrier() {
-  __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_barrier" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
 
 template <int FA, int FB, typename Out>
 __global__ __launch_bounds__(NW * 64) void gemm_tiled4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,

@@ -50,6 +50,7 @@ hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s);
 hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s);  // sums g.ksplit partial matrices at g.ks_part into g.C, with the epilogue
 bool gemm_ring_supports(const GemmArgs& g);  // batched decode: private streams of B per wave, A through a flag-guarded ring (no barrier per K-tile)
 int ring_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes, size_t* counters);  // its K split for this problem (want: 0 = by shape, 1 = none, n = n shares): shares (1 = none), bytes of partial tiles, arrival counters
+bool gemm_ring_preferred(const GemmArgs& g);  // by shape: weights streamed from HBM against 17 - 128 rows of a row-major A
 hipError_t launch_gemm_ring(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
 bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel

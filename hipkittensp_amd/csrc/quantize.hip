@@ -2,6 +2,7 @@
 // HBM-bound elementwise work: 4 B/element read, 0.78 B/element written.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "loader.hpp"
 
 namespace mxfp6 {
 
@@ -21,9 +22,6 @@ namespace mxfp6 {
 // 16-byte pieces the tile-major order permutes).
 constexpr int kQWaves = 4;  // waves per workgroup; a wave fetches 64 blocks at a time (8 KB of fp32, 4 KB of bf16)
 
-__device__ __forceinline__ void dma16_q(const __amdgpu_buffer_rsrc_t& rsrc, uint32_t lds_base, int voff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_base), "v"(voff), "s"(rsrc) : "memory");
-}
 
 // In: float, or uint16_t for bf16 (the same values after the exact widening: the bf16 instruction
 // v_cvt_scalef32_pk32_{fp6,bf6}_bf16 was checked against the fp32 one on 1 M values per format, no difference).
@@ -56,12 +54,12 @@ __global__ __launch_bounds__(kQWaves * 64) void quantize_kernel(const In* __rest
       const long g16 = ch / nkt, kt = ch - g16 * nkt;
       const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + (g16 * 16 * nkb + kt * 4) * BB, (uint32_t)(15 * nkb * BB + 4 * BB));
 #pragma unroll
-      for (int q = 0; q < NLD; q++) dma16_q(r, buf + q * 1024, voff[q]);
+      for (int q = 0; q < NLD; q++) dma16(r, buf + q * 1024, voff[q], 0);
     } else {
       const long left = nblocks * BB - ch * kChunk;
       const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const uint8_t*>(X) + ch * kChunk, (uint32_t)(left < kChunk ? left : kChunk));
 #pragma unroll
-      for (int q = 0; q < NLD; q++) dma16_q(r, buf + q * 1024, voff[q]);
+      for (int q = 0; q < NLD; q++) dma16(r, buf + q * 1024, voff[q], 0);
     }
   };
   if (chunk < nchunks) fetch(chunk);

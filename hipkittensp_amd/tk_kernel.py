@@ -327,16 +327,24 @@ def set_relayout(on: bool) -> bool:
     return bool(_lib.lib().mxfp6_set_relayout(1 if on else 0))
 
 
+def allow_e3m2_pair(allow: bool) -> bool:
+    """e3m2 x e3m2 is the one pair of formats whose result can miss the 2e-3 accuracy bar (the scaled MFMA's own sum is
+    inexact there, up to 1e-4 of sum |a||b| per output): dispatch_micro raises for it until this thread has accepted that
+    with allow_e3m2_pair(True).  Returns the previous setting."""
+    return bool(_lib.lib().mxfp6_allow_e3m2_pair(1 if allow else 0))
+
+
 def set_k_split(shares: int) -> int:
     """K split of the tiled kernel for this thread's later calls (measurement / tests): 0 = where it pays (default), 1 = never,
     -1 = wherever the shape allows it, n > 1 = n workgroups per output tile; returns the previous setting."""
-    return _lib.lib().mxfp6_probe_ksplit(int(shares))
+    return _lib.lib().mxfp6_set_k_split(int(shares))
 
 
 def k_split_plan(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, shares: int = 0, layout_b: int = LAYOUT_ROW):
-    """(workgroups per output tile, rows of A per tile) the tiled kernel's K split would use for this shape; (1, 0) = none."""
+    """(workgroups per output tile, rows of A per tile) the tiled kernel's K split would use for this shape; (1, 0) = none.
+    A query of the measurement build (libmxfp6_probes.so: the same host code as the operator's)."""
     rows = ctypes.c_int(0)
-    n = _lib.lib().mxfp6_probe_ksplit_plan(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1, int(shares), ctypes.byref(rows))
+    n = _lib.probes().mxfp6_probe_ksplit_plan(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1, int(shares), ctypes.byref(rows))
     if n < 0:
         _lib.check(n, "k_split_plan")
     return n, rows.value
@@ -348,15 +356,10 @@ CHOICE_BLOCK_K_SPLIT = 27  # kernel_choice(): the block kernel with its K split 
 
 def kernel_choice(M: int, N: int, K: int, layout_a: int = LAYOUT_ROW, layout_b: int = LAYOUT_ROW) -> int:
     """The kernel (KERNEL_* code, or CHOICE_TILED_K_SPLIT / CHOICE_BLOCK_K_SPLIT) the automatic path takes for this shape; launches nothing."""
-    n = _lib.lib().mxfp6_probe_choice(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1)
+    n = _lib.lib().mxfp6_kernel_choice(int(M), int(N), int(K), int(bool(layout_a)) | int(bool(layout_b)) << 1)
     if n < 0:
         _lib.check(n, "kernel_choice")
     return n
-
-
-def set_block_kernel(enable: bool) -> bool:
-    """Measurement: keep the block kernel out of (False) or in (True, the default) the automatic choice; returns the previous setting."""
-    return bool(_lib.lib().mxfp6_probe_block(int(bool(enable))))
 
 
 def set_kernel(which: int) -> int:

@@ -28,11 +28,17 @@
  *   - the gemm entry points on decode shapes whose K range is split between workgroups (M <= 32, N <= 2048,
  *     K >= 24576): 2 MB;
  *   - the gemm entry points on problems of few output tiles and long K (up to a few hundred rows of A, K >= 5120; see
- *     mxfp6_probe_ksplit), where the LDS-tiled kernel or the block kernel splits K between workgroups: shares * 4 M N
+ *     mxfp6_set_k_split), where the LDS-tiled kernel or the block kernel splits K between workgroups: shares * 4 M N
  *     bytes, at most 64 MB (one workspace for both kernels).
  * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K splits are left out
  * (same results up to the order of fp32 sums, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
- * hipErrorStreamCaptureUnsupported where it would need a new one.  mxfp6_gemm_noalloc never allocates.
+ * hipErrorStreamCaptureUnsupported where it would need a new one.  A workspace that a capture did use is recorded in the
+ * graph: the library never frees such a block again (when a later call needs a larger one, or at
+ * mxfp6_release_workspaces(), it is kept allocated until the process ends), so the graph stays valid.  Replay it on the
+ * stream it was captured on, or on another one only while no call of this library runs on the capture stream: the
+ * replays and those calls share the workspace.  At most 128 workspaces exist at a time; beyond that the least recently
+ * used one that no graph holds is returned to the allocator on its own stream, so call mxfp6_release_workspaces()
+ * before destroying streams this library has seen.  mxfp6_gemm_noalloc never allocates.
  *
  * Alignment.  Pointers are accepted from 4-byte alignment on (C: its element size).  The fast kernels
  * fetch 16 bytes per lane: they run when A_packed, B_packed, both scale tensors and C are 16-byte aligned
@@ -43,7 +49,9 @@
  * accumulators agree with an fp64 dequantise-and-matmul to fp32 rounding (relative error < 1e-6 of the
  * result's range).  e3m2 x e3m2 is weaker: the scaled MFMA's internal sum drops low-order bits of
  * wide-ranging products, giving an error of up to 1e-4 of sum_k |a_mk| |b_nk| per output, which is above
- * 2e-3 of the result only where the sum cancels to less than 5 % of its terms.
+ * 2e-3 of the result only where the sum cancels to less than 5 % of its terms.  Because that can exceed the library's
+ * stated bar without any sign, the gemm entry points return MXFP6_EACCURACY for that pair of formats until the calling
+ * thread has accepted it with mxfp6_allow_e3m2_pair(1); every other pair meets the bar by construction.
  */
 #ifndef MXFP6_GEMM_H
 #define MXFP6_GEMM_H
@@ -70,6 +78,7 @@ extern "C" {
 #define MXFP6_ESCRATCH (-8)     /* mxfp6_gemm_noalloc: the requested K split does not fit the static scratch memory */
 #define MXFP6_EINVAL_KERNEL (-9) /* mxfp6_set_kernel: unknown kernel code                        */
 #define MXFP6_EBLOB (-10)       /* not a tile-major operand blob of a version this library reads */
+#define MXFP6_EACCURACY (-12)   /* e3m2 x e3m2 without mxfp6_allow_e3m2_pair(1): the pair can miss the 2e-3 accuracy bar */
 #define MXFP6_EWORKSPACE (-11)  /* a call that cannot run without a workspace did not get one (allocator, or all slots held by graphs) */
 
 /* Activations of mxfp6_gemm_fused. */
@@ -119,11 +128,14 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *    4  mid-M kernel (needs 32 < M <= 512, K % 1024 == 0, row-major A)
  *   18  the 4-wave interleaved schedule of the LDS-tiled kernel (one wave per SIMD with a 128 x 128 wave tile; shapes
  *       of kernel 2, no fused epilogue); never chosen automatically, kept to compare the two schedules
+ *   28  ring kernel for batched decode (needs K % 512 == 0, N % 4 == 0): every wave streams its own 32 rows of B through
+ *       private LDS slots, A comes through a ring that a loader wave fills and flags guard, no barrier per K-tile;
+ *       splits K between workgroups by the thread's mxfp6_set_k_split setting
  *   22  block kernel: output tiles of 128 x 128, four waves in step with the operand fragments double-buffered in
  *       registers, one barrier per K-tile (needs N % 8 == 0, K % 128 == 0); chosen automatically where
  *       its tiles do not outnumber the CUs and K is of moderate length (a few hundred rows of A);
  *       23 / 24: with an operand ring of three slots (two workgroups per CU) / six slots (one); 26: with tiles of
- *       128 x 256 and eight waves.  22 - 24 split K between workgroups by the thread's mxfp6_probe_ksplit setting
+ *       128 x 256 and eight waves.  22 - 24 split K between workgroups by the thread's mxfp6_set_k_split setting
  *       (0: where the library's rule for this kernel says so; the same per-stream workspace as the tiled kernel's split)
  * No counterpart in the reference, whose shapes are compile-time constants per binary
  * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
@@ -278,7 +290,8 @@ int mxfp6_release_workspaces(void);
  *               of the tiled or block kernel, or a kernel of another family for the shape, the same products are
  *               added in another order: equal within the rounding of fp32 partial sums, and bit-identical whenever
  *               those sums are exact;
- *   nsplit = 1, 2, 4, 8: the skinny kernel with K split between that many workgroups per tile of C (needs M <= 32,
+ *   nsplit = 1: as nsplit = 0, but K is never split between workgroups (nothing touches the static array);
+ *   nsplit = 2, 4, 8: the skinny kernel with K split between that many workgroups per tile of C (needs M <= 32,
  *               K % 512 == 0; MXFP6_EINVAL_SHAPE otherwise).  A tile of C is 16 columns for N <= 4096 and 32 beyond:
  *               ceil(N / 16 or 32) * nsplit must not exceed 256, else MXFP6_ESCRATCH and nothing is launched.
  * Every call on a GPU shares that GPU's array: the counters are cleared by a small kernel in front of each split launch,
@@ -288,93 +301,34 @@ int mxfp6_release_workspaces(void);
 int mxfp6_gemm_noalloc(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale,
                        void *C_bf16, int M, int N, int K, int fmt_a, int fmt_b, int nsplit, void *hip_stream);
 
-/*
- * Measurement probes (no counterpart in the reference; bench.py reports them next to the roofline fractions).
- *
- * mxfp6_probe_mfma: a kernel that only issues v_mfma_scale_f32_32x32x64_f8f6f4 -- two waves per SIMD, each with two
- * fragments of A and two of B taken once from the given packed operands and scales (rows >= 32, K >= 64) and four
- * independent accumulators, `iters` rounds of four MFMAs.  Returns the number of waves launched (> 0; each issues
- * 4 * iters MFMAs of 131072 flop), or a negative MXFP6_E* code, or -(1000 + hipError_t).  stats[0..3] receive the shader
- * clock counter and the 100 MHz real-time counter of one workgroup at its start and end: clocks / time is the clock the
- * chip sustains under this load.  sink: one float of device memory (never written in practice).
- *
- * mxfp6_probe_stream: `workgroups` workgroups of `waves` (4 or 8) waves read `bytes` bytes (a multiple of
- * workgroups * waves * 8192) once, each wave a private contiguous range, through direct-to-LDS loads with 16 KB in flight
- * per wave, and do nothing else.  stats as above.
- *
- * mxfp6_probe_tiled_clock: per calling thread; while `stamps` is not NULL the LDS-tiled GEMM kernel's workgroup 0 writes
- * the same four counters (start, end) there on every launch.
- */
-int mxfp6_probe_mfma(const void *A_packed, const void *B_packed, const void *A_scale, const void *B_scale, int rows_a,
-                     int rows_b, int K, int fmt_a, int fmt_b, int iters, float *sink, uint32_t *stats, void *hip_stream);
-int mxfp6_probe_stream(const void *buf, size_t bytes, int workgroups, int waves, uint32_t *stats, void *hip_stream);
-int mxfp6_probe_tiled_clock(uint32_t *stamps);
+/* e3m2 x e3m2 (see "Accuracy" above): 1 lets this thread's later gemm calls run that pair of formats, 0 (the default) makes
+ * them return MXFP6_EACCURACY.  Returns the previous setting.  No counterpart in the reference. */
+int mxfp6_allow_e3m2_pair(int allow);
 
 /*
- * The workgroup -> output tile map of the LDS-tiled kernel, evaluated on the host with the kernel's own function:
- * order[b] = pm | pn << 16 is the tile (row pm, column pn of a tiles_m x tiles_n grid) that logical workgroup b works on.
- * The kernel uses group_m = 4 and xcd_remap = 1; mxfp6_probe_raster (per calling thread, measurement only; group_m = 0
- * restores the default) makes later launches use other values, for sweeps of the raster like the reference's
- * (analysis/paper_experiments/grid_micro/data_to_log.json; remap include/common/util.cuh:78-101).  A host-side pointer:
- * `order` holds tiles_m * tiles_n ints.  Launches with a K split between workgroups order (tile, share) pairs share by
- * share and hand each XCD an eighth of that order, so that an XCD's workgroups work on one K range of A and B;
- * mxfp6_probe_raster(group_m, 2) keeps the tile remap but orders them tile by tile (measurement: the order before).
+ * K split between workgroups (per calling thread; returns the previous setting).  Problems of few output tiles and long K
+ * (up to a few hundred rows of A against a wide weight matrix) run with several workgroups per output tile, each over a
+ * part of K.  The LDS-tiled and the block kernel's shares leave fp32 partial matrices in this stream's workspace and a
+ * second small kernel adds them in share order and applies the epilogue; the ring kernel's shares leave partial tiles
+ * there and the workgroup that arrives last at a tile adds them in share order.  Either way the result does not depend
+ * on timing.  0 = where it pays (default), 1 = never, -1 = wherever the shape allows it, n > 1 = n workgroups per output
+ * tile where the shape allows it, else unsplit.  No counterpart in the reference (its GEMMs are one workgroup per
+ * 256 x 256 tile, analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61).
  */
-int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int *order);
-
-/*
- * Ablations of the LDS-tiled kernel (per calling thread, measurement only, 0 = off): while mask != 0, e2m3 x e2m3 bf16
- * GEMMs on 256 x 256 tiles run a build of the kernel without its LDS reads of the operands (bit 0), without its
- * direct loads after the prologue (bit 1), without its MFMAs (bit 2); other calls fail with hipErrorInvalidValue.  The
- * output of such a launch is meaningless.  Timing the combinations 1 - 4 and 6 next to the full kernel (with
- * mxfp6_probe_tiled_clock for the shader clock) shows what each part costs and which ones the power management charges
- * (5 and 7, no LDS reads and no MFMAs at once, are not built and rejected: those builds spill registers).
- */
-int mxfp6_probe_tiled_ablation(int mask);
-int mxfp6_probe_raster(int group_m, int xcd_remap);
-
-/*
- * K split of the LDS-tiled kernel and of the block kernel (per calling thread, measurement and tests; returns the previous
- * setting; 1 switches both off, 0 lets each kernel's own rule decide, -1 / n apply to whichever of the two runs).  Problems of
- * few output tiles and long K (a few hundred rows of A against a wide weight matrix) run with several workgroups per
- * output tile, each over a part of K: the shares leave their fp32 sums in this stream's workspace (shares * M * N * 4
- * bytes, hipMallocAsync on the caller's stream at first use, kept until mxfp6_release_workspaces(); on a stream that is
- * being captured only if it exists already, else the launch runs unsplit) and a second small kernel adds them in share
- * order and applies the epilogue, so results do
- * not depend on timing.  0 = where it pays (default: K >= 14336 and at most 64 output tiles of 256 x 256, 128 from
- * K = 24576 on; 8192 <= K < 14336 only with at most 32 tiles and no skinny kernel for the shape; up to 64 rows of a
- * row-major A stay with the skinny kernel, except 33 - 64 rows against tile-major weights with K >= 24576 or N above 8192
- * and no multiple of it), 1 = never,
- * -1 = wherever the shape allows it, n > 1 = n workgroups per output tile where the shape allows it (K a multiple of 512 n,
- * at least 8 K-tiles of 128 per share, at most half as many output tiles as CUs), else unsplit.  The block kernel's own
- * rule (its 128 x 128 tiles on at most half the CUs, K >= 8192, or >= 5120 with both operands tile-major; asked before the
- * tiled kernel's) is described with mxfp6_set_kernel 22 and reported by mxfp6_probe_choice (code 27).
- * No counterpart in the reference (its GEMMs are one workgroup per 256 x 256 tile, analysis/bf16_gemm/mi325x/kernel_8192.cpp:45-61).
- */
-int mxfp6_probe_ksplit(int shares);
-/* The split the automatic path (shares = 0) or a forced setting would use for a shape on the current device: workgroups per
- * output tile (1 = none; negative = error code), and in *tile_rows (may be NULL) the rows of A per output tile (0 = none).
- * layouts: bit 0 set = A tile-major, bit 1 set = B tile-major (the e2m3 x e2m3 formats are assumed; the plan does not depend
- * on them). */
-int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int *tile_rows);
-
-/* Measurement switch, per calling thread: 0 keeps the block kernel (mxfp6_set_kernel 22 - 27) out of the automatic choice,
- * so that the same call can be timed with and without it; returns the previous setting.  Default 1. */
-int mxfp6_probe_block(int enable);
+int mxfp6_set_k_split(int shares);
 
 /* The kernel the automatic path takes for a problem of this shape on the current device (e2m3 x e2m3, bf16 output, no fused
- * epilogue, 16-byte aligned tensors): a code of mxfp6_set_kernel (1 generic, 2 tiled, 3 skinny, 4 mid-M, 22 block, 26
- * block with 128 x 256 tiles), or 25 / 27 for the tiled / the block kernel with its K split between workgroups; negative =
- * error code.  layouts as in
- * mxfp6_probe_ksplit_plan.  Reads the thread's mxfp6_probe_ksplit setting; launches nothing. */
-int mxfp6_probe_choice(int M, int N, int K, int layouts);
+ * epilogue, 16-byte aligned tensors): a code of mxfp6_set_kernel, or 25 / 27 for the tiled / the block kernel with its
+ * K split between workgroups; negative = error code.  layouts: bit 0 set = A tile-major, bit 1 set = B tile-major.
+ * Reads the thread's mxfp6_set_k_split setting; launches nothing. */
+int mxfp6_kernel_choice(int M, int N, int K, int layouts);
 
 /* Human-readable text for a return code of this library (never NULL). */
 const char *mxfp6_strerror(int code);
 
 /* ABI version of this header, major * 100 + minor, and what the loaded library reports: a caller built against this
  * header checks that the majors agree (entry points are only ever added within a major). */
-#define MXFP6_ABI_VERSION 120
+#define MXFP6_ABI_VERSION 200
 int mxfp6_abi_version(void);
 
 #ifdef __cplusplus

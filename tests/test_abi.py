@@ -11,18 +11,20 @@ import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "mxfp6_gemm.h")
+PROBES_HEADER = os.path.join(ROOT, "include", "mxfp6_probes.h")
 LIB = os.path.join(ROOT, "hipkittensp_amd", "libmxfp6_gemm.so")
+PROBES_LIB = os.path.join(ROOT, "hipkittensp_amd", "libmxfp6_probes.so")
 
 
-def _declared_functions():
-    src = open(HEADER).read()
+def _declared_functions(header=HEADER):
+    src = open(header).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     return sorted(set(re.findall(r"\b(mxfp6_[a-z0-9_]+)\s*\(", src)))
 
 
 @pytest.fixture(scope="module")
 def built_lib():
-    if not os.path.exists(LIB):
+    if not os.path.exists(LIB) or not os.path.exists(PROBES_LIB):
         from hipkittensp_amd import build
         build.build(verbose=False)
     return LIB
@@ -31,13 +33,17 @@ def built_lib():
 def test_header_declares_the_operator():
     names = _declared_functions()
     for want in ("mxfp6_gemm", "mxfp6_gemm_f32out", "mxfp6_gemm_ex", "mxfp6_gemm_fused", "mxfp6_gemm_fused_fp6", "mxfp6_quantize", "mxfp6_quantize_ex", "mxfp6_quantize_bf16", "mxfp6_tile_operand", "mxfp6_tile_scales",
-                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout", "mxfp6_gemm_noalloc", "mxfp6_release_workspaces"):
+                 "mxfp6_strerror", "mxfp6_abi_version", "mxfp6_set_kernel", "mxfp6_set_relayout", "mxfp6_gemm_noalloc", "mxfp6_release_workspaces",
+                 "mxfp6_set_k_split", "mxfp6_kernel_choice"):
         assert want in names
+    # the operator's header is the operator: measurement entry points live in mxfp6_probes.h
+    assert not [n for n in names if "probe" in n] and len(names) <= 25, names
+    assert {"mxfp6_probe_mfma", "mxfp6_probe_stream", "mxfp6_probe_tiled_clock", "mxfp6_probe_tiled_ablation", "mxfp6_probe_raster", "mxfp6_tile_order"} <= set(_declared_functions(PROBES_HEADER))
 
 
 def test_header_compiles_as_plain_c(tmp_path):
     c = tmp_path / "t.c"
-    c.write_text('#include "mxfp6_gemm.h"\nint main(void){return MXFP6_FMT_E2M3 + MXFP6_FMT_E3M2 == 5 ? 0 : 1;}\n')
+    c.write_text('#include "mxfp6_gemm.h"\n#include "mxfp6_probes.h"\nint main(void){return MXFP6_FMT_E2M3 + MXFP6_FMT_E3M2 == 5 ? 0 : 1;}\n')
     subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(c), "-o", str(tmp_path / "t.o")])
 
 
@@ -46,9 +52,15 @@ def test_library_exports_every_declared_symbol(built_lib):
     exported = {l.split()[-1] for l in out.splitlines() if " T " in l}
     for name in _declared_functions():
         assert name in exported, f"{name} declared in the header but not exported"
+    # ... and nothing else: no measurement entry point is part of the operator's library
+    assert {n for n in exported if n.startswith("mxfp6_")} == set(_declared_functions())
+    out = subprocess.check_output(["nm", "-D", "--defined-only", PROBES_LIB], text=True)
+    exported_probes = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    for name in _declared_functions() + _declared_functions(PROBES_HEADER):
+        assert name in exported_probes, f"{name} not exported by the measurement build"
     L = ctypes.CDLL(built_lib)          # loads without a GPU
     L.mxfp6_abi_version.restype = ctypes.c_int
-    assert L.mxfp6_abi_version() == 120
+    assert L.mxfp6_abi_version() == 200
     L.mxfp6_strerror.restype = ctypes.c_char_p
     L.mxfp6_strerror.argtypes = [ctypes.c_int]
     assert L.mxfp6_strerror(0) == b"success"
@@ -112,14 +124,20 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     L.mxfp6_set_kernel.argtypes = [ci]
     assert L.mxfp6_set_kernel(99) == -9 and L.mxfp6_set_kernel(-1) == -9
     # measurement switches validate their argument too (they only set per-thread state: no GPU needed)
-    assert L.mxfp6_probe_tiled_ablation(5) == -2 and L.mxfp6_probe_tiled_ablation(7) == -2 and L.mxfp6_probe_tiled_ablation(0) == 0
-    assert L.mxfp6_probe_ksplit(65) == -2 and L.mxfp6_probe_ksplit(-2) == -2
-    prev = L.mxfp6_probe_ksplit(1)
-    assert prev == 0 and L.mxfp6_probe_ksplit(0) == 1
-    L.mxfp6_probe_choice.restype = ci
-    L.mxfp6_probe_choice.argtypes = [ci, ci, ci, ci]
-    assert L.mxfp6_probe_choice(0, 16, 512, 0) == -2 and L.mxfp6_probe_choice(16, 16, 48, 0) == -2    # shape
-    assert L.mxfp6_probe_choice(16, 16, 512, 4) == -6 and L.mxfp6_probe_choice(40, 64, 512, 1) == -2  # layouts; tile-major needs rows % 32
+    P = ctypes.CDLL(PROBES_LIB)
+    assert P.mxfp6_probe_tiled_ablation(5) == -2 and P.mxfp6_probe_tiled_ablation(7) == -2 and P.mxfp6_probe_tiled_ablation(0) == 0
+    assert L.mxfp6_set_k_split(65) == -2 and L.mxfp6_set_k_split(-2) == -2
+    prev = L.mxfp6_set_k_split(1)
+    assert prev == 0 and L.mxfp6_set_k_split(0) == 1
+    L.mxfp6_kernel_choice.restype = ci
+    L.mxfp6_kernel_choice.argtypes = [ci, ci, ci, ci]
+    assert L.mxfp6_kernel_choice(0, 16, 512, 0) == -2 and L.mxfp6_kernel_choice(16, 16, 48, 0) == -2    # shape
+    assert L.mxfp6_kernel_choice(16, 16, 512, 4) == -6 and L.mxfp6_kernel_choice(40, 64, 512, 1) == -2  # layouts; tile-major needs rows % 32
+    # e3m2 x e3m2 needs the caller's consent (it can miss the accuracy bar); the check comes before any HIP call
+    assert L.mxfp6_gemm(one, one, one, one, one, 16, 16, 512, 3, 3, None) == -12 and b"e3m2 x e3m2" in L.mxfp6_strerror(-12)
+    assert L.mxfp6_allow_e3m2_pair(1) == 0 and L.mxfp6_gemm(one, one, one, one, one, 0, 16, 512, 3, 3, None) == 0 and L.mxfp6_allow_e3m2_pair(0) == 1
+    # the entry point that allocates nothing: nsplit = 1 is "never split", whatever the shape; 2, 4, 8 need a decode shape
+    assert L.mxfp6_gemm_noalloc(one, one, one, one, one, 0, 16, 640, 2, 2, 1, None) == 0
     assert L.mxfp6_set_kernel(2) == 0
     import threading
     seen = []
@@ -218,7 +236,7 @@ def test_tile_order_is_a_bijection(built_lib, tiles_m, tiles_n, group_m, xcd):
     include/common/util.cuh:92), and with the remap on, the tiles one XCD works on form a contiguous run of the raster."""
     import numpy as np
 
-    L = ctypes.CDLL(built_lib)
+    L = ctypes.CDLL(PROBES_LIB)
     L.mxfp6_tile_order.restype = ctypes.c_int
     L.mxfp6_tile_order.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p]
     nb = tiles_m * tiles_n

@@ -46,7 +46,9 @@ def hk():
     from hipkittensp_amd import _lib
 
     _lib.lib()  # fails loudly if the HIP library is not built: there is no fallback path
+    prev = m.tk_kernel.allow_e3m2_pair(True)   # the tests of that pair know its bound (TOL_E3M2_BOTH); test_e3m2_pair_needs_opt_in checks the default
     yield m
+    m.tk_kernel.allow_e3m2_pair(prev)
     m.tk_kernel.set_kernel(0)
 
 
@@ -68,6 +70,25 @@ def gemm(hk, ap, bp, asc, bsc, fa=2, fb=2, out="f32", kernel=0):
     return C.view(torch.int16).cpu().numpy().view(np.uint16)
 
 
+def gemm_probes_lib(ap, bp, asc, bsc, fa=2, fb=2, kernel=0):
+    """The same call through the measurement build of the library (libmxfp6_probes.so), whose overrides (raster, clock
+    stamps, ablations) only its own entry points see; fp32 output."""
+    from hipkittensp_amd import _lib
+
+    P = _lib.probes()
+    M, N, K = ap.shape[0], bp.shape[0], ap.shape[1] // 3 * 4
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    dA, dB, dAs, dBs = dev(ap), dev(bp), dev(asc), dev(bsc)
+    prev = P.mxfp6_set_kernel(kernel)
+    try:
+        rc = P.mxfp6_gemm_ex(dA.data_ptr(), dB.data_ptr(), dAs.data_ptr(), dBs.data_ptr(), C.data_ptr(), M, N, K, fa, fb, 0, 0, 1, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+    finally:
+        P.mxfp6_set_kernel(prev)
+    return C.cpu().numpy()
+
+
 def operands(M, N, K, fa, fb, seed, kind_a="normal", kind_b="normal"):
     xa = o.make_source(kind_a, (M, K), np.random.default_rng(seed))
     xb = o.make_source(kind_b, (N, K), np.random.default_rng(seed + 1000))
@@ -80,6 +101,21 @@ def one_hot_b(K):
     codes = np.zeros((K, K), np.uint8)
     codes[np.arange(K), np.arange(K)] = 0b001000  # 1.0 in e2m3
     return o.pack_fp6(codes), np.full((K, K // 32), 127, np.uint8)
+
+
+def test_e3m2_pair_needs_opt_in(hk):
+    """e3m2 x e3m2 can exceed the 2e-3 bar (the MFMA's own sum of such products is inexact): by default the operator
+    refuses the pair with a distinct error, and runs it once the caller has accepted the weaker bound."""
+    ap, asc, bp, bsc = operands(64, 64, 256, 3, 3, seed=5)
+    prev = hk.tk_kernel.allow_e3m2_pair(False)
+    try:
+        with pytest.raises(RuntimeError, match="e3m2 x e3m2"):
+            gemm(hk, ap, bp, asc, bsc, 3, 3)
+        gemm(hk, ap, bp, asc, bsc, 3, 2)   # every other pair runs
+        assert hk.tk_kernel.allow_e3m2_pair(True) is False
+        check(gemm(hk, ap, bp, asc, bsc, 3, 3), o.gemm_ref(ap, bp, asc, bsc, 3, 3, acc=np.float64), 3, 3, ap, asc, bp, bsc)
+    finally:
+        hk.tk_kernel.allow_e3m2_pair(prev)
 
 
 # ------------------------------------------------------------------ decode: bit exact
@@ -263,57 +299,77 @@ def test_block_kernel_k_split(hk, M, N, K, shares, fa, fb):
         tk.set_k_split(prev)
 
 
-def test_kernel_choice_by_shape(hk):
-    """The automatic choice over the library's kernels, as mxfp6_probe_choice reports it (A row-major unless stated)."""
+# The automatic choice is judged by what it costs, not by which kernel it names: on this list of shapes (decode and batched
+# decode against row-major and tile-major weights, a few hundred rows, prefill-sized and square problems, a K no K split
+# divides, wide and narrow N) the call as the library dispatches it must be within 10 % of the fastest forced candidate.
+CHOICE_SHAPES = [(16, 8192, 28672, 0, 0), (16, 8192, 28672, 0, 1), (32, 8192, 28672, 0, 1), (64, 8192, 28672, 0, 1), (64, 8192, 28672, 0, 0),
+                 (128, 8192, 28672, 0, 1), (256, 8192, 28672, 1, 1), (512, 8192, 8192, 1, 1), (256, 8192, 8192, 0, 1), (1024, 8192, 8192, 0, 1),
+                 (64, 28672, 8192, 0, 0), (32, 28672, 4096, 0, 1), (128, 4096, 14336, 0, 1), (2048, 4096, 4096, 1, 1), (96, 10240, 8192, 0, 1),
+                 (16, 4096, 11008, 0, 1), (4096, 4096, 4096, 0, 0), (48, 57344, 8192, 0, 0), (192, 2048, 8192, 0, 1), (8, 2048, 8192, 0, 0)]
+
+
+def test_automatic_choice_is_within_ten_percent_of_the_best_forced_candidate(hk):
     tk = hk.tk_kernel
-    assert tk.kernel_choice(8192, 8192, 8192) == tk.KERNEL_TILED
-    assert tk.kernel_choice(16, 8192, 28672) == tk.KERNEL_SKINNY and tk.kernel_choice(64, 8192, 8192, 0, 1) == tk.KERNEL_SKINNY
-    assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT
-    assert tk.kernel_choice(256, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT    # K this long and 128 tiles of 128 x 128: the tiled kernel's split streams B faster
-    assert tk.kernel_choice(256, 8192, 16384, 1, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 4096, 14336, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT
-    assert tk.kernel_choice(96, 8192, 2048, 1, 1) != tk.CHOICE_BLOCK_K_SPLIT      # two launches for a K this short lose
-    assert tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(32, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY
-    assert tk.kernel_choice(256, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(512, 4096, 4096, 0, 1) == tk.KERNEL_BLOCK
-    assert tk.kernel_choice(2048, 8192, 8192, 1, 1) == tk.KERNEL_TILED      # more 128 x 256 tiles than CUs
-    assert tk.kernel_choice(4096, 2048, 1024, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(4096, 2048, 4096, 1, 1) == tk.KERNEL_BLOCK_WIDE  # K up to 2048: up to two 128 x 128 tiles per CU
-    assert tk.kernel_choice(1024, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK_WIDE and tk.kernel_choice(1024, 8192, 8192, 0, 1) == tk.KERNEL_TILED
-    assert tk.kernel_choice(256, 8192, 4096 + 128, 1, 1) == tk.KERNEL_BLOCK  # K % 512 != 0 is fine
+    candidates = ((tk.KERNEL_TILED, 1), (tk.KERNEL_TILED_128, 1), (tk.KERNEL_TILED_256, 1), (tk.KERNEL_TILED_128x128, 1), (tk.KERNEL_BLOCK, 1), (tk.KERNEL_BLOCK_WIDE, 1),
+                  (tk.KERNEL_SKINNY, 0), (tk.KERNEL_MID, 0), (tk.KERNEL_RING, 0), (tk.KERNEL_TILED, -1), (tk.KERNEL_BLOCK, -1))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(123)
+
+    def time_us(ops, C, la, lb, kernel, split, reps=12):
+        pk, ps = tk.set_kernel(kernel), tk.set_k_split(split)
+        try:
+            for i in range(3):
+                hk.dispatch_micro(*ops[i % len(ops)], C, layout_a=la, layout_b=lb)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(reps):
+                hk.dispatch_micro(*ops[i % len(ops)], C, layout_a=la, layout_b=lb)
+            e1.record()
+            torch.cuda.synchronize()
+        except RuntimeError:
+            return None   # the forced kernel does not take the shape
+        finally:
+            tk.set_kernel(pk)
+            tk.set_k_split(ps)
+        return e0.elapsed_time(e1) / reps * 1e3
+
+    behind = {}
+    for M, N, K, la, lb in CHOICE_SHAPES:
+        a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2, layout=la)
+        ops = []
+        for _ in range(2):   # two weight sets: a small B must not simply sit in the last-level cache for one candidate and not the other
+            b, bsc = hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2, layout=lb)
+            ops.append((a, b, asc, bsc))
+        C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        ratio = None
+        for attempt in range(3):   # timings on a shared box scatter: the best of up to three rounds counts
+            auto = time_us(ops, C, la, lb, tk.KERNEL_AUTO, 0)
+            forced = [t for t in (time_us(ops, C, la, lb, k, sp) for k, sp in candidates) if t is not None]
+            auto = min(auto, time_us(ops, C, la, lb, tk.KERNEL_AUTO, 0))
+            r = (auto - 0.7) / min(forced)   # 0.7 us: what the host side of two otherwise equal calls can differ by
+            ratio = r if ratio is None else min(ratio, r)
+            if ratio <= 1.10:
+                break
+        if ratio > 1.10:
+            behind[(M, N, K, la, lb)] = round(ratio, 3)
+        del ops, C
+    assert len(behind) <= 1 and all(r <= 1.25 for r in behind.values()), behind
+
+
+def test_kernel_choice_reports_the_unambiguous_cases(hk):
+    """mxfp6_kernel_choice on shapes where one kernel is the only sensible answer."""
+    tk = hk.tk_kernel
+    assert tk.kernel_choice(8192, 8192, 8192) == tk.KERNEL_TILED and tk.kernel_choice(8192, 8192, 8192, 1, 1) == tk.KERNEL_TILED
+    assert tk.kernel_choice(16, 8192, 28672) == tk.KERNEL_SKINNY
     assert tk.kernel_choice(40, 36, 96) == tk.KERNEL_GENERIC
-    # few output tiles and a long K: this kernel's split however few workgroups it makes (4 tiles x 8 shares here), for every layout pair
-    for la, lb in ((0, 0), (0, 1), (1, 1)):
-        assert tk.kernel_choice(128, 512, 16384, la, lb) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 1024, 8192, la, lb) == tk.CHOICE_BLOCK_K_SPLIT
-    assert tk.kernel_choice(64, 1024, 28672) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 1024, 8192) == tk.KERNEL_SKINNY   # the skinny kernel's up to 64 rows at K = 8192
-    assert tk.kernel_choice(16, 4096, 11008, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT   # K % 512 != 0: not the skinny kernel's
-    assert tk.kernel_choice(128, 2048, 5504, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 2048, 4096, 0, 1) != tk.CHOICE_BLOCK_K_SPLIT  # split from K = 5120 on
-    assert tk.kernel_choice(32, 14592, 11904, 1, 1) == tk.KERNEL_BLOCK          # A tile-major, few rows, no split for this K
-    # the skinny kernel's last round of workgroups (32 rows of B each, 256 a round) nearly empty, long K, tile-major weights
-    assert tk.kernel_choice(16, 8800, 14848, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(16, 8192, 14848, 0, 1) == tk.KERNEL_SKINNY
-    assert tk.kernel_choice(96, 23344, 8704) != tk.KERNEL_SKINNY                # K % 1024 != 0: the tiled kernel's, not the skinny kernel's
-    assert tk.kernel_choice(128, 128, 16384) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 384, 28672, 1, 1) == tk.CHOICE_BLOCK_K_SPLIT  # one and six tiles
-    # few rows against wide weights: the block kernel with a tile for every CU, and beyond K = 16384 where its tiles fill the CUs
-    assert tk.kernel_choice(48, 32768, 12288, 0, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(32, 16640, 28672, 0, 1) == tk.KERNEL_BLOCK
-    assert tk.kernel_choice(16, 27392, 19456, 0, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(16, 23808, 19968, 0, 1) == tk.KERNEL_SKINNY
-    # B row-major: a short K wherever the skinny kernel does not come first, 24 rows at K = 4096, 32 rows only up to K = 7168
-    assert tk.kernel_choice(160, 9216, 1536, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(24, 28672, 4096, 0, 0) == tk.KERNEL_BLOCK
-    assert tk.kernel_choice(32, 24576, 8192, 0, 0) == tk.KERNEL_SKINNY and tk.kernel_choice(48, 24576, 8192, 0, 0) == tk.KERNEL_BLOCK
-    # the tiled kernel's split: three shares a tile for 33 - 64 rows against a wide row-major B, 65 - 128 tiles with few rows or a row-major B
-    assert tk.kernel_choice(64, 16640, 12288, 0, 0) == tk.CHOICE_TILED_K_SPLIT and tk.k_split_plan(64, 16640, 12288, 0, 0, 0)[0] == 3
-    assert tk.kernel_choice(64, 24576, 12288, 0, 0) != tk.CHOICE_TILED_K_SPLIT   # two shares a tile: level, not split
-    assert tk.kernel_choice(160, 18304, 13824, 0, 1) == tk.CHOICE_TILED_K_SPLIT and tk.kernel_choice(384, 12928, 19456, 0, 0) == tk.CHOICE_TILED_K_SPLIT
-    # the mid-M kernel's estimate counts a thin last round of workgroups (268 of them here): not chosen
-    assert tk.kernel_choice(256, 8576, 10240, 0, 0) != tk.KERNEL_MID
-    # a K the skinny kernel cannot take against a row-major B, few rows, many tiles; 17 - 31 rows count as 32
-    assert tk.kernel_choice(8, 21624, 2688, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(24, 19968, 14848, 0, 1) == tk.KERNEL_BLOCK
-    # the tiled split beyond 104 tiles against a tile-major B: only with a row-major A (both tile-major, the 128 x 256 tiles win)
-    assert tk.kernel_choice(192, 28672, 12288, 1, 1) != tk.CHOICE_TILED_K_SPLIT and tk.kernel_choice(160, 28672, 16384, 0, 1) == tk.CHOICE_TILED_K_SPLIT
-    # a long K goes to the tiled split only where its workgroups fill half the CUs (K = 31744 leaves it two shares a tile)
-    assert tk.kernel_choice(320, 4224, 31744, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(128, 11008, 23040, 0, 1) == tk.CHOICE_TILED_K_SPLIT
-    assert tk.kernel_choice(2048, 26624, 640, 0, 0) == tk.KERNEL_BLOCK and tk.kernel_choice(2048, 26624, 640, 0, 1) != tk.KERNEL_BLOCK   # K up to 640, B row-major: any number of tiles
-    # 17 - 32 rows, a very long K, more than one round of the skinny kernel's workgroups; a very short K from 33 rows on
-    assert tk.kernel_choice(32, 14080, 26112, 0, 1) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(64, 10496, 1024, 0, 1) == tk.KERNEL_BLOCK
-    prev = tk.set_k_split(1)
+    assert tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.KERNEL_RING and tk.kernel_choice(64, 28672, 8192, 0, 0) == tk.KERNEL_RING
+    assert tk.kernel_choice(512, 8192, 8192, 1, 1) == tk.KERNEL_BLOCK
+    assert tk.kernel_choice(128, 512, 16384) == tk.CHOICE_BLOCK_K_SPLIT and tk.kernel_choice(256, 8192, 28672, 1, 1) == tk.CHOICE_TILED_K_SPLIT
+    prev = tk.set_k_split(1)   # no K split: neither the splits nor the ring kernel, whose shapes need one
     try:
-        assert tk.kernel_choice(512, 8192, 28672, 1, 1) == tk.KERNEL_BLOCK and tk.kernel_choice(64, 8192, 28672, 0, 1) == tk.KERNEL_SKINNY   # no split
+        assert tk.kernel_choice(128, 512, 16384) not in (tk.CHOICE_BLOCK_K_SPLIT, tk.CHOICE_TILED_K_SPLIT, tk.KERNEL_RING)
+        assert tk.kernel_choice(64, 8192, 28672, 0, 1) not in (tk.CHOICE_BLOCK_K_SPLIT, tk.CHOICE_TILED_K_SPLIT, tk.KERNEL_RING)
     finally:
         tk.set_k_split(prev)
 
@@ -551,16 +607,17 @@ def test_skinny_k_split_chosen_by_shape_streams_and_capture(hk):
 @pytest.mark.parametrize("block", [True, False])
 def test_k_split_streams_and_capture(hk, block):
     """A K split on a shape where the automatic path chooses one (a few hundred rows of A, long K) -- the block kernel's,
-    and with that kernel kept out of the choice the tiled kernel's: against the generic kernel; two streams at once, each
+    and with the tiled kernel forced, the tiled kernel's own: against the generic kernel; two streams at once, each
     with its own workspace of partial sums; under stream capture on a stream that has its workspace already (captured
     with the split) and replayed with eager work in between."""
     M, N, K = 192, 1024, 16384
-    prev_block = hk.tk_kernel.set_block_kernel(block)
+    tk = hk.tk_kernel
+    assert tk.kernel_choice(M, N, K) == tk.CHOICE_BLOCK_K_SPLIT and tk.k_split_plan(M, N, K)[0] > 1
+    prev = tk.set_kernel(tk.KERNEL_AUTO if block else tk.KERNEL_TILED)
     try:
-        assert hk.tk_kernel.kernel_choice(M, N, K) == (hk.tk_kernel.CHOICE_BLOCK_K_SPLIT if block else hk.tk_kernel.CHOICE_TILED_K_SPLIT)
         _k_split_streams_and_capture(hk, M, N, K)
     finally:
-        hk.tk_kernel.set_block_kernel(prev_block)
+        tk.set_kernel(prev)
 
 
 def test_capture_on_a_stream_without_workspace_runs_unsplit(hk):
@@ -597,7 +654,7 @@ def _k_split_streams_and_capture(hk, M, N, K):
     try:
         hk.dispatch_micro(a, b, asc, bsc, ref)
     finally:
-        hk.tk_kernel.set_kernel(prev)
+        hk.tk_kernel.set_kernel(prev)   # the caller's setting: automatic, or the tiled kernel forced
     torch.cuda.synchronize()
     refn = ref.cpu().numpy()
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
@@ -1223,7 +1280,7 @@ def test_measurement_probes_run_and_leave_results_alone(hk):
     gives the same bits as without."""
     from hipkittensp_amd import _lib
 
-    L = _lib.lib()
+    L = _lib.probes()
     M = N = 512
     K = 1024
     ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=77)
@@ -1241,11 +1298,11 @@ def test_measurement_probes_run_and_leave_results_alone(hk):
     assert L.mxfp6_probe_stream(buf.data_ptr(), buf.numel(), 512, 4, stats.data_ptr(), None) == 0
     assert L.mxfp6_probe_stream(buf.data_ptr(), buf.numel() - 8192, 256, 8, stats.data_ptr(), None) == -2
     torch.cuda.synchronize()
-    ref = gemm(hk, ap, bp, asc, bsc, kernel=2)
+    ref = gemm(hk, ap, bp, asc, bsc, kernel=2)   # the operator's own library
     assert L.mxfp6_probe_tiled_clock(stats.data_ptr()) == 0 and L.mxfp6_probe_raster(2, 0) == 0
     try:
         stats.zero_()
-        got = gemm(hk, ap, bp, asc, bsc, kernel=2)
+        got = gemm_probes_lib(ap, bp, asc, bsc, kernel=2)
         st = stats.cpu().numpy().astype(np.int64)
         assert (st[2] - st[0]) % 2**32 > 8 * 1024 and (st[3] - st[1]) % 2**32 > 0  # eight K-tiles of MFMA work at least
     finally:
@@ -1259,18 +1316,18 @@ def test_k_split_order_of_workgroups_does_not_change_the_result(hk, M, N, K, ker
     """(tile, share) pairs share by share with an eighth of that order per XCD (the library's own), tile by tile, and with
     no XCD remap at all: the same bits, and the oracle's values.  Workgroup counts that are multiples of eight take the
     remap (32, 24, 64 and 24 here); the fourth shape's 18 tiles x 3 shares do not, and its K % 512 != 0 gives a shorter last share."""
-    tk, L = hk.tk_kernel, hk._lib.lib()
+    L = hk._lib.probes()   # the raster override is the measurement build's
     ap, asc, bp, bsc = operands(M, N, K, 2, 2, seed=M + K, kind_b="weights")
     ref = o.gemm_ref(ap, bp, asc, bsc, 2, 2, acc=np.float64)
-    prev = tk.set_k_split(shares)
+    prev = L.mxfp6_set_k_split(shares)
     got = {}
     try:
         for xcd in (1, 2, 0):
             assert L.mxfp6_probe_raster(0, xcd) == 0
-            got[xcd] = gemm(hk, ap, bp, asc, bsc, kernel=kernel)
+            got[xcd] = gemm_probes_lib(ap, bp, asc, bsc, kernel=kernel)
     finally:
         L.mxfp6_probe_raster(0, 1)
-        tk.set_k_split(prev)
+        L.mxfp6_set_k_split(prev)
     check(got[1], ref, 2, 2, ap, asc, bp, bsc)
     assert np.array_equal(got[1], got[2]) and np.array_equal(got[1], got[0])
 
