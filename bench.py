@@ -418,7 +418,7 @@ def square_sizes(hk, torch, steps, warmup):
     return out
 
 
-def dispatch_sweep(hk, torch, full):
+def dispatch_sweep(hk, torch, grid):
     """How good is the automatic kernel choice?  For every shape of a grid (rows of A x a set of (N, K) pairs x both
     layouts of B; A row-major) the call is timed with the automatic choice (twice, before and after the others: the better
     of the two) and with every kernel / tile shape forced in turn, the tiled, the block and the ring kernel also with their K
@@ -426,7 +426,11 @@ def dispatch_sweep(hk, torch, full):
     the best forced time and which kernel that was, and the shapes where the automatic choice is more than 8 % behind.
     Small shapes (below about 15 us) are bound by the host side of the Python operator and only scatter."""
     tk = hk.tk_kernel
-    if full:
+    if grid == "offgrid":  # none of these (N, K) pairs and none of these row counts is in the calibration table
+        shapes = [(6144, 6144), (12288, 6144), (3072, 12288), (20480, 5120), (18432, 9216), (7168, 20480), (49152, 4096), (2560, 10240),
+                  (13824, 5120), (5120, 13824), (100352, 2048), (1536, 32768)]
+        rows_of_a = [12, 40, 80, 112, 160, 224, 320, 448, 640, 896, 1536, 3072]
+    elif grid == "full":
         shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096),
                   (8192, 28672), (2048, 8192), (5120, 16384), (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096)]
         rows_of_a = [8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 2048]
@@ -434,7 +438,7 @@ def dispatch_sweep(hk, torch, full):
         shapes = [(8192, 8192), (28672, 8192), (8192, 28672), (57344, 8192), (1024, 16384)]
         rows_of_a = [16, 32, 64, 128, 256, 512, 1024]
     forced = (("tiled", 2, 1), ("tiled_128x256", 5, 1), ("tiled_256x256", 6, 1), ("tiled_128x128", 17, 1), ("block", 22, 1), ("block_128x256", 26, 1), ("skinny", 3, 0), ("mid", 4, 0),
-              ("tiled_k_split", 2, -1), ("block_k_split", 22, -1), ("ring", tk.KERNEL_RING, 0))
+              ("tiled_k_split_256", 6, -1), ("tiled_k_split_128", 5, -1), ("block_k_split", 22, -1), ("ring", tk.KERNEL_RING, 0))
 
     def time_us(sets, C, lay, kernel, k_split, reps=10):
         prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
@@ -486,6 +490,90 @@ def dispatch_sweep(hk, torch, full):
     return {"what": "automatic kernel choice against every forced kernel, tile shape and K split; e2m3 x e2m3, bf16 out, A row-major", "shapes": len(per_shape),
             "within_8_percent": sum(1 for r in ratios if r <= 1.08), "median_auto_over_best": ratios[len(ratios) // 2], "worst_auto_over_best": ratios[-1],
             "behind_by_more_than_8_percent": behind, "per_shape": per_shape}
+
+
+CANDIDATES = (("tiled_256x256", 6, 1), ("tiled_128x256", 5, 1), ("tiled_128x128", 17, 1), ("block", 22, 1), ("block_128x256", 26, 1), ("skinny", 3, 0),
+              ("tiled_k_split_256", 6, -1), ("tiled_k_split_128", 5, -1), ("block_k_split", 22, -1), ("ring", 28, 0))  # in the order of the library's candidate numbers
+
+
+def calibration_sweep(hk, torch):
+    """The sweep behind the kernel choice's calibration table (hipkittensp_amd/csrc/dispatch_table.inc): every candidate of the
+    choice, forced, on a grid of shapes x three layout pairs, each timed twice (the better counts), next to the time model's
+    figure for it (mxfp6_probe_candidate of the measurement build).  `python -m hipkittensp_amd.calibrate` turns the JSON this
+    prints into the table: per shape and candidate, measured / modelled time."""
+    import ctypes
+
+    from hipkittensp_amd import _lib
+
+    tk, P = hk.tk_kernel, _lib.probes()
+    P.mxfp6_probe_candidate.restype = ctypes.c_int
+    P.mxfp6_probe_candidate.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
+    shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096), (8192, 28672), (2048, 8192), (5120, 16384),
+              (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096), (4096, 4096), (16384, 16384), (2048, 28672), (11008, 4096), (4096, 11008), (2048, 2048), (512, 8192), (8192, 1024),
+              (1024, 32768), (2048, 16384), (4096, 8192), (4096, 24576), (8192, 4096), (8192, 14336), (16384, 4096), (16384, 8192), (65536, 2048), (3072, 3072), (6144, 4096), (1024, 4096),
+              (12288, 12288), (2048, 5120), (24576, 2048), (73728, 4096)]
+    rows_of_a = [1, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 4096, 8192]
+
+    def time_us(ops, C, la, lb, kernel, k_split, reps=8):
+        prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
+        try:
+            for i in range(2):
+                hk.dispatch_micro(*ops[i % len(ops)], C, layout_a=la, layout_b=lb)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(reps):
+                hk.dispatch_micro(*ops[i % len(ops)], C, layout_a=la, layout_b=lb)
+            e1.record()
+            torch.cuda.synchronize()
+        except RuntimeError:
+            return None
+        finally:
+            tk.set_kernel(prev_k)
+            tk.set_k_split(prev_s)
+        return e0.elapsed_time(e1) / reps * 1e3
+
+    points = []
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    for N, K in shapes:
+        bs = [hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2) for _ in range(2)]
+        bts = [(hk.tile_operand(b), hk.tile_scales(sc, K)) for b, sc in bs]
+        for M in rows_of_a:
+            if M * N > 1 << 28:
+                continue
+            a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
+            C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+            for la, lb in ((0, 0), (0, 1), (1, 1)):
+                if la and (M % 32 or K % 128):
+                    continue
+                at, ast = (hk.tile_operand(a), hk.tile_scales(asc, K)) if la else (a, asc)
+                ops = [(at, (bts if lb else bs)[i][0], ast, (bts if lb else bs)[i][1]) for i in range(2)]
+                layouts = la | lb << 1
+                measured, model = [], []
+                for cand, (name, kernel, k_split) in enumerate(CANDIDATES):
+                    m, c, sh = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
+                    prev = P.mxfp6_set_k_split(k_split)
+                    rc = P.mxfp6_probe_candidate(M, N, K, layouts, cand, 0, ctypes.byref(m), ctypes.byref(c), ctypes.byref(sh))
+                    P.mxfp6_set_k_split(prev)
+                    assert rc == 0, rc
+                    t = None
+                    if m.value >= 0:
+                        t = time_us(ops, C, la, lb, kernel, k_split)
+                        t2 = time_us(ops, C, la, lb, kernel, k_split) if t is not None else None
+                        t = min(t, t2) if t2 is not None else t
+                    measured.append(round(t, 2) if t is not None else None)
+                    model.append(round(m.value, 2) if m.value >= 0 else None)
+                auto = time_us(ops, C, la, lb, 0, 0)
+                point = {"M": M, "N": N, "K": K, "layouts": layouts, "measured_us": measured, "model_us": model, "auto_us": round(auto, 2), "choice": tk.kernel_choice(M, N, K, la, lb)}
+                if measured[-1] is not None:  # the ring kernel as one share of K: not a candidate of its own, a point for the model's per-workgroup rate
+                    one = time_us(ops, C, la, lb, CANDIDATES[-1][1], 1)
+                    point["ring_one_share_us"] = round(one, 2) if one is not None else None
+                points.append(point)
+        del bs, bts
+        torch.cuda.empty_cache()
+    return {"what": "calibration sweep of the kernel choice: measured and modelled microseconds per candidate", "candidates": [c[0] for c in CANDIDATES],
+            "device": torch.cuda.get_device_name(0), "cus": torch.cuda.get_device_properties(0).multi_processor_count, "points": points}
 
 
 def source_hash(kernel):
@@ -557,7 +645,7 @@ def main():
     p.add_argument("--sweep-settings", choices=["all", "default", "ksplit-order"], default="all",
                    help="with --raster-sweep: all raster settings, only the kernel's own (to compare schedules under a profiler), or the kernel's own and, as "
                         "xcd_remap=2, a K split's workgroups in tile-by-tile order instead of share by share (for shapes that take a K split)")
-    p.add_argument("--dispatch-sweep", choices=["small", "full"], default=None,
+    p.add_argument("--dispatch-sweep", choices=["small", "full", "offgrid", "calibrate"], default=None,
                    help="only compare the automatic kernel choice with every forced kernel / tile shape / K split over a grid of shapes and print one JSON line")
     p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the decode run with tile-major weights (used for profiling one layout of the skinny kernel)")
     p.add_argument("--profile-kernels", action="store_true", help="only loops of the tiled kernel (8192^3, tile-major), the skinny kernel (configs[3], row-major) and the ring "
@@ -582,8 +670,11 @@ def main():
     _lib.lib()  # fail loudly if the HIP library is missing
     tk = hk.tk_kernel
 
+    if args.dispatch_sweep == "calibrate":
+        print(json.dumps(calibration_sweep(hk, torch)))
+        return
     if args.dispatch_sweep:
-        print(json.dumps(dispatch_sweep(hk, torch, args.dispatch_sweep == "full")))
+        print(json.dumps(dispatch_sweep(hk, torch, args.dispatch_sweep)))
         return
 
     cfg1 = CONFIGS["cfg1"]

@@ -20,7 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmxfp6_gemm.so")
 PROBES_LIB = os.path.join(HERE, "libmxfp6_probes.so")
-SOURCES = ["api.hip", "gemm_generic.hip", "gemm_tiled.hip", "gemm_tiled4.hip", "gemm_block.hip", "gemm_mid.hip", "gemm_skinny.hip", "gemm_ring.hip", "quantize.hip"]
+SOURCES = ["api.hip", "dispatch.hip", "gemm_generic.hip", "gemm_tiled.hip", "gemm_tiled4.hip", "gemm_block.hip", "gemm_mid.hip", "gemm_skinny.hip", "gemm_ring.hip", "quantize.hip"]
 # (source, object name, extra flags).  gemm_tiled.hip gives five objects: its host-side part, and the kernel
 # instantiations of each pair of operand formats (the bulk of the build time; they compile side by side).
 UNITS = [(src, src.replace(".hip", ""), []) for src in SOURCES] + [

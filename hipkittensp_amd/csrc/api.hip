@@ -108,87 +108,84 @@ uint8_t* stream_workspace(hipStream_t s, int kind, size_t bytes, bool zeroed = f
   return p;
 }
 
-// The tiled kernel's K split for this call, if its shape wants one and this stream has (or can get) the workspace:
-// fills in g.ksplit, g.tile_rows and the workspace pointer.
-void plan_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
-  int rows = 0;
-  size_t part = 0;
-  const int shares = mxfp6::tiled_ksplit_plan(g, g_ksplit, &rows, &part);
-  if (shares <= 1) return;
-  uint8_t* pp = stream_workspace(s, 2, part);
-  if (!pp) return;
-  g.ksplit = shares, g.tile_rows = rows, g.tile_cols = 256;
-  g.ks_part = reinterpret_cast<float*>(pp);
-}
+// Candidate sets of the kernel choice (bits of mxfp6::Candidate)
+constexpr unsigned kTiledUnsplit = 1u << mxfp6::kCandTiled256 | 1u << mxfp6::kCandTiled128x256 | 1u << mxfp6::kCandTiled128x128;
+constexpr unsigned kTiledSplits = 1u << mxfp6::kCandTiledSplit256 | 1u << mxfp6::kCandTiledSplit128;
+constexpr unsigned kTiledFamily = kTiledUnsplit | kTiledSplits;
+constexpr unsigned kBlockFamily = 1u << mxfp6::kCandBlock | 1u << mxfp6::kCandBlockSplit;
+constexpr unsigned kBlockAll = kBlockFamily | 1u << mxfp6::kCandBlockWide;
+constexpr unsigned kNeedsWorkspace = kTiledSplits | 1u << mxfp6::kCandBlockSplit;
 
-// The block kernel's K split for this call, likewise.
-void plan_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
-  size_t part = 0;
-  const int shares = mxfp6::block_ksplit_plan(g, g_ksplit, &part);
-  if (shares <= 1) return;
-  uint8_t* pp = stream_workspace(s, 2, part);
-  if (!pp) return;
-  g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp);
-}
-// The ring kernel's K split, likewise.
-// returns false when the plan is a split whose workspace is not to be had (capture, allocator): then nothing is set
-bool plan_ring_ksplit(mxfp6::GemmArgs& g, hipStream_t s) {
-  size_t part = 0, counters = 0;
-  const int shares = mxfp6::ring_ksplit_plan(g, g_ksplit, &part, &counters);
-  if (shares <= 1) return true;
-  uint8_t* pp = stream_workspace(s, 2, part);
-  uint8_t* pc = pp ? stream_workspace(s, 3, counters * sizeof(int), true) : nullptr;
-  if (!pc) return false;
-  g.ksplit = shares, g.ks_part = reinterpret_cast<float*>(pp), g.ks_counters = reinterpret_cast<int*>(pc);
-  return true;
-}
-bool launch_block_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
-  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
-  plan_block_ksplit(g, s);
-  if (g.ksplit <= 1) return false;
-  e = mxfp6::launch_gemm_block(g, s);
-  return true;
-}
-
-// Automatic path: launches the tiled kernel with its K split if the shape calls for one (and the workspace is there).
-bool launch_tiled_ksplit(mxfp6::GemmArgs& g, hipStream_t s, hipError_t& e) {
-  if (g.no_alloc || g.K == 0 || !mxfp6::gemm_tiled_supports(g)) return false;
-  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
-  plan_ksplit(g, s);
-  if (g.ksplit <= 1) return false;
-  e = mxfp6::launch_gemm_tiled(g, s);
-  return true;
-}
-
-// The kernel the automatic path takes for a call, by shape, layouts and alignment alone (codes of mxfp6_set_kernel; the
-// tiled kernel with its K split: kChoiceTiledKsplit).  allow_ksplit = false: what it takes when the split's workspace is
-// not to be had (a stream that is being captured, the allocator's refusal).
-constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceMid = 4, kChoiceBlock = 22, kChoiceTiledKsplit = 25, kChoiceBlockWide = 26, kChoiceBlockKsplit = 27, kChoiceRing = 28;
-int auto_choice(const mxfp6::GemmArgs& g, int force_split, bool allow_ksplit) {
-  if (g.K == 0) return kChoiceGeneric;  // act(bias) everywhere: the generic kernel's K loop runs zero times
-  const bool block = g_block && !force_split;  // the block kernel may be chosen
-  // weights streamed from HBM against a few dozen rows of A: private streams of B per wave (its K split needs no workspace to
-  // be correct: without one it runs unsplit, which the shapes it is chosen for would not survive, so only with one)
-  if (!force_split && allow_ksplit && g_ksplit != 1 && mxfp6::gemm_ring_preferred(g)) return kChoiceRing;
-  // 128 x 128 tiles on at most half the CUs: the block kernel with its K split between workgroups
-  if (block && allow_ksplit) {
-    size_t part = 0;
-    if (mxfp6::block_ksplit_plan(g, g_ksplit, &part) > 1) return kChoiceBlockKsplit;
+// Codes mxfp6_kernel_choice reports (those of mxfp6_set_kernel; 25 / 27: the tiled / the block kernel with its K split)
+constexpr int kChoiceGeneric = 1, kChoiceTiled = 2, kChoiceSkinny = 3, kChoiceBlock = 22, kChoiceTiledKsplit = 25, kChoiceBlockWide = 26, kChoiceBlockKsplit = 27, kChoiceRing = 28;
+int choice_code(const mxfp6::KernelChoice& c) {
+  switch (c.cand) {
+    case mxfp6::kCandTiled256: case mxfp6::kCandTiled128x256: case mxfp6::kCandTiled128x128: return kChoiceTiled;
+    case mxfp6::kCandBlock: return kChoiceBlock;
+    case mxfp6::kCandBlockWide: return kChoiceBlockWide;
+    case mxfp6::kCandSkinny: return kChoiceSkinny;
+    case mxfp6::kCandTiledSplit256: case mxfp6::kCandTiledSplit128: return kChoiceTiledKsplit;
+    case mxfp6::kCandBlockSplit: return kChoiceBlockKsplit;
+    case mxfp6::kCandRing: return kChoiceRing;
+    default: return kChoiceGeneric;
   }
-  // 128 x 128 tiles that fill more than half the CUs (a quarter with K <= 8192), K of moderate length: ahead of the K split too
-  if (block && mxfp6::gemm_block_preferred(g, true)) return kChoiceBlock;
-  // few output tiles, long K: the tiled kernel with K split between workgroups (before the skinny and mid-M kernels,
-  // which it beats there; the plan leaves up to 64 rows of a row-major A to the skinny kernel)
-  if (!force_split && allow_ksplit && !g.no_alloc && mxfp6::gemm_tiled_supports(g)) {
-    int rows = 0;
-    size_t part = 0;
-    if (mxfp6::tiled_ksplit_plan(g, g_ksplit, &rows, &part) > 1) return kChoiceTiledKsplit;
+}
+
+// What the automatic path may choose from for a call.  force_split: the entry point that allocates nothing fixes the skinny
+// kernel's split (1 = never split): no kernel that needs a workspace, and the skinny kernel whenever a split is asked for.
+unsigned auto_mask(const mxfp6::GemmArgs& g, int force_split) {
+  unsigned mask = ~0u;
+  if (!g_block || force_split) mask &= ~kBlockAll;
+  if (force_split || g.no_alloc) mask &= ~(kNeedsWorkspace | 1u << mxfp6::kCandRing);
+  if (force_split > 1 && mxfp6::gemm_skinny_supports(g)) mask = 1u << mxfp6::kCandSkinny;
+  return mask;
+}
+
+// The choice for a call: by the time model and the calibration table (dispatch.hip).  allow_split = false: what it is when a
+// K split's workspace is not to be had (a stream that is being captured, the allocator's refusal).
+mxfp6::KernelChoice auto_choice(const mxfp6::GemmArgs& g, int force_split, bool allow_split) {
+  if (g.K == 0) return {-1, 1, 0, 0.0};  // act(bias) everywhere: the generic kernel's K loop runs zero times
+  return mxfp6::choose_kernel(g, g_ksplit, allow_split, auto_mask(g, force_split));
+}
+
+// Sets a call up as the choice says: tile shape, K split and its workspace.  false: the split's workspace is not to be had.
+bool apply_choice(mxfp6::GemmArgs& g, const mxfp6::KernelChoice& c, hipStream_t s) {
+  switch (c.cand) {
+    case mxfp6::kCandTiled256: g.tile_rows = 256, g.tile_cols = 256; return true;
+    case mxfp6::kCandTiled128x256: g.tile_rows = 128, g.tile_cols = 256; return true;
+    case mxfp6::kCandTiled128x128: g.tile_rows = 128, g.tile_cols = 128; return true;
+    case mxfp6::kCandBlockWide: g.tile_cols = 256; return true;
+    case mxfp6::kCandTiledSplit256: case mxfp6::kCandTiledSplit128: case mxfp6::kCandBlockSplit: {
+      uint8_t* pp = stream_workspace(s, 2, (size_t)c.shares * g.M * g.N * sizeof(float));
+      if (!pp) return false;
+      g.ksplit = c.shares, g.ks_part = reinterpret_cast<float*>(pp);
+      if (c.cand != mxfp6::kCandBlockSplit) g.tile_rows = c.rows, g.tile_cols = 256;
+      return true;
+    }
+    case mxfp6::kCandRing: {
+      if (c.shares <= 1) return true;
+      size_t part = 0, counters = 0;
+      if (mxfp6::ring_ksplit_plan(g, c.shares, &part, &counters) != c.shares) return false;
+      uint8_t* pp = stream_workspace(s, 2, part);
+      uint8_t* pc = pp ? stream_workspace(s, 3, counters * sizeof(int), true) : nullptr;
+      if (!pc) return false;
+      g.ksplit = c.shares, g.ks_part = reinterpret_cast<float*>(pp), g.ks_counters = reinterpret_cast<int*>(pc);
+      return true;
+    }
+    default: return true;
   }
-  if (block && mxfp6::gemm_block_preferred(g, false)) return kChoiceBlock;
-  if (block && mxfp6::gemm_block_wide_preferred(g)) return kChoiceBlockWide;
-  if (mxfp6::gemm_skinny_preferred(g) || (force_split > 1 && mxfp6::gemm_skinny_supports(g))) return kChoiceSkinny;
-  if (!mxfp6::gemm_wide_n_prefers_tiled(g) && (mxfp6::gemm_mid_preferred(g) || (mxfp6::gemm_mid_supports(g) && !mxfp6::gemm_tiled_supports(g)))) return kChoiceMid;
-  return mxfp6::gemm_tiled_supports(g) ? kChoiceTiled : kChoiceGeneric;
+}
+
+// A forced kernel family with this thread's K-split setting: 0 = the family's split where the model prefers it to the
+// family's unsplit form, -1 / n = the split wherever the shape has one, 1 = never.  The tile shape of a forced tiled kernel
+// without one (mxfp6_set_kernel 2) is the model's choice as well.
+mxfp6::KernelChoice family_choice(const mxfp6::GemmArgs& g, unsigned unsplit, unsigned splits) {
+  mxfp6::KernelChoice c = mxfp6::choose_kernel(g, g_ksplit, true, unsplit | (g_ksplit != 1 ? splits : 0u));
+  if (g_ksplit != 0 && g_ksplit != 1 && !(splits >> c.cand & 1)) {  // the split is wanted wherever possible
+    const mxfp6::KernelChoice forced = mxfp6::choose_kernel(g, g_ksplit, true, splits);
+    if (forced.cand >= 0) c = forced;
+  }
+  return c;
 }
 
 hipError_t release_stream_workspaces() {
@@ -326,15 +323,17 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
   const int force = no_alloc ? 0 : g_force;  // the entry point that allocates nothing takes no override
   hipError_t e;
   if (no_alloc && force_split > 1 && !(M <= 32 && mxfp6::gemm_skinny_supports(g))) return MXFP6_EINVAL_SHAPE;
-  if (no_alloc && (force_split || mxfp6::gemm_skinny_preferred(g)) && mxfp6::gemm_skinny_supports(g) && !mxfp6::gemm_skinny_scratch_fits(g)) return MXFP6_ESCRATCH;
+  if (no_alloc && mxfp6::gemm_skinny_supports(g) && (force_split || auto_choice(g, force_split, false).cand == mxfp6::kCandSkinny) && !mxfp6::gemm_skinny_scratch_fits(g)) return MXFP6_ESCRATCH;
+  std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
   if (K != 0 && force == 1) {
     e = mxfp6::launch_gemm_generic(g, s);
   } else if (K != 0 && (force == 2 || force == 5 || force == 6 || force == 17)) {
     if (!mxfp6::gemm_tiled_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
-    std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
-    plan_ksplit(g, s);
-    e = mxfp6::launch_gemm_tiled(g, s);
+    const unsigned shapes = force == 2 ? kTiledUnsplit : 1u << (force == 6 ? mxfp6::kCandTiled256 : force == 5 ? mxfp6::kCandTiled128x256 : mxfp6::kCandTiled128x128);
+    mxfp6::KernelChoice c = family_choice(g, shapes, kTiledSplits);
+    if (!apply_choice(g, c, s)) apply_choice(g, mxfp6::choose_kernel(g, 1, false, shapes), s);
+    if (g.ksplit > 1 || !relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
   } else if (K != 0 && (force == 3 || (force >= 7 && force <= 16) || (force >= 19 && force <= 21))) {
     if (!mxfp6::gemm_skinny_supports(g)) return MXFP6_EINVAL_SHAPE;
     g.skinny_geometry = force == 3 ? 0 : force >= 19 ? force - 8 : force - 6;
@@ -347,38 +346,29 @@ int gemm_common(const void* A, const void* B, const void* As, const void* Bs, vo
     e = mxfp6::launch_gemm_tiled4(g, s);
   } else if (K != 0 && force == 28) {
     if (!mxfp6::gemm_ring_supports(g)) return MXFP6_EINVAL_SHAPE;
-    std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
-    (void)plan_ring_ksplit(g, s);  // without a workspace: unsplit
+    (void)apply_choice(g, mxfp6::choose_kernel(g, g_ksplit, true, 1u << mxfp6::kCandRing), s);  // without a workspace: unsplit
     e = mxfp6::launch_gemm_ring(g, s);
   } else if (K != 0 && ((force >= 22 && force <= 24) || force == 26)) {
     if (!mxfp6::gemm_block_supports(g)) return MXFP6_EINVAL_SHAPE;
+    if (force != 26) (void)apply_choice(g, family_choice(g, 1u << mxfp6::kCandBlock, 1u << mxfp6::kCandBlockSplit), s);  // without a workspace: unsplit
     g.tile_rows = force == 23 ? 3 : force == 24 ? 6 : 0, g.tile_cols = force == 26 ? 256 : 0;
-    std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // a K split writes and then reads this stream's workspace
-    if (force != 26) plan_block_ksplit(g, s);
     e = mxfp6::launch_gemm_block(g, s);
   } else {
-    int choice = auto_choice(g, force_split, true);
-    // the split needs this stream's workspace: without it, what the shape gets otherwise
-    if (choice == kChoiceBlockKsplit && !launch_block_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
-    if (choice == kChoiceTiledKsplit && !launch_tiled_ksplit(g, s, e)) choice = auto_choice(g, force_split, false);
-    if (choice == kChoiceRing) {
-      std::lock_guard<std::recursive_mutex> launch_lock(g_sws_launch_mutex);  // the split writes and then reads this stream's workspace
-      if (plan_ring_ksplit(g, s)) e = mxfp6::launch_gemm_ring(g, s);
-      else choice = auto_choice(g, force_split, false);  // no workspace (capture, allocator): what the shape gets otherwise
+    mxfp6::KernelChoice c = auto_choice(g, force_split, true);
+    // a split needs this stream's workspace: without it, what the shape gets otherwise
+    if (!apply_choice(g, c, s)) {
+      c = auto_choice(g, force_split, false);
+      (void)apply_choice(g, c, s);
     }
-    if (choice == kChoiceBlock) {
-      e = mxfp6::launch_gemm_block(g, s);
-    } else if (choice == kChoiceBlockWide) {
-      g.tile_cols = 256;
-      e = mxfp6::launch_gemm_block(g, s);
-    } else if (choice == kChoiceSkinny) {
-      e = mxfp6::launch_gemm_skinny(g, s);
-    } else if (choice == kChoiceMid) {
-      e = mxfp6::launch_gemm_mid(g, s);
-    } else if (choice == kChoiceTiled) {
-      if (!relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
-    } else if (choice == kChoiceGeneric) {
-      e = mxfp6::launch_gemm_generic(g, s);
+    switch (c.cand) {
+      case mxfp6::kCandTiled256: case mxfp6::kCandTiled128x256: case mxfp6::kCandTiled128x128:
+        if (!relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
+        break;
+      case mxfp6::kCandTiledSplit256: case mxfp6::kCandTiledSplit128: e = mxfp6::launch_gemm_tiled(g, s); break;
+      case mxfp6::kCandBlock: case mxfp6::kCandBlockWide: case mxfp6::kCandBlockSplit: e = mxfp6::launch_gemm_block(g, s); break;
+      case mxfp6::kCandSkinny: e = mxfp6::launch_gemm_skinny(g, s); break;
+      case mxfp6::kCandRing: e = mxfp6::launch_gemm_ring(g, s); break;
+      default: e = mxfp6::launch_gemm_generic(g, s); break;
     }
   }
   return e == hipSuccess ? MXFP6_OK : (int)e;
@@ -430,12 +420,14 @@ int mxfp6_gemm_fused_fp6(const void* A, const void* B, const void* As, const voi
   // small there) the product goes to an fp32 workspace of the stream-ordered allocator and through the quantiser
   mxfp6::GemmArgs g{(const uint8_t*)A, (const uint8_t*)B, (const uint8_t*)As, (const uint8_t*)Bs, C_packed, M, N, K, fmt_a, fmt_b, false, layout_a, layout_b};
   const int force = g_force;
+  // the tiled kernel's own fp6 epilogue only where the automatic choice is that kernel (unsplit); any other choice runs as
+  // it would for an fp32 output, into the workspace, and the quantiser follows
   const bool tiled = K > 0 && mxfp6::gemm_tiled_supports(g) &&
-                     (force == 2 || force == 5 || force == 6 || force == 17 ||
-                      (force == 0 && !mxfp6::gemm_skinny_preferred(g) && !mxfp6::gemm_mid_preferred(g)));
+                     (force == 2 || force == 5 || force == 6 || force == 17 || (force == 0 && choice_code(auto_choice(g, 0, true)) == kChoiceTiled));
   if (tiled) {
     g.ep = ep, g.C_scale = (uint8_t*)C_scale, g.fmt_c = fmt_c;
     g.tile_rows = force == 5 || force == 17 ? 128 : force == 6 ? 256 : 0, g.tile_cols = force == 17 ? 128 : 0;
+    if (force == 0 || force == 2) (void)apply_choice(g, mxfp6::choose_kernel(g, 1, false, kTiledUnsplit), s);  // the tile height (the fp6 epilogue needs 256 columns)
     hipError_t e;
     if (force != 0 || !relayout_then_tiled(g, s, e)) e = mxfp6::launch_gemm_tiled(g, s);
     return e == hipSuccess ? MXFP6_OK : (int)e;
@@ -593,7 +585,7 @@ int mxfp6_kernel_choice(int M, int N, int K, int layouts) {
   // aligned stand-ins for the pointers: the choice looks at their alignment only
   const uint8_t* p = reinterpret_cast<const uint8_t*>((uintptr_t)4096);
   mxfp6::GemmArgs g{p, p, p, p, const_cast<uint8_t*>(p), M, N, K, 2, 2, false, layout_a, layout_b};
-  return auto_choice(g, 0, true);
+  return choice_code(auto_choice(g, 0, true));
 }
 
 #ifdef MXFP6_PROBES  // ---- measurement entry points (include/mxfp6_probes.h)
@@ -612,11 +604,25 @@ int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int* t
   const int rc = check_device();
   if (rc) return rc;
   mxfp6::GemmArgs g{nullptr, nullptr, nullptr, nullptr, nullptr, M, N, K, 2, 2, false, layout_a, layout_b};
-  int rows = 0;
-  size_t part = 0;
-  const int n = N % 8 == 0 && K % 128 == 0 ? mxfp6::tiled_ksplit_plan(g, shares, &rows, &part) : 1;
+  int rows = 0, n = 1;
+  // shares == 0: the split where the model prefers it to the tiled kernel's unsplit tiles; else the better of the two tile heights' splits
+  const mxfp6::KernelChoice c = mxfp6::choose_kernel(g, shares, true, shares == 0 ? kTiledFamily : kTiledSplits);
+  if (c.cand >= 0 && (kTiledSplits >> c.cand & 1)) n = c.shares, rows = c.rows;
   if (tile_rows) *tile_rows = n > 1 ? rows : 0;
   return n;
+}
+
+int mxfp6_probe_candidate(int M, int N, int K, int layouts, int candidate, int cus, double* model_us, double* calibrated_us, int* shares) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 32 || candidate < 0 || candidate >= mxfp6::kNumCandidates || cus < 0) return MXFP6_EINVAL_SHAPE;
+  if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;
+  if (!model_us || !calibrated_us || !shares) return MXFP6_EINVAL_PTR;
+  const uint8_t* p = reinterpret_cast<const uint8_t*>((uintptr_t)4096);  // aligned stand-ins: the candidates look at the alignment only
+  mxfp6::GemmArgs g{p, p, p, p, const_cast<uint8_t*>(p), M, N, K, 2, 2, false, layouts & 1, layouts >> 1};
+  int rows = 0;
+  *model_us = mxfp6::candidate_model_us(g, candidate, g_ksplit, cus ? cus : mxfp6::device_cus(), shares, &rows);
+  const mxfp6::KernelChoice c = mxfp6::choose_kernel(g, g_ksplit, true, 1u << candidate);
+  *calibrated_us = c.cand == candidate ? c.us : -1.0;
+  return MXFP6_OK;
 }
 
 int mxfp6_probe_block(int enable) {

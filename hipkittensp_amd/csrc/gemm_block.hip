@@ -439,212 +439,6 @@ bool gemm_block_supports(const GemmArgs& g) {
          !g.no_alloc;
 }
 
-// Automatic choice, from a sweep of 64 - 2048 rows of A against fourteen (N, K) pairs on MI355X (us, the kernel chosen
-// before -> this one): the kernel wins where its tiles do not outnumber the CUs and K is not so long that splitting it
-// between workgroups (tiled kernel) or the skinny kernel wins.  Both operands tile-major: 256 x 8192 x 8192 31.7 -> 23,
-// 512 x 8192 x 8192 33 -> 29, 512 x 4096 x 4096 17.2 -> 14.1, 1024 x 2048 x 8192 32 -> 23.5, 64 .. 1024 rows at K <= 5120
-// 0.75 - 0.86 of the time; up to 128 rows only for K <= 8192 (beyond, the K split is ahead).  A row-major, B tile-major:
-// more than 128 rows 0.81 - 0.9 (256 x 8192 x 8192 0.89, 512 x 6144 x 16384 0.80); up to 128 rows only at K <= 2048, or
-// K <= 4096 against 12288 rows of B or more (0.86 - 0.96), the skinny kernel's otherwise (64 x 4096 x 4096: 1.37).  B
-// row-major: more than 256 rows and K <= 5120 0.87 - 0.93, tiles on three quarters of the CUs and K <= 16384
-// (512 x 6144 x 16384 85 -> 67), K <= 4096 against 12288 rows of B or more 0.84 - 0.92; otherwise level or behind.  More
-// tiles than CUs: level with the 8-wave kernel's 128 x 256 tiles up to 512 tiles, behind beyond; not chosen.
-// first: asked before the tiled kernel's K split is considered -- where the tiles fill more than half the CUs, K is at
-// most 16384 and both operands are tile-major this kernel is ahead of the split as well (640 x 4096 x 14336 0.85,
-// 384 x 6144 x 16384 0.84; with a row-major operand 0.92 - 1.11: left to the split), and with K up to
-// 8192 from a quarter of the CUs on (192 x 8192 x 8192 30.7 -> 22.5, 1024 x 2048 x 8192 32 -> 23.5; not with many rows of
-// a row-major A: 512 x 2048 x 8192 24.3 -> 28.8); with fewer tiles or a longer K the split wins (256 x 8192 x 28672 1.38,
-// 256 x 6144 x 16384 1.02, 256 x 4096 x 14336 1.11).
-bool gemm_block_preferred(const GemmArgs& g, bool first) {
-  if (!gemm_block_supports(g) || g.ablation || g.clock_stamps) return false;
-  const int cus = cu_count_of_device();
-  const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
-  const int nkt = g.K / kBK;
-  // (up to twice as many tiles as CUs for K up to 2048 with both operands tile-major: two workgroups share a CU, one round;
-  // us, the 128 x 256 tiles -> this: 4096 x 2048 x 1024 16.4 -> 12.9, 1024 x 8192 x 1024 17.1 -> 13.3, 2048 x 4096 x 2048 20.6 -> 18.9)
-  const bool short_k = nkt <= 16 && g.layout_a && g.layout_b;
-  // (K up to 640 against a row-major B: any number of tiles -- the launch is prologue and epilogue, and two of these
-  // workgroups share a CU; us, tiled kernel -> this: 640 x 24192 x 640 23.9 -> 19.9, 2048 x 26624 x 640 68.4 -> 57.0,
-  // 768 x 5888 x 512 10.5 -> 9.3, 256 x 25216 x 512 11.8 -> 10.7)
-  // (not where the tiled kernel's 256 x 256 tiles make one round on three quarters of the CUs or more: 512 x 28928 x 512,
-  // 226 of them, 15.1 us there against 18.0 here)
-  const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  const bool very_short_k = nkt <= 5 && !g.layout_b && !(tiles256 <= cus && tiles256 * 4 >= (long)cus * 3);
-  if (cus <= 0 || (!very_short_k && tiles > (short_k ? 2 * cus : cus))) return false;
-  // tiles on more than half the CUs (three quarters with a row-major B), K up to 16384
-  const bool fills = nkt <= 128 && (g.layout_b ? tiles * 16 >= (long)cus * 9 : tiles * 4 >= (long)cus * 3);
-  // ... or on a quarter of them, K up to 8192 (a row-major A: up to 256 rows of it)
-  const bool quarter = nkt <= 64 && tiles * 4 >= cus && g.layout_b && (g.layout_a || g.M <= 256);
-  if (first && !(fills && g.layout_a && g.layout_b) && !quarter) return false;
-  bool wide_short = nkt <= 32 && g.N >= 12288;
-  if (!g.layout_b) {
-    // more than 256 rows up to K = 5120, more than 128 where the tiles fill the CUs
-    if ((g.M > 256 && nkt <= 40) || (g.M > 128 && fills)) return true;
-    // K up to 2048 wherever the skinny kernel does not come first: 160 x 9216 x 1536 10.1 us on the tiled kernel -> 8.9,
-    // 96 x 4840 x 1792 9.9 -> 8.1, 24 x 12032 x 768 6.9 -> 6.1
-    // (up to K = 3072 likewise: 96 x 2952 x 2432 11.5 -> 8.8, 96 x 21352 x 2304 14.1 -> 13.2, 96 x 18048 x 3072 16.4 -> 15.2)
-    // (and K up to 1024 from 33 rows on, as against a tile-major B: 48 x 15872 x 512 6.8 us on the skinny kernel -> 6.0)
-    if ((nkt <= 24 && (g.M > 128 || !gemm_skinny_preferred(g))) || (nkt <= 8 && g.M > 32)) return true;
-    // K up to 4096 against 12288 rows of B or more: from 65 rows on, from 24 with tiles on five eighths of the CUs
-    // (24 x 28672 x 4096 21.1 us on the skinny kernel -> 18.5, 16 rows level)
-    if (wide_short && (g.M > 64 || (g.M >= 24 && tiles * 8 >= (long)cus * 5))) return true;
-    // up to 64 rows and a K the skinny kernel cannot take (K % 512 != 0), against the
-    // tiled kernel: 8 x 21624 x 2688 13.3 us -> 11.4, 4 x 20224 x 13184 66.3 -> 60.2, 32 x 30976 x 7424 49.5 -> 44.3
-    // (96 - 128 rows the other way: 96 x 20736 x 12672 80.2 -> 83.9)
-    // (with few tiles as well: 24 x 6992 x 4864, 55 tiles, 19.3 -> 16.9)
-    if (g.M <= 64 && !gemm_skinny_supports(g)) return true;
-    // from 32 rows on with tiles on more than half the CUs, up to K = 10240 (48 x 18816 x 4608 27.2 us on the skinny kernel
-    // -> 18.9, 48 x 23280 x 9216 53.9 -> 51.9; beyond, 64 x 22784 x 10752 60.9 -> 62.8, 64 x 16640 x 16384 82.2 -> 89.3);
-    // 32 rows, the skinny kernel's largest single row group, only up to K = 7168 (32 x 24576 x 8192 38.9 -> 43.3)
-    return g.M >= 32 && tiles * 2 > cus && tiles < cus && nkt <= (g.M > 32 ? 80 : 56) && gemm_skinny_preferred(g);
-  }
-  // (A tile-major: neither the skinny nor the mid-M kernel takes it, and against the tiled kernel's 256-row tiles this one
-  // wins for any K once the splits have been asked: 32 x 14592 x 11904 47.2 us -> 35.4, 32 x 27008 x 21248 89.0 -> 75.4)
-  if (g.layout_a) return g.M > 128 || nkt <= 64 || !first;
-  // A row-major, B tile-major, few rows: the skinny kernel's (where it takes the shape: K % 512 == 0; 16 x 4096 x 11008
-  // otherwise went to the tiled kernel, 35 us against 26 here), except a short K (above) and a B of 20480 .. 32767 rows
-  // (its tiles on more than half the CUs, one CU at least left over: the skinny kernel's workgroups of 32 rows of B then
-  // need a third round that is mostly empty): 32 x 20480 x 8192 38.3 -> 30.7 us, 16 x 28672 x 8192 37.9 -> 33.6,
-  // 32 x 28672 x 16384 74.6 -> 66.3, 48 x 18944 x 5120 28.1 -> 16.1, 32 x 18944 x 8192 36.5 -> 29.0 (16 rows level);
-  // 16384 rows 21 -> 26, 32768 rows level.  K up to 2048: from 65 rows on, or with that many tiles (up to 64 rows the
-  // skinny kernel is 10 - 20 % ahead: 48 x 4096 x 2048 6.1 us against 7.8)
-  // (K = 5120 as well from 65 rows on: 96 x 14336 x 5120 20.9 us on the tiled kernel -> 18.9, 128 x 12288 x 5120 22.4 -> 20.4)
-  // (and from 10240 rows of B: 96 x 11008 x 3584 18.0 us on the skinny kernel -> 14.1, 128 x 11008 x 5120 22.1 on the tiled kernel -> 20.1)
-  wide_short = wide_short || (nkt <= 40 && g.M > 64 && g.N >= 10240);
-  // (up to 31 rows only from five eighths of the CUs on: 1 x 20736 x 6144 18.9 us on the skinny kernel, 25.0 here)
-  // (from 32 rows on a tile for every CU as well: 48 x 32768 x 12288 63.6 us on the tiled kernel, 70.6 on the skinny kernel -> 58.7)
-  // (K beyond 16384: from 32 rows on as well, 32 x 16640 x 28672 102 us on the skinny kernel -> 91.7; with fewer rows
-  // only up to K = 20480 with tiles on thirteen sixteenths of the CUs, 16 x 27392 x 19456 81.6 -> 70.9, 8 x 27904 x 18944
-  // 76.2 -> 69.9; 16 x 23808 x 19968 level, 8 x 16640 x 28672 76.4 -> 79.6)
-  // (17 - 31 rows like 32, the skinny kernel handles them as 32: 24 x 19968 x 14848 57.9 us there -> 48.0)
-  const bool many_tiles = g.M > 16 ? tiles * 2 > cus && tiles <= cus && nkt <= 256
-                                    : tiles * 8 >= (long)cus * 5 && tiles < cus && (nkt <= 128 || (nkt <= 160 && tiles * 16 >= (long)cus * 13));
-  // (K up to 1024 from 33 rows on: 64 x 10496 x 1024 7.4 us on the skinny kernel -> 5.9)
-  return g.M > 128 || (nkt <= 16 && (g.M > 64 || many_tiles)) || (nkt <= 8 && g.M > 32) || (wide_short && g.M > 32) || many_tiles || !gemm_skinny_supports(g);
-}
-
-// The 128 x 256 tiles (eight waves, four ring slots): both operands tile-major, more 128 x 128 tiles than CUs but no more
-// 128 x 256 ones, K up to 16384.  Measured (us, the 8-wave tiled kernel's choice -> this): 640 x 8192 x 8192 42.1 -> 37.5,
-// 1024 x 8192 x 8192 48.7 -> 45.3, 2048 x 4096 x 4096 27.7 -> 26.3; with a row-major A level (1024 x 8192 x 8192 50.3 / 50.7), with
-// more tiles than CUs behind (1536 x 8192 x 8192 62.5 -> 72.6).
-bool gemm_block_wide_preferred(const GemmArgs& g) {
-  if (!gemm_block_supports(g) || g.ablation || g.clock_stamps || !g.layout_a || !g.layout_b) return false;
-  const int cus = cu_count_of_device();
-  const long rows = (g.M + kBM - 1) / kBM, tiles = rows * ((g.N + 127) / 128), wide = rows * ((g.N + 255) / 256);
-  return cus > 0 && tiles > cus && wide <= cus && g.K <= 16384;
-}
-
-// K split of this kernel's 128 x 128 tiles: shares per output tile (1 = none) and the workspace they need.
-// want: 0 = where it pays (below), 1 = never, -1 = wherever the shape allows it, n > 1 = n shares if the shape allows it.
-// Every share gets the same whole number of groups of four K-tiles, the last share what is left of K (so K need not be a
-// multiple of 512), and at least 16 K-tiles (8 where no such split exists, and for K = 8192 with few tiles); the shares of
-// all tiles together do not outnumber the CUs.  Where it pays (sweep of 48 - 512 rows x nine (N, K) pairs x three layout pairs on MI355X, us, the
-// choice before -> this, each timed twice in alternation): K from 8192 on (5120 with both operands tile-major; shorter,
-// two launches lose), at most half as many tiles as CUs, more than three eighths of them only for K = 14336 .. 16384
-// (with K = 8192 an unsplit launch of that many tiles is as fast, with K = 28672 the tiled kernel's split is:
-// 256 x 8192 x 28672 63.7 against 69.1), e.g. both operands tile-major 64 x 8192 x 28672 50 -> 40,
-// 128 x 8192 x 28672 62 -> 48 (the tiled kernel's split before), 128 x 4096 x 14336 23.8 -> 17.9, 256 x 8192 x 16384 50 -> 44.5,
-// 64 x 8192 x 8192 20.9 -> 16.1, 384 x 2048 x 8192 26.3 -> 17.5; A row-major (more than 32 rows of it: fewer are the skinny
-// kernel's), B tile-major: 64 x 8192 x 28672 46.8 -> 42.4, 96 x 8192 x 16384 40.7 -> 30.9, 192 x 4096 x 14336 33.1 -> 24.9; a
-// row-major operand: only up to a quarter as many tiles as CUs (256 x 2048 x 8192 23.3 -> 18.7, 128 x 4096 x 14336 27.9 -> 23.7;
-// beyond, level with or behind the tiled kernel's split: 128 x 12288 x 14336 47.5 against 50.8).
-int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes) {
-  if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps) return 1;
-  if (!gemm_block_supports(g)) return 1;
-  const int cus = cu_count_of_device();
-  const long tiles = (long)((g.M + kBM - 1) / kBM) * ((g.N + 127) / 128);
-  const int nkt = g.K / kBK, groups = (nkt + 3) / 4;  // groups of four K-tiles, the last one short if K % 512 != 0
-  if (cus < 8 || tiles * 2 > cus) return 1;
-  // whether the tiled kernel has a split for this K (a multiple of 512 whose groups of four K-tiles divide among shares:
-  // 18944 = 37 groups and 22016 = 43 do not)
-  int tiled_rows = 0;
-  size_t tiled_part = 0;
-  // ... and its workgroups fill half the CUs at least: K = 31744 = 62 groups gives it two shares a tile only
-  // (320 x 4224 x 31744: 68 workgroups, 94.6 us, against 72.4 with two shares of this kernel's 99 tiles;
-  // 256 x 5888 x 29696, both tile-major: 86.2 against 59.5)
-  const int tiled_shares = want == 0 && gemm_tiled_supports(g) ? tiled_ksplit_plan(g, 0, &tiled_rows, &tiled_part) : 1;
-  const bool tiled_splits = tiled_shares > 1 && (long)((g.M + tiled_rows - 1) / tiled_rows) * ((g.N + 255) / 256) * tiled_shares * 2 >= cus;
-  if (want == 0) {
-    // two launches for a K below 5120 lose (96 x 8192 x 2048: 11 -> 14 us; 256 x 2048 x 4096 13.3 -> 13.9); from there on
-    // they pay (us, unsplit -> split: 256 x 2048 x 5120, A row-major 19.8 -> 16.9, both row-major 24.1 -> 18.2;
-    // 512 x 1024 x 7168 25.2 -> 17.1; 128 x 2048 x 5504, which the skinny kernel cannot take, 20.8 -> 14.9)
-    if (nkt < 40) return 1;
-    const bool both = g.layout_a && g.layout_b;
-    if (tiles * 8 > (long)cus * 3) {  // more than three eighths as many tiles as CUs
-      // both tile-major: only K = 12288 .. 16384 (at 8192 the unsplit launch is as fast: 256 x 8192 x 8192 22.9 us against
-      // 26.5; at 28672 the tiled kernel's split is as fast or faster); a row-major operand: only K = 8192 (192 x 8192 x 8192,
-      // A row-major: 26.9 -> 22.8, both row-major 29.9 -> 25.3; 256 x 8192 x 16384 49.3 -> 51.6: beyond, the tiled kernel's
-      // split).  Where the tiled kernel has no split for K, a long K is split here (two shares on 96 - 128
-      // tiles against the unsplit launch, 13 shapes of 256 - 1024 rows: K = 11008 with a row-major operand 0.73 - 0.89 of
-      // its time, K = 18944 and 22016 0.62 - 0.76, both tile-major 0.67 - 0.93; K = 11008 both tile-major 0.86 - 1.08: not split)
-      // (a row-major operand, 96 - 128 tiles, two shares against the tiled kernel's split: K = 12288 0.73 - 0.81 of the unsplit
-      // time against 0.76 - 0.96, K = 14336 0.70 - 0.78 against 0.72 - 0.89, K = 16384 level, K = 28672 behind)
-      // (K = 19456, both tile-major, 121 tiles: two shares here 49.6 us, the tiled kernel's split 67.4: it takes over from K = 24576)
-      if (both ? (nkt < 96 || (nkt >= 192 && tiled_splits)) : (nkt >= 192 && tiled_splits)) return 1;
-    } else if (!both && tiles * 3 > cus && nkt >= 192 && tiled_splits) {
-      // a row-major operand and more than a third as many tiles as CUs (two shares at most): likewise only K = 8192.  Up
-      // to a third, three shares beat the tiled kernel's split (us, 52 shapes of 128 - 768 rows, 65 - 85 tiles, K = 12288 ..
-      // 28672: 192 x 5120 x 16384 33.0 -> 27.6, both row-major 39.7 -> 31.3; 512 x 2560 x 28672 47.8 -> 43.1 / 67.4 -> 51.6;
-      // 128 x 10240 x 14336 43.0 -> 38.7; all between 0.77 and 0.95 of its time)
-      return 1;
-    }
-    // the skinny kernel's (level at 33 - 64 rows and K = 8192 while N is one of its whole rounds: 64 x 8192 x 8192 16.1 us
-    // both ways, 64 x 10240 x 8192 21.0 -> 18.2)
-    // (the skinny kernel needs K % 512 == 0: other K, e.g. 11008 or 18944, stay here for any number of rows --
-    // 16 x 4096 x 11008 on 32 tiles unsplit: 26 us, the tiled kernel 35)
-    if (!g.layout_a && gemm_skinny_supports(g)) {
-      // up to 32 rows: the skinny kernel's, unless K is long and its last round of workgroups (32 rows of B each, 256 a
-      // round) is at most five eighths full -- 16 x 8800 x 14848 (275 workgroups) 26.8 us -> 21.9, 32 x 9088 x 28672 61.6 -> 41.2,
-      // 8 x 10240 x 28672 49.6 -> 42.4, 16 x 8800 x 13824 24.7 -> 20.2; at K = 8192 it stays ahead (16 x 9088 x 8192 14.1
-      // against 15.1), with the last round three quarters full as well (16 x 14336 x 28672 59.0 against 57.0), and against
-      // row-major weights (1 x 11264 x 32256 58 against 76)
-      const long wgs = (g.N + 31) / 32;
-      const bool last_round_thin = wgs > 256 && wgs % 256 >= 1 && wgs % 256 <= 160;
-      // (17 - 32 rows with K from 24576 on and more than one round of workgroups there: 32 x 14080 x 26112, last round
-      // seven tenths full, 64.4 us -> 55.5)
-      const bool long_k_32 = g.M > 16 && wgs > 256 && nkt >= 192;
-      if (g.M <= 32 && !(((last_round_thin && nkt >= 96) || long_k_32) && g.layout_b)) return 1;
-      if (g.M <= 64 && nkt <= 64 && (g.N < 8192 || g.N % 8192 == 0)) return 1;
-      // K below 8192: the skinny kernel's up to 96 rows (64 x 4096 x 6144 10.9 us against 12.9 split), up to 128 below 7168
-      // (128 x 2048 x 7680 18.4 -> 15.7, 128 x 2048 x 6144 level)
-      if (nkt < 64 && gemm_skinny_preferred(g) && (g.M <= 96 || (g.M <= 128 && nkt < 56))) return 1;  // (where it would be chosen: 96 x 9344 x 7680 goes to the tiled kernel otherwise, 32.5 us against 21.1 split)
-    }
-  }
-  // The most shares that leave each at least 16 K-tiles, however few workgroups that makes: with up to 32 tiles such a
-  // split beats shorter shares and every other kernel (us, 64 - 256 rows, what was chosen before -> this; each side
-  // timed twice in alternation): 128 x 512 x 16384 19.7 -> 15.7 (8 shares on 4 tiles = 32 workgroups), 64 x 512 x 28672
-  // 20.9 -> 15.3 (14 shares), 64 x 1024 x 28672 both row-major 30.0 -> 17.0, 128 x 1024 x 16384 18.1 -> 17.1 (8 shares
-  // instead of 16), 128 x 1024 x 14336 17.3 -> 16.4 (7 instead of 14), 128 x 128 x 16384 (one tile, 8 workgroups)
-  // 16.7 -> 13.3, 64 x 256 x 28672 both row-major 30.5 -> 16.7.  K = 8192 with up to 12 tiles: shares of 8 K-tiles
-  // (128 x 512 x 8192: 8 shares 12.3, 4 shares 12.9, tiled kernel's split 16.8, skinny kernel 19.3; with 16 tiles and
-  // more 4 shares are level or ahead: 256 x 2048 x 8192 16.7 against 18.2).  K beyond 16384 with 12 tiles or more and a
-  // tile-major B: shares of at least 28 K-tiles (512 x 512 x 28672, 16 tiles: 8 shares 19.6, 14 shares 21.9;
-  // 128 x 2048 x 28672 22.0 / 23.2; with 8 tiles 14 shares are ahead: 128 x 1024 x 28672 19.0 against 21.0; with a
-  // row-major B as well: 128 x 2048 x 28672 24.5 against 25.6, 512 x 384 x 28672 21.9 against 25.4).
-  int best = 1;
-  // (up to 64 rows the partial sums are small and shorter shares win: 48 x 2304 x 18304, 18 tiles, 5 shares 17.2 us, 9 shares 14.4)
-  const int first = want != 0 ? 16 : nkt == 64 && tiles <= 12 ? 8 : nkt > 128 && tiles >= 12 && g.layout_b && g.M > 64 ? 28 : 16;
-  for (int min_tiles = first; min_tiles >= 8 && best <= 1; min_tiles = min_tiles > 16 ? 16 : min_tiles - 8) {
-    for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
-      // every share the same number of whole groups, the last share what is left (at least one group)
-      const int per = (groups + sh - 1) / sh;
-      if ((sh - 1) * per < groups && per * 4 >= min_tiles && tiles * sh <= cus) {
-        best = sh;
-        break;
-      }
-      if (want > 1) break;
-    }
-  }
-  if (best <= 1) return 1;
-  // K from 24576 on, more than 32 tiles and shares on fewer than three quarters of the CUs: the tiled kernel's split
-  // streams B faster (128 x 5120 x 28672, A row-major: 44.3 us against 49.0; 256 x 5120 x 28672: 55.4 against 59.7; up
-  // to 32 tiles this kernel's: 128 x 2048 x 28672 22.0 against 26.0, 128 x 4096 x 28672 30.4 against 34.1)
-  // (from K = 20480 on: 128 x 11008 x 23040, 86 tiles, two shares here 71.5 us, five shares of the tiled kernel's 43 tiles 56.9)
-  if (want == 0 && nkt >= 160 && tiles > 32 && tiles * best * 4 < (long)cus * 3 && tiled_splits) return 1;
-  *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
-  return best;
-}
-
 // g.ksplit > 1 (with g.ks_part): the K range of every output tile split between that many workgroups, then
 // ksplit_reduce_kernel (gemm_tiled.hip), which also applies a fused epilogue.  The caller has checked that the last share
 // is not empty (block_ksplit_plan).

@@ -276,36 +276,6 @@ static bool mid_wide(const GemmArgs& g) {
   return narrow > 256 && (!g.layout_b || g.N % 64 == 0) && (long)64 * (g.K / 4 * 3) < (1L << 31);
 }
 
-// Estimated time of this kernel in microseconds: rounds of workgroups x K-tiles x time per K-tile and round.
-// Constants measured on MI355X.  One block of rows of A (M <= 128; N = 8192 and 28672, K = 8192): 0.33 / 0.48 us for 64
-// rows of A with 32 / 64 rows of B per workgroup, 0.45 / 0.55 us for 128 rows of A, 5 us fixed.  Several blocks (they
-// share B through one XCD's L2; N = 2048 .. 28672, K = 4096 .. 14336): 0.32 / 0.37 us in one round (12 % less when half
-// the CUs have a workgroup), 0.47 us per round in several, 7 / 9.5 us fixed.  Row-major B costs about 6 % more.
-double mid_estimate_us(const GemmArgs& g) {
-  const bool wide = mid_wide(g);
-  const int bn = wide ? 64 : 32;
-  const double wgs = (double)((g.N + bn - 1) / bn) * (g.M <= 64 ? 1 : (g.M + 127) / 128);
-  // (a last round of few workgroups still walks the whole of K: counted as six tenths of a round at least;
-  // 256 x 8576 x 10240, 268 workgroups: 74.5 us measured, 51 estimated with the fraction alone)
-  const double whole = (double)(long)(wgs / 256), part = wgs / 256 - whole;
-  const double rounds = wgs > 256 ? whole + (part > 0 && part < 0.6 ? 0.6 : part) : 1;
-  const double layout = g.layout_b ? 1.0 : 1.06;
-  if (g.M > 128) {
-    const double c = rounds > 1 ? 0.47 : (wide ? 0.37 : 0.32) * (0.76 + 0.24 * wgs / 256);
-    return (wide ? 9.5 : 7.0) + rounds * (g.K / 128) * c * layout;
-  }
-  const double c = g.M <= 64 ? (wide ? 0.48 : 0.33) : (wide ? 0.55 : 0.45);
-  return 5.0 + rounds * (g.K / 128) * c * layout;
-}
-
-// Automatic choice against the LDS-tiled kernel with either tile height.
-bool gemm_mid_preferred(const GemmArgs& g) {
-  if (!gemm_mid_supports(g)) return false;
-  if (!gemm_tiled_supports(g)) return true;
-  const double t = mid_estimate_us(g);
-  return t < tiled_estimate_us(g, 128) && t < tiled_estimate_us(g, 256) && t < tiled_estimate_us(g, 128, 128);
-}
-
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   typedef typename Out::type T;

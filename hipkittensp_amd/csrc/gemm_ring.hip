@@ -19,8 +19,10 @@
 // There is no workgroup-wide barrier after the first one (which publishes the zeroed flags).  Every wait is on waves of
 // the same workgroup, which are all resident, and every spin is bounded.
 //
-// Shares of a K split leave fp32 partial matrices in a workspace, summed in share order by ksplit_reduce_kernel
-// (gemm_tiled.hip), which also applies the epilogue: bit-reproducible, no atomics.  Unsplit, the epilogue is applied here.
+// Shares of a K split leave fp32 partial tiles in a workspace and count themselves in at the tile's arrival counter; the
+// workgroup that arrives last sums all shares' tiles in share order (whoever it is: the order of the sum is fixed, so the
+// result is bit-reproducible), applies the epilogue, writes C and puts the counter back to zero.  Unsplit, the epilogue is
+// applied straight from the accumulators.
 // LDS images: B and a row-major A sub-chunk as in the skinny kernel (rows of 96 * KT bytes, 16-byte pieces permuted inside
 // groups so that a ds_read_b128 phase is conflict-free), tile-major operands as they are stored.
 // The reference has no kernel for these shapes (its GEMMs need M, N multiples of the 256 tile,
@@ -349,22 +351,6 @@ RingPlan ring_plan(const GemmArgs& g, int want) {
 bool gemm_ring_supports(const GemmArgs& g) {
   return g.M >= 1 && g.N >= 4 && g.N % 4 == 0 && g.K >= 512 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) && !g.fmt_c &&
          ((uintptr_t)g.C % 16) == 0 && operands_aligned16(g) && (long)g.M * g.N < (1L << 40);
-}
-
-// Where the automatic path takes this kernel: measured against what it replaces (the skinny kernel, the block and the tiled
-// kernel with and without their K splits) over 17 (N, K) pairs x 10 row counts x both layouts of B, A row-major.  It wins
-// where the weights are what the call moves -- from about 75 MB of them (N * K >= 1e8; below, the tail of the K split, three
-// round trips to memory, outweighs the faster stream) and K >= 8192 (at K = 4096 the block kernel's tiles win by 10 - 30 %:
-// 96 x 28672 x 4096 27.5 us here, 21.6 there) -- for 17 - 64 rows of A (0.75 - 0.99 of the time before against a
-// row-major B, 0.87 - 0.99 against a tile-major one), and for 65 - 128 rows against a row-major B (0.92 - 0.98); with more
-// column tiles than compute units only against a row-major B and up to 64 rows (a tile-major B then streams as fast
-// through the tiled kernel's walk).
-bool gemm_ring_preferred(const GemmArgs& g) {
-  if (!gemm_ring_supports(g) || g.no_alloc || g.layout_a || g.M < 17 || g.M > 128 || g.K < 8192 || (double)g.N * g.K < 1e8) return false;
-  int cus = cu_count_ring();
-  if (cus <= 0) cus = 256;
-  const bool one_round = (g.N + kRingBN - 1) / kRingBN <= cus;
-  return g.M <= 64 ? (!g.layout_b || one_round) : (!g.layout_b && one_round);
 }
 
 // K split of this kernel for a call: shares (1 = none), and the bytes of partial tiles and the arrival counters it needs

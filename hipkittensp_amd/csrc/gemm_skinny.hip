@@ -279,36 +279,6 @@ bool gemm_skinny_supports(const GemmArgs& g) {
   return g.layout_a == 0 && g.M >= 1 && g.M <= 128 && g.N >= 1 && g.K >= 512 && g.K % 512 == 0 && (long)128 * (g.K / 4 * 3) < (1L << 31) && operands_aligned16(g);
 }
 
-// Automatic choice.  Up to 64 rows of A this kernel is the fastest everywhere (measured against the mid-M kernel: 18 us
-// against 22 at 64 x 8192 x 8192, 48 against 66 at K = 28672, level at N = 28672).  With 65 - 128 rows a wave's chunk is
-// mostly A (24 KB of 30), so few bytes of B are in flight per CU: it wins by 10 - 15 % while one round of workgroups covers
-// N and loses by 25 % beyond, where the mid-M kernel's 64 rows of B per workgroup halve the traffic of A.
-// Wide N (a vocabulary projection, fused gate / up matrices) with 17 - 128 rows of A: the tiled kernel's tiles hold all
-// of A and walk through hundreds of output tiles, while here every 32 or 64 rows of B pull A through L2 again.  Measured
-// (us, this kernel -> tiled kernel; tile-major B): 32 x 40960 x 8192 62 -> 55, 64 x 57344 x 8192 102 -> 73,
-// 64 x 128256 x 4096 128 -> 82, 24 x 128256 x 8192 164 -> 141, and with its 128 x 128 tiles (two workgroups per CU) already
-// at N = 28672: 32 x 28672 x 8192 41 -> 38, 64 x 28672 x 8192 50 -> 42; row-major B from 33 rows on and N >= 57344:
-// 64 x 57344 x 8192 105 -> 95, 64 x 128256 x 8192 212 -> 188 (24 - 32 rows level), and from 65 rows on from N = 24576:
-// 128 x 28672 x 8192 72 (mid-M kernel) -> 60; with K <= 4096 already from 33 rows and N = 24576 (a workgroup's K range is
-// then eight chunks or fewer, mostly load latency): 64 x 28672 x 4096 29 -> 23.  At N = 14336 and below this kernel wins.
-// Up to 16 rows only with tile-major B, K <= 4096 and N >= 65536: 16 x 128256 x 4096 82 -> 73, 16 x 65536 x 4096 45 -> 39
-// (level at K = 8192).
-bool gemm_wide_n_prefers_tiled(const GemmArgs& g) {
-  if (g.M > 128 || !gemm_tiled_supports(g)) return false;
-  const long tiles = (g.N + 255) / 256;
-  if (g.M <= 16) return g.layout_b && tiles >= 256 && g.K <= 4096;
-  if (g.layout_b) return tiles >= 160 || (tiles >= 96 && g.M >= 24);
-  // (24 - 32 rows with K <= 4096 from N = 98304 on: 32 x 128256 x 4096 105 -> 94, 24 x 128256 x 4096 99 -> 91)
-  if (g.M <= 32) return g.M >= 24 && tiles >= 384 && g.K <= 4096;
-  return g.M > 64 ? tiles >= 96 : tiles >= 224 || (tiles >= 96 && g.K <= 4096);
-}
-
-bool gemm_skinny_preferred(const GemmArgs& g) {
-  if (!gemm_skinny_supports(g) || gemm_wide_n_prefers_tiled(g)) return false;
-  // (where the mid-M kernel cannot take the shape -- K % 1024 != 0 -- the tiled kernel does: 96 x 23344 x 8704 92 us here, 56 there)
-  return g.M <= 64 || (g.N + 31) / 32 <= 256 || (!gemm_mid_supports(g) && !gemm_tiled_supports(g));
-}
-
 // Workspace of the K split: 4 KB of partial tile per (tile, split) and a counter per tile that is zero between
 // launches.  One per (device, stream), taken from the stream-ordered allocator on the caller's stream at the first split
 // launch there (no device-wide synchronisation) and kept until release_split_workspaces(): launches on one stream are

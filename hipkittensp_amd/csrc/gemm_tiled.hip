@@ -60,9 +60,8 @@ namespace mxfp6 {
 
 // defined in the host-side object, used by the launchers of the per-format objects
 int tiled_grid_size(const GemmArgs& g, int tiles, int per_cu);
-int tiled_tile_shape(const GemmArgs& g);
 hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s);
-constexpr int kMinShareTiles = 8;  // K-tiles a share of a K split has at least
+constexpr int kMinShareTiles = 8;  // K-tiles a share of a K split has at least (dispatch.hip plans with the same figure)
 // defined in the per-format objects
 hipError_t launch_gemm_tiled_fmt22(const GemmArgs& g, hipStream_t s);
 hipError_t launch_gemm_tiled_fmt23(const GemmArgs& g, hipStream_t s);
@@ -764,45 +763,6 @@ int tiled_grid_size(const GemmArgs& g, int tiles, int per_cu) {
   return tiles < cus ? tiles : cus;
 }
 
-// Estimated time of this kernel with tiles of `rows` (128 or 256) rows of A, in microseconds: the tiles are
-// dealt to the CUs in rounds, and a K-tile of a round takes longer the fuller the round is (fewer active CUs run
-// at a higher clock and meet less L2 contention).  Constants measured on MI355X with tile-major B: 8192-wide
-// problems of 64 K-tiles took 57.7 / 62.7 / 70.1 / 86.9 us with 64 / 128 / 192 / 256 tiles of 256 rows and
-// 43.5 / 46.5 / 53.9 us with 128 / 192 / 256 tiles of 128 rows, 34.1 / 38.9 / 73.8 us with 128 / 256 / 512 tiles of
-// 128 x 128; row-major B costs about 28 % more, and no shape runs faster than its bytes stream.  Rounds after the first
-// are cheaper for 256-row tiles (the walk overlaps tile changes, and the launch's slow start is paid once): 8192^3 is
-// four rounds in 290 - 300 us, not 4 x 87.  The streaming floor grows with the workgroups that stream side by side:
-// measured on problems whose B comes from HBM (N = 28672 and 57344, K = 8192, 8 - 128 rows of A), tile-major B: 4.5 TB/s
-// with 112 workgroups, 5.2 - 5.6 with 224 and more (128 x 128 tiles, two per CU, reach that at N = 28672 where 128 x 256
-// tiles have 112: 37 us against 42 - 45); row-major B: 2.7 - 2.9 TB/s with 112, 4.2 - 4.5 with 224.
-double tiled_estimate_us(const GemmArgs& g, int rows, int cols) {
-  int cus = cu_count();
-  if (cus <= 0) cus = 256;
-  const long tiles = (long)((g.M + rows - 1) / rows) * ((g.N + cols - 1) / cols);
-  const long full = tiles / cus;
-  const double f = (double)(tiles % cus) / cus;
-  const double c0 = cols == 128 ? 0.45 : rows == 128 ? 0.62 : 0.85, c1 = cols == 128 ? 0.10 : rows == 128 ? 0.22 : 0.50;
-  const double later = rows == 256 && full >= 1 ? 0.82 : 1.0;  // what a round after the first costs against the first
-  const double per_ktile = (full >= 1 ? (c0 + c1) * (1.0 + (full - 1) * later) : 0.0) + (f > 0 ? (c0 + c1 * f * f) * later : 0.0);
-  const double layout = 1.0 + (g.layout_b ? 0.0 : 0.28) - (g.layout_a ? 0.05 : 0.0);
-  const double bytes = (0.75 + 1.0 / 32) * g.K * ((double)g.M + g.N) + 2.0 * g.M * g.N;
-  const double side_by_side = (double)(tiles < (long)cus * (cols == 128 ? 2 : 1) ? tiles : (long)cus * (cols == 128 ? 2 : 1)) / 224.0;
-  const double conc = g.layout_b ? 0.6 + 0.4 * side_by_side : 0.3 + 0.7 * side_by_side;
-  const double stream = bytes / ((g.layout_b ? 5.4e6 : 4.5e6) * (conc < 1.0 ? conc : 1.0));
-  const double compute = 3.0 + (g.K / kBK) * per_ktile * layout;
-  return compute > stream ? compute : stream;
-}
-
-// Tile shape: 256 x 256 unless tiles of 128 rows of A, or of 128 x 128, fill the machine better (the fp6 output needs
-// 256 columns).  Returns rows | cols << 16.
-int tiled_tile_shape(const GemmArgs& g) {
-  if (g.tile_rows == 128 || g.tile_rows == 256) return g.tile_rows | (g.tile_cols == 128 && g.tile_rows == 128 && !g.fmt_c ? 128 : 256) << 16;
-  const double t256 = tiled_estimate_us(g, 256, 256), t128 = tiled_estimate_us(g, 128, 256);
-  const double t128n = g.fmt_c ? 1e30 : tiled_estimate_us(g, 128, 128);
-  if (t128n < t128 && t128n < t256) return 128 | 128 << 16;
-  return (t128 < t256 ? 128 : 256) | 256 << 16;
-}
-
 // Sum of the K split's partial matrices, in share order, with the epilogue: 4 consecutive outputs per thread.
 template <typename T>
 __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restrict__ part, int nsplit, T* __restrict__ C, int M, int N, const Epilogue ep) {
@@ -823,82 +783,6 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(const float* __restr
   } else {
     *reinterpret_cast<v4f*>(C + i4) = acc;
   }
-}
-
-// K split (KSPLIT instantiations): for problems of few output tiles and long K, typically 100 - 1000 rows of A against a
-// wide weight matrix, where one workgroup per output tile would leave most CUs idle and the kernel would stream B at a
-// fraction of HBM speed.  Shares per tile = CUs / tiles, rounded down to a divisor of the groups of four K-tiles that
-// leaves every share at least kMinShareTiles K-tiles; the tile height is the one whose shares finish first.
-// want: 0 = where it pays (below), -1 = wherever the shape allows it, 1 = never, n > 1 = n shares if the shape allows it
-// (the last three for measurement).  Returns the shares per tile (1: no split) and the tile height and workspace size
-// that go with them.
-// Where it pays (measured on MI355X against the best unsplit kernel over 360 shapes, M = 8 .. 2048, N = 1024 .. 57344,
-// tile-major and row-major B), in output tiles of 256 x 256: with K >= 12288 up to 64 tiles (128 from K = 20480 on
-// -- 768 x 6912 x 20480 131 -> 118, 1536 x 4096 x 21504 127 -> 121 -- and
-// for up to 256 rows of A: 256 x 17920 x 23040 159 -> 114 us, 160 x 16768 x 17408 138 -> 110, 160 x 18304 x 13824 81 -> 60;
-// up to 1024 rows against a row-major B: 384 x 12928 x 19456 160 -> 121, 768 x 9216 x 17408 142 -> 127;
-// with 2048 rows it loses: 2048 x 5120 x 16384 122 -> 134, and so it does with both operands tile-major beyond 104
-// tiles: 192 x 28672 x 12288 76.4 on the block kernel's 128 x 256 tiles -> 88.5; with a row-major A, which those tiles
-// do not take, it wins there as well, 160 x 28672 x 16384 116 -> 104, 160 x 27904 x 18432 130 -> 113):
-// 0.45 - 0.9 of the unsplit time, e.g. 256 x 8192 x 28672 108 -> 63 us, 128 x 4096 x 14336 46 -> 24 us, 1024 x 1024 x 16384
-// 60 -> 34 us; with 8192 <= K < 14336 up to 32 tiles where the skinny kernel is not an option (more than 128 rows of A, or
-// a tile-major A): 256 x 2048 x 8192 28.5 -> 21 us, 768 x 2048 x 8192 33 -> 27 us; and up to 64 tiles for 65 - 128 rows of A
-// against more than 8192 rows of B, where the skinny kernel needs more than one round of workgroups:
-// 96 x 10240 x 8192 35 -> 27 us, 96 x 10240 x 12288 66 -> 37 us.  More tiles or a shorter K lose (the
-// partial sums cost 12 - 25 us to write, read and add): 256 x 8192 x 4096 19 -> 24 us, 512 x 8192 x 8192 36 -> 40 us.
-int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes) {
-  if (want == 1 || g.fmt_c || g.ablation || g.no_alloc || g.clock_stamps || g.K % (4 * kBK) != 0) return 1;
-  const int cus = cu_count() & ~7, groups = g.K / (4 * kBK), nkt = g.K / kBK;
-  if (cus < 8) return 1;
-  int min_shares = 2;
-  if (want == 0) {
-    const long tiles256 = (long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    // (K = 8192 .. 12287, a row-major B, more than 128 rows, 65 - 85 tiles -- more 128 x 128 tiles than CUs, so the block
-    // kernel is out -- and three shares a tile: 640 x 6800 x 10752 66.4 us -> 57.6, 768 x 6760 x 9216 60.3 -> 56.2; two
-    // shares lose, 768 x 6144 x 8192 51.6 -> 54.1, and so do three against a tile-major B, 512 x 10496 x 9216 49.3 -> 60.5)
-    const bool three_shares_mid_k = nkt >= 64 && nkt < 96 && !g.layout_b && g.M > 128 && tiles256 > 64 && tiles256 * 3 <= cus;
-    if (three_shares_mid_k || (nkt < 96 && tiles256 > 64 && g.M > 64 && g.M <= 128)) min_shares = 3;
-    const bool pays = nkt >= 96 ? (tiles256 <= 64 || (tiles256 <= 128 && (nkt >= 160 || (g.layout_b ? g.M <= 256 && (tiles256 <= 104 || !g.layout_a) : g.M <= 1024))))
-                                 : nkt >= 64 && ((tiles256 <= 32 && (g.M > 128 || g.layout_a)) ||
-                                                 // 65 - 128 rows and more than 256 x 32 rows of B: the skinny kernel is past its one round of workgroups
-                                                 // (up to 85 tiles with three shares a tile: 96 x 19584 x 10752 55.3 us on the block kernel -> 44.8)
-                                                 (tiles256 * 3 <= cus && g.M > 64 && g.M <= 128 && g.N > 8192) ||
-                                                 // 33 - 64 rows against a wide row-major B, three shares a tile (below)
-                                                 (g.M > 32 && g.M <= 64 && !g.layout_a && !g.layout_b && g.N > 16384 && tiles256 * 3 <= cus) ||
-                                                 three_shares_mid_k);
-    if (!pays) return 1;
-    if (g.M <= 64 && !g.layout_a) {
-      // up to 64 rows of a row-major A are the skinny kernel's, except more than 32 against tile-major weights with a
-      // very long K, or a long K and a width that leaves the skinny kernel's last round of workgroups part empty
-      // (with K < 24576 up to 104 tiles: beyond, two shares a tile lose to the block kernel's unsplit tiles,
-      // 48 x 28672 x 12288 59.9 us -> 53.8; and against a row-major B of more than 16384 rows with three shares a tile or more:
-      // 64 x 16640 x 12288 64.9 us on the skinny kernel -> 53.3, 48 x 16640 x 9216 49.7 -> 39.4, 64 x 17024 x 21504 103 -> 84.5, two shares level)
-      const bool ragged = g.N > 8192 && g.N % 8192 != 0 && tiles256 <= 104;
-      if (g.M > 32 && !g.layout_b && nkt >= 64 && g.N > 16384 && tiles256 * 3 <= cus) min_shares = 3;
-      else if (!(g.M > 32 && g.layout_b && tiles256 <= 128 && (nkt >= 192 || ragged))) return 1;
-    }
-  }
-  int best = 1, best_rows = 0;
-  double best_us = 0;
-  for (int bm = 256; bm >= 128; bm -= 128) {
-    if ((g.tile_rows && g.tile_rows != bm) || g.tile_cols == 128) continue;
-    const long tiles = (long)((g.M + bm - 1) / bm) * ((g.N + 255) / 256);
-    if (tiles * 2 > cus) continue;
-    for (int sh = want > 1 ? want : (int)(cus / tiles); sh > 1; sh--) {
-      if (groups % sh != 0 || nkt / sh < kMinShareTiles) {
-        if (want > 1) break;
-        continue;
-      }
-      // a share's K-tiles at this tile height's pace with every CU busy, plus writing and reading the partial matrices
-      const double us = (double)nkt / sh * (bm == 256 ? 1.35 : 0.84) + 2.0 * sh * g.M * g.N * 4.0 / 4e6;
-      if (best_rows == 0 || us < best_us) best = sh, best_rows = bm, best_us = us;
-      if (want > 1) break;
-    }
-  }
-  if (best < min_shares) return 1;
-  *rows = best_rows;
-  *part_bytes = (size_t)best * g.M * g.N * sizeof(float);
-  return best;
 }
 
 hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s) {
@@ -922,7 +806,8 @@ hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s) {
 template <int FA, int FB, typename Out>
 static hipError_t launch(const GemmArgs& g, hipStream_t s) {
   const bool ksplit = g.ksplit > 1 && g.ks_part;
-  const int shape = ksplit ? g.tile_rows | 256 << 16 : tiled_tile_shape(g), bm = shape & 0xffff, bn = shape >> 16;
+  // the tile shape is the caller's (the dispatcher's choice, or a forced one); 256 x 256 unless told otherwise
+  const int bm = g.tile_rows == 128 ? 128 : 256, bn = !ksplit && g.tile_cols == 128 && bm == 128 && !g.fmt_c ? 128 : 256;
   const int tm = (g.M + bm - 1) / bm, tn = (g.N + bn - 1) / bn;
   const TiledArgs ta = {g.A, g.B, g.As, g.Bs, g.C, g.M, g.N, g.K, tm, tn, g.layout_a, g.layout_b, g.ep, g.C_scale, g.fmt_c, g.raster_group_m > 0 ? g.raster_group_m : kGroupM, g.raster_no_xcd_remap == 1 ? 0 : g.raster_no_xcd_remap == 2 ? 2 : 1, ksplit ? g.ksplit : 1
 #ifdef MXFP6_PROBES

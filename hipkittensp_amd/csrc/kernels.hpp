@@ -34,32 +34,34 @@ inline bool operands_aligned16(const GemmArgs& g) {
   return (((uintptr_t)g.A | (uintptr_t)g.B | (uintptr_t)g.As | (uintptr_t)g.Bs) & 15) == 0;
 }
 
+// ---- kernel choice (dispatch.hip): candidates of the automatic path, a time model per candidate, a calibration table
+enum Candidate : int { kCandTiled256 = 0, kCandTiled128x256, kCandTiled128x128, kCandBlock, kCandBlockWide, kCandSkinny, kCandTiledSplit256, kCandTiledSplit128, kCandBlockSplit, kCandRing, kNumCandidates };
+struct KernelChoice {
+  int cand;    // a Candidate, or -1: none of them takes the shape (the generic kernel does)
+  int shares;  // K split: workgroups per output tile (1 = none)
+  int rows;    // tiled kernel's split: rows of A per tile
+  double us;   // modelled time x calibration factor
+};
+int device_cus();
+double candidate_model_us(const GemmArgs& g, int cand, int want_split, int cus, int* shares, int* rows);  // modelled microseconds; < 0: the candidate does not take the shape
+KernelChoice choose_kernel(const GemmArgs& g, int want_split, bool allow_split, unsigned mask = ~0u);  // mask: bit per Candidate that may be chosen; want_split: 0 = by the model, 1 = never, n = n shares where a candidate splits; allow_split: a workspace is to be had
+int tiled_split_shares(const GemmArgs& g, int want, int cus, int bm);  // the tiled kernel's K split with tiles of bm (256 or 128) rows when it is to split: shares (1 = the shape has none)
+int block_split_shares(const GemmArgs& g, int want, int cus);             // ... the block kernel's
+
 hipError_t launch_gemm_generic(const GemmArgs& g, hipStream_t s);
 bool gemm_tiled_supports(const GemmArgs& g);
 hipError_t launch_gemm_tiled(const GemmArgs& g, hipStream_t s);
-// K split of the tiled kernel for this problem (want: 0 = by shape, 1 = never, n = n shares if possible): shares per output tile
-// (1 = none), rows of A per tile and workspace bytes for the partial sums
-int tiled_ksplit_plan(const GemmArgs& g, int want, int* rows, size_t* part_bytes);
 bool gemm_tiled4_supports(const GemmArgs& g);  // the 4-wave variant of the tiled kernel (selectable, never chosen automatically)
 hipError_t launch_gemm_tiled4(const GemmArgs& g, hipStream_t s);
 bool gemm_block_supports(const GemmArgs& g);  // 128 x 128 tiles, four waves in step (a few hundred to a few thousand rows of A)
-bool gemm_block_preferred(const GemmArgs& g, bool first);  // by shape; first: even before the tiled kernel's K split is considered
-bool gemm_block_wide_preferred(const GemmArgs& g);  // its 128 x 256 tiles (eight waves) beat the 8-wave tiled kernel's
-int block_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes);  // K split of the block kernel for this problem: shares per tile (1 = none)
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s);
 hipError_t launch_ksplit_reduce(const GemmArgs& g, hipStream_t s);  // sums g.ksplit partial matrices at g.ks_part into g.C, with the epilogue
 bool gemm_ring_supports(const GemmArgs& g);  // batched decode: private streams of B per wave, A through a flag-guarded ring (no barrier per K-tile)
 int ring_ksplit_plan(const GemmArgs& g, int want, size_t* part_bytes, size_t* counters);  // its K split for this problem (want: 0 = by shape, 1 = none, n = n shares): shares (1 = none), bytes of partial tiles, arrival counters
-bool gemm_ring_preferred(const GemmArgs& g);  // by shape: weights streamed from HBM against 17 - 128 rows of a row-major A
 hipError_t launch_gemm_ring(const GemmArgs& g, hipStream_t s);
 bool gemm_mid_supports(const GemmArgs& g);
-bool gemm_mid_preferred(const GemmArgs& g);  // supported and expected to beat the LDS-tiled kernel
-double tiled_estimate_us(const GemmArgs& g, int rows, int cols = 256);  // estimated time of the tiled kernel with tiles of rows x cols
-double mid_estimate_us(const GemmArgs& g);
 hipError_t launch_gemm_mid(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_supports(const GemmArgs& g);
-bool gemm_skinny_preferred(const GemmArgs& g);  // over the mid-M kernel, by shape
-bool gemm_wide_n_prefers_tiled(const GemmArgs& g);  // 17 - 64 rows of A against a very wide B: the tiled kernel's 128-row tile beats the skinny and mid-M kernels
 hipError_t launch_gemm_skinny(const GemmArgs& g, hipStream_t s);
 bool gemm_skinny_scratch_fits(const GemmArgs& g);  // no_alloc: the K split this call would use fits the static scratch array
 hipError_t release_split_workspaces();             // returns every K-split workspace to the stream-ordered allocator

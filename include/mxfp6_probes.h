@@ -63,6 +63,16 @@ int mxfp6_probe_raster(int group_m, int xcd_remap);
  * on them). */
 int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int *tile_rows);
 
+/* The kernel choice's view of one candidate on a shape (e2m3 x e2m3, bf16 output, 16-byte aligned tensors): *model_us is the
+ * structural time model's figure in microseconds (negative: the candidate does not take the shape), *calibrated_us that figure
+ * times the calibration factor of the nearest calibrated shape (what the choice compares), *shares the K split the candidate
+ * would run with under the thread's mxfp6_set_k_split setting.  candidate: 0 - 2 the tiled kernel with tiles of 256 x 256 /
+ * 128 x 256 / 128 x 128, 3 block, 4 block with tiles of 128 x 256, 5 skinny, 6 / 7 the tiled / the block kernel with its K
+ * split, 8 ring.  cus: compute units to plan for (0 = the current device's).  Pure host code: the calibration tool
+ * (python -m hipkittensp_amd.calibrate) calls it to turn a sweep's measured times into the table's factors. */
+int mxfp6_probe_candidate(int M, int N, int K, int layouts, int candidate, int cus, double *model_us, double *calibrated_us,
+                          int *shares);
+
 /* Measurement switch, per calling thread: 0 keeps the block kernel (mxfp6_set_kernel 22 - 27) out of the automatic choice,
  * so that the same call can be timed with and without it; returns the previous setting.  Default 1. */
 int mxfp6_probe_block(int enable);

@@ -119,10 +119,17 @@ static int run_case(int M, int N, int K, int fmt_a, int fmt_b, hipStream_t strea
   size_t wrong_bf16 = 0, wrong_noalloc = 0;
   for (size_t i = 0; i < mn; i++) {
     wrong_bf16 += cb[i] != mxfp6o_f32_to_bf16(cf[i]);
-    wrong_noalloc += cn[i] != cb[i];
+    /* bit-identical where both entry points take the same kernel; where mxfp6_gemm takes one the no-allocation path has not,
+       the same products are added in another order: within one bf16 step of the fp32 result */
+    if (cn[i] != cb[i]) {
+      const uint32_t u = (uint32_t)cn[i] << 16;
+      float v;
+      memcpy(&v, &u, 4);
+      wrong_noalloc += !(fabs((double)v - (double)cf[i]) <= fabs((double)cf[i]) * 0.0078125);
+    }
   }
   if (wrong_bf16) bad++, printf("  bf16 output: %zu values are not the rounding of the accumulators\n", wrong_bf16);
-  if (wrong_noalloc) bad++, printf("  mxfp6_gemm_noalloc: %zu values differ from mxfp6_gemm\n", wrong_noalloc);
+  if (wrong_noalloc) bad++, printf("  mxfp6_gemm_noalloc: %zu values are more than one bf16 step from the fp32 result\n", wrong_noalloc);
   printf("case M=%d N=%d K=%d fmt=%d,%d: metric %.2e  %s\n", M, N, K, fmt_a, fmt_b, metric, bad ? "FAIL" : "ok");
   fflush(stdout);
 

@@ -106,7 +106,14 @@ def test_limit_and_other_kernels(hk):
     a2, asc2, b2, bsc2 = _operands(hk, 64, 64, 1024, 32)
     C2 = torch.empty(64, 64, dtype=torch.bfloat16, device="cuda")
     assert L.mxfp6_gemm_noalloc(a2.data_ptr(), b2.data_ptr(), asc2.data_ptr(), bsc2.data_ptr(), C2.data_ptr(), 64, 64, 1024, 2, 2, 2, None) == -2
-    # shapes of the other kernels run unchanged (mid-M, tiled without the pre-pass, generic), bit-identical to mxfp6_gemm's
+    # shapes of the other kernels run too.  The header promises bit-identity only where both entry points take the same
+    # kernel; here mxfp6_gemm may take one the no-allocation path has not (the block kernel, a K split), which adds the same
+    # products in another order: equal within one bf16 step of the fp32 result
     for M, N, K, seed in ((64, 64, 1024, 33), (300, 264, 640, 34), (70, 40, 96, 35)):
         ops = _operands(hk, M, N, K, seed)
-        assert np.array_equal(_bits(_noalloc(hk, *ops)), _bits(_existing(hk, *ops)))
+        got = _noalloc(hk, *ops).float()
+        a_, asc_, b_, bsc_ = ops
+        ref = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        hk.dispatch_micro(a_, b_, asc_, bsc_, ref)
+        torch.cuda.synchronize()
+        assert torch.all((got - ref).abs() <= ref.abs() * 2.0 ** -7 + 1e-30)
