@@ -427,9 +427,9 @@ def dispatch_sweep(hk, torch, grid):
     Small shapes (below about 15 us) are bound by the host side of the Python operator and only scatter."""
     tk = hk.tk_kernel
     if grid == "offgrid":  # none of these (N, K) pairs and none of these row counts is in the calibration table
-        shapes = [(6144, 6144), (12288, 6144), (3072, 12288), (20480, 5120), (18432, 9216), (7168, 20480), (49152, 4096), (2560, 10240),
-                  (13824, 5120), (5120, 13824), (100352, 2048), (1536, 32768)]
-        rows_of_a = [12, 40, 80, 112, 160, 224, 320, 448, 640, 896, 1536, 3072]
+        shapes = [(7168, 7168), (3584, 18944), (18944, 3584), (9216, 4608), (27648, 5120), (1792, 14336), (22016, 4096), (5632, 22528),
+                  (13312, 6656), (36864, 3072), (2304, 24576), (15360, 10240)]
+        rows_of_a = [20, 56, 72, 144, 208, 288, 416, 576, 832, 1152, 1792, 2560]
     elif grid == "full":
         shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096),
                   (8192, 28672), (2048, 8192), (5120, 16384), (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096)]
@@ -511,8 +511,9 @@ def calibration_sweep(hk, torch):
     shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096), (8192, 28672), (2048, 8192), (5120, 16384),
               (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096), (4096, 4096), (16384, 16384), (2048, 28672), (11008, 4096), (4096, 11008), (2048, 2048), (512, 8192), (8192, 1024),
               (1024, 32768), (2048, 16384), (4096, 8192), (4096, 24576), (8192, 4096), (8192, 14336), (16384, 4096), (16384, 8192), (65536, 2048), (3072, 3072), (6144, 4096), (1024, 4096),
-              (12288, 12288), (2048, 5120), (24576, 2048), (73728, 4096)]
-    rows_of_a = [1, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 4096, 8192]
+              (12288, 12288), (2048, 5120), (24576, 2048), (73728, 4096),
+              (6144, 6144), (12288, 6144), (3072, 12288), (20480, 5120), (18432, 9216), (7168, 20480), (49152, 4096), (2560, 10240), (13824, 5120), (5120, 13824), (100352, 2048), (1536, 32768)]
+    rows_of_a = [1, 8, 12, 16, 24, 32, 40, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1536, 2048, 3072, 4096, 8192]
 
     def time_us(ops, C, la, lb, kernel, k_split, reps=8):
         prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
