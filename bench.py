@@ -47,7 +47,10 @@ PUBLISHED_FP6_8192 = 2861.52  # reference's published FP6 GEMM at 8192^3 on MI35
 PUBLISHED_FP6_SQUARES = {1024: 74.9089, 2048: 470.161, 4096: 1865.47, 16384: 3122.13}
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
 # the sources whose text decides what the two profiled kernels move; profiles/traffic.json records their hash
-TRAFFIC_SOURCES = {"gemm_tiled_kernel": ("gemm_tiled.hip", "common.hpp", "loader.hpp"), "gemm_skinny_kernel": ("gemm_skinny.hip", "common.hpp", "loader.hpp")}
+TRAFFIC_SOURCES = {"gemm_tiled_kernel": ("gemm_tiled.hip", "common.hpp", "loader.hpp"), "gemm_skinny_kernel": ("gemm_skinny.hip", "common.hpp", "loader.hpp"),
+                   "gemm_ring_kernel_m16": ("gemm_ring.hip", "common.hpp", "loader.hpp"), "gemm_ring_kernel_m64": ("gemm_ring.hip", "common.hpp", "loader.hpp")}
+# kernel behind a code of tk_kernel.kernel_choice, for the decode shapes
+DECODE_KERNELS = {3: "gemm_skinny_kernel", 28: "gemm_ring_kernel", 22: "gemm_block_kernel", 26: "gemm_block_kernel", 27: "gemm_block_kernel", 2: "gemm_tiled_kernel", 25: "gemm_tiled_kernel", 1: "gemm_generic_kernel"}
 
 # BASELINE.json configs: shape, formats, source distributions (A, B), seed
 CONFIGS = {
@@ -608,7 +611,7 @@ def traffic_from(fetch_csv, write_csv):
     def per_kernel(path):
         agg = collections.defaultdict(list)
         for r in csv.DictReader(open(path)):
-            agg[re.sub(r"\(.*$", "", re.sub(r"^void ", "", r["Kernel_Name"]))].append(float(r["Counter_Value"]))
+            agg[re.sub(r"\(.*$", "", re.sub(r"^void ", "", r["Kernel_Name"].replace("(anonymous namespace)::", "")))].append(float(r["Counter_Value"]))
         return agg
 
     fetch, write = per_kernel(fetch_csv), per_kernel(write_csv)
@@ -623,10 +626,13 @@ def traffic_from(fetch_csv, write_csv):
     out = {"what": "FETCH_SIZE and WRITE_SIZE (KiB per dispatch) of rocprofv3 --pmc runs of `python3 bench.py --profile-kernels`, each scaled by what the same "
                    "counter reads for an elementwise in-place multiply of 8192 x 28672 fp32 (917 504 KiB each way) in the same run",
            "fetch_factor": ff, "write_factor": wf, "kernels": {}}
-    for kernel, match in (("gemm_tiled_kernel", "gemm_tiled_kernel<2, 2, mxfp6::OutBf16, 4, 2"), ("gemm_skinny_kernel", "gemm_skinny_kernel<2, 2, mxfp6::OutBf16, 16, 8, 32")):
+    for kernel, match in (("gemm_tiled_kernel", "gemm_tiled_kernel<2, 2, mxfp6::OutBf16, 4, 2"), ("gemm_skinny_kernel", "gemm_skinny_kernel<2, 2, mxfp6::OutBf16, 16, 8, 32"),
+                          ("gemm_ring_kernel_m16", "gemm_ring_kernel<2, 2, mxfp6::OutBf16, 1>"), ("gemm_ring_kernel_m64", "gemm_ring_kernel<2, 2, mxfp6::OutBf16, 2>")):
         f = [max(v) for k, v in fetch.items() if match in k]
         w = [max(v) for k, v in write.items() if match in k]
-        assert f and w, f"{kernel} not found in the traces"
+        if not (f and w):   # the decode loop ran on the other of the two kernels that are level at configs[3]
+            assert "tiled" not in kernel, f"{kernel} not found in the traces"
+            continue
         out["kernels"][kernel] = {"fetch_kib": max(f), "write_kib": max(w), "traffic_bytes": int((max(f) * ff + max(w) * wf) * 1024), "source_hash": source_hash(kernel),
                                   "what": f"FETCH_SIZE {max(f):.0f} KiB x {ff:.2f} + WRITE_SIZE {max(w):.0f} KiB x {wf:.2f}"}
     json.dump(out, open(TRAFFIC_JSON, "w"), indent=1)
@@ -691,7 +697,13 @@ def main():
         cfg3 = CONFIGS["cfg3"]
         d = make_inputs(hk, torch, cfg3, 5)
         dC = torch.empty(16, 8192, dtype=torch.bfloat16, device="cuda")
-        out["gemm_skinny_kernel_cfg3_row_major_ms"] = timed_loop(hk, torch, d, dC, args.steps, args.warmup)[1]
+        for name, code in (("gemm_skinny_kernel", tk.KERNEL_SKINNY), ("gemm_ring_kernel", tk.KERNEL_RING)):  # level with each other at configs[3]: both
+            prev = tk.set_kernel(code)
+            try:
+                out[name + "_cfg3_row_major_ms"] = timed_loop(hk, torch, d, dC, args.steps, args.warmup)[1]
+            finally:
+                tk.set_kernel(prev)
+        out["cfg3_row_major_automatic_choice"] = DECODE_KERNELS.get(tk.kernel_choice(16, 8192, cfg3["K"], 0, 0), "?")
         dt = [tiled(hk, ops, cfg3["K"], "b") for ops in d]
         del d
         ba, bas = hk.quantize(torch.from_numpy(cpu_source("normal", (64, cfg3["K"]), 3164)).cuda(), 2)
@@ -932,14 +944,15 @@ def main():
     del qx, qp, qs, q0
     torch.cuda.empty_cache()
     stream_p = stream_probe(torch, _lib.probes())
-    dtraffic, dtraffic_what = traffic_of("gemm_skinny_kernel")
+    dkernel = DECODE_KERNELS.get(tk.kernel_choice(dM, dN, dK, 0, 0), "?")  # the skinny and the ring kernel are level here
+    dtraffic, dtraffic_what = traffic_of("gemm_ring_kernel_m16" if dkernel == "gemm_ring_kernel" else dkernel)
     decode = {
         "metric": "MXFP6 decode GEMM achieved GB/s @M=16,N=8192,K=28672",
         "value": dbytes / (dwall / args.steps) / 1e9,
         "unit": "GB/s",
         "ms_per_step": dwall / args.steps * 1e3,
         "roofline": {
-            "kernel": "gemm_skinny_kernel",
+            "kernel": dkernel,
             "bound": "hbm",
             "achieved": d_achieved,
             "peak": HBM_PEAK_GBS,
