@@ -249,6 +249,7 @@ def test_block_kernel_matches_the_tiled_kernel(hk, M, N, K, la, lb):
 
 
 @pytest.mark.parametrize("M,N,K,shares", [(128, 256, 4096, 2), (128, 512, 8192, 4), (100, 264, 4096, 2), (256, 512, 8192, 8), (64, 1024, 16384, 0), (192, 2048, 8192, 0),
+                                          (128, 256, 32768, 16), (200, 136, 18432, 9),   # many shares
                                           (128, 512, 8192, 0), (96, 520, 28672, 0), (100, 128, 16384, 0), (512, 512, 28672, 0),
                                           # K % 512 != 0: the last share takes what is left of K, down to a single K-tile
                                           (128, 256, 2816, 2), (100, 264, 4480, 3), (128, 384, 4224, 4), (16, 4096, 11008, 0), (256, 512, 11008, 0), (64, 1024, 18944, 0)])
@@ -256,7 +257,7 @@ def test_block_kernel_matches_the_tiled_kernel(hk, M, N, K, la, lb):
 def test_block_kernel_k_split(hk, M, N, K, shares, fa, fb):
     """The block kernel with the K range of every output tile split between several workgroups: fp32 partial matrices in
     the stream's workspace, summed in share order by the tiled kernel's reduction.  Forced share counts on the forced
-    kernel, and shapes on which the automatic path chooses this split itself.  Against the fp64 oracle; bf16 output = RNE
+    kernel, and shapes on which the automatic path may choose this split itself.  Against the fp64 oracle; bf16 output = RNE
     of the fp32 output; a second call gives the same bits; tile-major operands give the same bits as row-major ones; a
     fused epilogue is applied by the reduction."""
     tk = hk.tk_kernel
@@ -281,13 +282,16 @@ def test_block_kernel_k_split(hk, M, N, K, shares, fa, fb):
                 assert np.array_equal(C.cpu().numpy(), got)
             else:
                 check(C.cpu().numpy(), ref, fa, fb, ap, asc, bp, bsc)  # the automatic path may take another split for another layout
-        if not shares:
-            bias = torch.linspace(-1, 1, N, device="cuda")
-            C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        bias = torch.linspace(-1, 1, N, device="cuda")
+        C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        pk = tk.set_kernel(kernel)
+        try:
             hk.dispatch_micro(dev(ap), dev(bp), dev(asc), dev(bsc), C, fa, fb, bias=bias, activation="relu")
             torch.cuda.synchronize()
-            want = np.maximum(got + bias.cpu().numpy()[None, :], 0)
-            assert np.allclose(C.cpu().numpy(), want, rtol=1e-6, atol=1e-6 * np.abs(got).max())
+        finally:
+            tk.set_kernel(pk)
+        want = np.maximum(got + bias.cpu().numpy()[None, :], 0)
+        assert np.allclose(C.cpu().numpy(), want, rtol=1e-6, atol=1e-6 * np.abs(got).max())
     finally:
         tk.set_k_split(prev)
 
