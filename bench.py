@@ -236,12 +236,20 @@ def probes(hk, torch, P, inputs, kinputs, C, M, N, K):
                                            "clocks_per_k_tile": clk / ((M // 256) * (N // 256) / 256.0 * (K // 128))}
         # what each part of the kernel costs: builds of the same kernel without its LDS reads (1), its loads (2), its MFMAs (4)
         abl = {}
-        names = {0: "full", 1: "no_lds_reads", 2: "no_loads", 3: "mfma_only", 4: "no_mfma", 6: "lds_reads_only"}
-        for mask in (0, 1, 2, 3, 4, 6, 0):
+        names = {0: "full", 1: "no_lds_reads", 2: "no_loads", 3: "mfma_only", 4: "no_mfma", 6: "lds_reads_only", 8: "full_plus_idle_clocks"}
+        for mask in (0, 1, 2, 3, 4, 6, 8, 0):
             assert P.mxfp6_probe_tiled_ablation(mask) == 0
-            _, ms = timed_loop(hk, torch, [kinputs[0]], C, 20, 10, prewarm_ms=PREWARM_MS if mask in (0, 3) else 0.0, call=call)
+            _, ms = timed_loop(hk, torch, [kinputs[0]], C, 20, 10, prewarm_ms=PREWARM_MS if mask in (0, 3, 8) else 0.0, call=call)
             ghz, clk = _clock_ghz(stats.cpu().numpy())
             abl[names[mask]] = {"launch_ms_mean": ms, "shader_clock_ghz": ghz, "kclocks": clk / 1e3}
+        # the same two builds on all-zero operands, where nothing is power-limited: there the idle clocks cost their time
+        zops = (torch.zeros_like(kinputs[0][0]), torch.zeros_like(kinputs[0][1]), torch.full_like(kinputs[0][2], 127), torch.full_like(kinputs[0][3], 127))
+        for mask in (8, 0):
+            assert P.mxfp6_probe_tiled_ablation(mask) == 0
+            _, ms = timed_loop(hk, torch, [zops], C, 20, 10, prewarm_ms=PREWARM_MS, call=call)
+            ghz, clk = _clock_ghz(stats.cpu().numpy())
+            abl[names[mask] + "_zero_operands"] = {"launch_ms_mean": ms, "shader_clock_ghz": ghz, "kclocks": clk / 1e3}
+        del zops
         out["tiled_kernel_ablations"] = abl
         # the builds with MFMAs run at a power-managed clock: what adding a part costs there, in time
         t = {k: v["launch_ms_mean"] * 1e3 for k, v in abl.items()}

@@ -590,7 +590,7 @@ int mxfp6_kernel_choice(int M, int N, int K, int layouts) {
 
 #ifdef MXFP6_PROBES  // ---- measurement entry points (include/mxfp6_probes.h)
 int mxfp6_probe_tiled_ablation(int mask) {
-  if (mask < 0 || mask > 6 || mask == 5) return MXFP6_EINVAL_SHAPE;
+  if (mask < 0 || (mask > 6 && mask != 8) || mask == 5) return MXFP6_EINVAL_SHAPE;
   g_ablation = mask;
   return MXFP6_OK;
 }

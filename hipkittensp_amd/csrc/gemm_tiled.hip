@@ -129,7 +129,7 @@ struct TiledArgs {
 // unfused 8192^3 GEMM).
 // ABL (measurement build only, -DMXFP6_PROBES; results are then meaningless): bit 0 leaves out the LDS reads of the operands after the first
 // K-tile of an output tile, bit 1 the direct loads after the prologue, bit 2 the MFMAs after the first K-tile of an output
-// tile.  What the remaining parts of the kernel take, in time and in shader clocks, is how bench.py splits the kernel's
+// tile; bit 3 leaves everything in and adds idle clocks (a wave sleeps 128 clocks after every fourth MFMA).  What the remaining parts of the kernel take, in time and in shader clocks, is how bench.py splits the kernel's
 // time between the matrix cores, the LDS reads and the loads.
 // KSPLIT: the K range of an output tile is split between args.nsplit workgroups (few output tiles, long K: M of a few
 // hundred rows).  Share s of a tile multiplies K-tiles [s, s + 1) * nkt / nsplit and stores its fp32 sums into matrix s of
@@ -442,6 +442,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_tiled_kernel(const TiledArgs arg
         __builtin_amdgcn_sched_barrier(0);
         issue_one.template operator()<STEADY, GRP>(kt + AHEAD, slotx, i / 2);
         __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr ((ABL & 8) != 0) {  // the full kernel with idle clocks added: the wave sleeps 128 clocks after every fourth MFMA
+        if ((i & 3) == 3) {
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_sleep(2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     });
     __builtin_amdgcn_s_setprio(0);
@@ -837,7 +844,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
     else if (bm == 128) gemm_tiled_kernel<FA, FB, Out, 2, 2, true><<<grid, NW * 64, 0, s>>>(ta);
     else gemm_tiled_kernel<FA, FB, Out, 4, 2, true><<<grid, NW * 64, 0, s>>>(ta);
 #ifdef MXFP6_PROBES
-  } else if (g.ablation > 0 && g.ablation < 8) {
+  } else if (g.ablation > 0 && g.ablation <= 8) {
     // measurement instantiations: e2m3 x e2m3, bf16 output, 256 x 256 tiles only
     if constexpr (FA == 2 && FB == 2 && sizeof(typename Out::type) == 2) {
       if (bm != 256 || bn != 256) return hipErrorInvalidValue;
@@ -847,6 +854,7 @@ static hipError_t launch(const GemmArgs& g, hipStream_t s) {
         case 3: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 3><<<grid, NW * 64, 0, s>>>(ta); break;
         case 4: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 4><<<grid, NW * 64, 0, s>>>(ta); break;
         case 6: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 6><<<grid, NW * 64, 0, s>>>(ta); break;
+        case 8: gemm_tiled_kernel<2, 2, Out, 4, 2, false, 8><<<grid, NW * 64, 0, s>>>(ta); break;
         default: return hipErrorInvalidValue;  // 5 and 7 (no LDS reads and no MFMAs at once) are not built: the register allocator spills in them, which is all they would measure
       }
     } else {

@@ -52,7 +52,10 @@ int mxfp6_tile_order(int tiles_m, int tiles_n, int group_m, int xcd_remap, int *
  * direct loads after the prologue (bit 1), without its MFMAs (bit 2); other calls fail with hipErrorInvalidValue.  The
  * output of such a launch is meaningless.  Timing the combinations 1 - 4 and 6 next to the full kernel (with
  * mxfp6_probe_tiled_clock for the shader clock) shows what each part costs and which ones the power management charges
- * (5 and 7, no LDS reads and no MFMAs at once, are not built and rejected: those builds spill registers).
+ * (5 and 7, no LDS reads and no MFMAs at once, are not built and rejected: those builds spill registers).  mask = 8 is the
+ * whole kernel with idle clocks added (every wave sleeps 128 clocks after every fourth MFMA; the output stays correct): if
+ * the launch takes as long as without them while the shader clock rises, time is set by the power budget and not by the
+ * schedule's clocks.
  */
 int mxfp6_probe_tiled_ablation(int mask);
 int mxfp6_probe_raster(int group_m, int xcd_remap);

@@ -125,7 +125,7 @@ def test_abi_argument_validation_without_a_gpu(built_lib):
     assert L.mxfp6_set_kernel(99) == -9 and L.mxfp6_set_kernel(-1) == -9
     # measurement switches validate their argument too (they only set per-thread state: no GPU needed)
     P = ctypes.CDLL(PROBES_LIB)
-    assert P.mxfp6_probe_tiled_ablation(5) == -2 and P.mxfp6_probe_tiled_ablation(7) == -2 and P.mxfp6_probe_tiled_ablation(0) == 0
+    assert P.mxfp6_probe_tiled_ablation(5) == -2 and P.mxfp6_probe_tiled_ablation(7) == -2 and P.mxfp6_probe_tiled_ablation(9) == -2 and P.mxfp6_probe_tiled_ablation(0) == 0
     assert L.mxfp6_set_k_split(65) == -2 and L.mxfp6_set_k_split(-2) == -2
     prev = L.mxfp6_set_k_split(1)
     assert prev == 0 and L.mxfp6_set_k_split(0) == 1

@@ -1306,6 +1306,18 @@ def test_measurement_probes_run_and_leave_results_alone(hk):
         L.mxfp6_probe_tiled_clock(None)
         L.mxfp6_probe_raster(0, 1)
     assert np.array_equal(got, ref)
+    # the build with idle clocks added (ablation 8: bf16 output, 256 x 256 tiles) multiplies like the kernel itself
+    C8 = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert L.mxfp6_probe_tiled_ablation(8) == 0
+    pk = L.mxfp6_set_kernel(6)
+    try:
+        rc = L.mxfp6_gemm_ex(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), C8.data_ptr(), M, N, K, 2, 2, 0, 0, 0, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+    finally:
+        L.mxfp6_set_kernel(pk)
+        L.mxfp6_probe_tiled_ablation(0)
+    assert rc == 0, rc
+    assert np.array_equal(C8.view(torch.int16).cpu().numpy().view(np.uint16), o.f32_to_bf16_bits(ref))
 
 
 @pytest.mark.parametrize("M,N,K,kernel,shares", [(256, 1024, 8192, 2, 8), (300, 520, 8192, 2, 4), (128, 1024, 8192, 22, 8), (200, 1032, 4096 + 128, 22, 3), (128, 384, 8192, 22, 8)])
