@@ -429,18 +429,67 @@ def square_sizes(hk, torch, steps, warmup):
     return out
 
 
+def weight_sets(hk, torch, N, K, gen):
+    """A weight matrix [N, K] in as many rotated copies as make 400 MB (2 to 16), row-major and tile-major, each kind in one
+    contiguous buffer: the timing probe takes launch i's weights from copy i % sets, so that B comes from HBM as the weights
+    of a model's layers do, not from the 256 MB last-level cache."""
+    b, sc = hk.quantize(torch.randn(N, K, device="cuda", generator=gen) * 0.02, 2)
+    sets = min(16, max(2, -(-400_000_000 // (N * K * 3 // 4))))
+    bp = torch.stack([torch.roll(b, 32 * i, 0) for i in range(sets)])
+    bs = torch.stack([torch.roll(sc, 32 * i, 0) for i in range(sets)])
+    del b, sc
+    bt = torch.stack([hk.tile_operand(bp[i]) for i in range(sets)])
+    bst = torch.stack([hk.tile_scales(bs[i], K) for i in range(sets)])
+    return sets, (bp, bs), (bt, bst)
+
+
+def probe_time_us(P, torch, a, asc, weights, sets, C, M, N, K, la, lb, kernel, k_split):
+    """Microseconds per launch of one GEMM with a kernel forced (0: the automatic choice) and a K-split setting, timed by the
+    measurement build between two events around back-to-back launches (mxfp6_probe_time_gemm: no interpreter between the
+    launches, so a shape of a few microseconds is timed as a replayed graph would run it); None: the forced kernel does not
+    take the shape.  A first short run sizes the timed one to about 0.6 ms."""
+    import ctypes
+
+    B, Bs = weights
+    stream = torch.cuda.current_stream().cuda_stream
+    us = ctypes.c_double()
+    prev_k, prev_s = P.mxfp6_set_kernel(kernel), P.mxfp6_set_k_split(k_split)
+    try:
+        def run(warmup, reps):
+            return P.mxfp6_probe_time_gemm(a.data_ptr(), B.data_ptr(), asc.data_ptr(), Bs.data_ptr(), C.data_ptr(), M, N, K, 2, 2, la, lb, 0, sets,
+                                           B.stride(0) * B.element_size(), Bs.stride(0) * Bs.element_size(), warmup, reps, ctypes.byref(us), stream)
+        if run(2, 4) != 0:
+            return None
+        if run(2, max(8, min(64, int(600.0 / max(us.value, 1.0))))) != 0:
+            return None
+    finally:
+        P.mxfp6_set_kernel(prev_k)
+        P.mxfp6_set_k_split(prev_s)
+    return us.value
+
+
+CANDIDATES = (("tiled_256x256", 6, 1), ("tiled_128x256", 5, 1), ("tiled_128x128", 17, 1), ("block", 22, 1), ("block_128x256", 26, 1), ("skinny", 3, 0),
+              ("tiled_k_split_256", 6, -1), ("tiled_k_split_128", 5, -1), ("block_k_split", 22, -1), ("ring", 28, 0))  # in the order of the library's candidate numbers
+
+
 def dispatch_sweep(hk, torch, grid):
     """How good is the automatic kernel choice?  For every shape of a grid (rows of A x a set of (N, K) pairs x both
     layouts of B; A row-major) the call is timed with the automatic choice (twice, before and after the others: the better
-    of the two) and with every kernel / tile shape forced in turn, the tiled, the block and the ring kernel also with their K
-    split wherever the shape allows one.  Reports, per shape, the automatic time,
-    the best forced time and which kernel that was, and the shapes where the automatic choice is more than 8 % behind.
-    Small shapes (below about 15 us) are bound by the host side of the Python operator and only scatter."""
-    tk = hk.tk_kernel
+    of the two) and with every kernel / tile shape forced in turn, the tiled and the block kernel also with their K split
+    wherever the shape allows one.  Reports, per shape, the automatic time, the best forced time and which kernel that was,
+    and the shapes where the automatic choice is more than 8 % behind.  Timed on the GPU's side (probe_time_us), weights
+    rotating through 400 MB."""
+    from hipkittensp_amd import _lib
+
+    tk, P = hk.tk_kernel, _lib.probes()
     if grid == "offgrid":  # none of these (N, K) pairs and none of these row counts is in the calibration table
         shapes = [(7168, 7168), (3584, 18944), (18944, 3584), (9216, 4608), (27648, 5120), (1792, 14336), (22016, 4096), (5632, 22528),
                   (13312, 6656), (36864, 3072), (2304, 24576), (15360, 10240)]
         rows_of_a = [20, 56, 72, 144, 208, 288, 416, 576, 832, 1152, 1792, 2560]
+    elif grid == "offgrid2":  # a second held-out set, never used to tune anything
+        shapes = [(5120, 5120), (9216, 9216), (14336, 7168), (3328, 16640), (25600, 5632), (2816, 11264), (45056, 3584), (6656, 13312),
+                  (19456, 6144), (1280, 28160), (10752, 10752), (30720, 2560)]
+        rows_of_a = [28, 36, 88, 104, 176, 240, 352, 480, 704, 960, 1280, 2304]
     elif grid == "full":
         shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096),
                   (8192, 28672), (2048, 8192), (5120, 16384), (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096)]
@@ -448,77 +497,53 @@ def dispatch_sweep(hk, torch, grid):
     else:
         shapes = [(8192, 8192), (28672, 8192), (8192, 28672), (57344, 8192), (1024, 16384)]
         rows_of_a = [16, 32, 64, 128, 256, 512, 1024]
-    forced = (("tiled", 2, 1), ("tiled_128x256", 5, 1), ("tiled_256x256", 6, 1), ("tiled_128x128", 17, 1), ("block", 22, 1), ("block_128x256", 26, 1), ("skinny", 3, 0), ("mid", 4, 0),
-              ("tiled_k_split_256", 6, -1), ("tiled_k_split_128", 5, -1), ("block_k_split", 22, -1), ("ring", tk.KERNEL_RING, 0))
-
-    def time_us(sets, C, lay, kernel, k_split, reps=10):
-        prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
-        try:
-            for i in range(3):
-                hk.dispatch_micro(*sets[i % len(sets)], C, layout_b=lay)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for i in range(reps):
-                hk.dispatch_micro(*sets[i % len(sets)], C, layout_b=lay)
-            e1.record()
-            torch.cuda.synchronize()
-        except RuntimeError:
-            return None  # the forced kernel does not take this shape
-        finally:
-            tk.set_kernel(prev_k)
-            tk.set_k_split(prev_s)
-        return e0.elapsed_time(e1) / reps * 1e3
+    forced = (("tiled", 2, 1), ("mid", 4, 0)) + CANDIDATES
 
     per_shape, behind = [], []
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
     for N, K in shapes:
-        g = torch.Generator(device="cuda")
-        g.manual_seed(1)
-        bs = [hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2) for _ in range(2)]
-        bts = [(hk.tile_operand(b), hk.tile_scales(sc, K)) for b, sc in bs]
+        sets, row, tile = weight_sets(hk, torch, N, K, g)
         for M in rows_of_a:
             a, asc = hk.quantize(torch.randn(M, K, device="cuda", generator=g), 2)
             C = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
             for lay in (1, 0):
-                sets = [(a, (bts if lay else bs)[i][0], asc, (bts if lay else bs)[i][1]) for i in range(2)]
-                auto = time_us(sets, C, lay, 0, 0)
+                def t(kernel, k_split):
+                    return probe_time_us(P, torch, a, asc, tile if lay else row, sets, C, M, N, K, 0, lay, kernel, k_split)
+                auto = t(0, 0)
                 times = {}
                 for name, kernel, k_split in forced:
                     if (name == "skinny" and M > 128) or (name == "mid" and (M <= 32 or M > 512)) or (name == "ring" and M > 256):
                         continue
-                    t = time_us(sets, C, lay, kernel, k_split)
-                    if t is not None:
-                        times[name] = t
-                auto = min(auto, time_us(sets, C, lay, 0, 0))  # again after the others: the first timing on new operands runs 5 - 10 % slow
+                    us = t(kernel, k_split)
+                    if us is not None:
+                        times[name] = us
+                auto = min(auto, t(0, 0))
                 best = min(times, key=times.get)
-                rec = {"M": M, "N": N, "K": K, "layout_b": "tile" if lay else "row", "auto_us": round(auto, 1), "best_us": round(times[best], 1),
-                       "best": best, "auto_over_best": round(auto / times[best], 3), "times_us": {k: round(v, 1) for k, v in times.items()},
+                rec = {"M": M, "N": N, "K": K, "layout_b": "tile" if lay else "row", "auto_us": round(auto, 2), "best_us": round(times[best], 2),
+                       "best": best, "auto_over_best": round(auto / times[best], 3), "times_us": {k: round(v, 2) for k, v in times.items()},
                        "choice": tk.kernel_choice(M, N, K, 0, lay)}
                 per_shape.append(rec)
                 if rec["auto_over_best"] > 1.08:
                     behind.append(rec)
+        del row, tile
+        torch.cuda.empty_cache()
     ratios = sorted(r["auto_over_best"] for r in per_shape)
-    return {"what": "automatic kernel choice against every forced kernel, tile shape and K split; e2m3 x e2m3, bf16 out, A row-major", "shapes": len(per_shape),
-            "within_8_percent": sum(1 for r in ratios if r <= 1.08), "median_auto_over_best": ratios[len(ratios) // 2], "worst_auto_over_best": ratios[-1],
+    return {"what": "automatic kernel choice against every forced kernel, tile shape and K split; e2m3 x e2m3, bf16 out, A row-major; timed on the GPU's side, weights rotating through 400 MB",
+            "shapes": len(per_shape), "within_8_percent": sum(1 for r in ratios if r <= 1.08), "median_auto_over_best": ratios[len(ratios) // 2], "worst_auto_over_best": ratios[-1],
             "behind_by_more_than_8_percent": behind, "per_shape": per_shape}
-
-
-CANDIDATES = (("tiled_256x256", 6, 1), ("tiled_128x256", 5, 1), ("tiled_128x128", 17, 1), ("block", 22, 1), ("block_128x256", 26, 1), ("skinny", 3, 0),
-              ("tiled_k_split_256", 6, -1), ("tiled_k_split_128", 5, -1), ("block_k_split", 22, -1), ("ring", 28, 0))  # in the order of the library's candidate numbers
 
 
 def calibration_sweep(hk, torch):
     """The sweep behind the kernel choice's calibration table (hipkittensp_amd/csrc/dispatch_table.inc): every candidate of the
-    choice, forced, on a grid of shapes x three layout pairs, each timed twice (the better counts), next to the time model's
-    figure for it (mxfp6_probe_candidate of the measurement build).  `python -m hipkittensp_amd.calibrate` turns the JSON this
-    prints into the table: per shape and candidate, measured / modelled time."""
+    choice, forced, on a grid of shapes x three layout pairs, timed on the GPU's side with weights rotating through 400 MB
+    (probe_time_us), twice (the better counts).  `python -m hipkittensp_amd.calibrate` turns the JSON this prints into the
+    table: per shape and candidate, measured time / the time model's figure."""
     import ctypes
 
     from hipkittensp_amd import _lib
 
     tk, P = hk.tk_kernel, _lib.probes()
-    P.mxfp6_probe_candidate.restype = ctypes.c_int
-    P.mxfp6_probe_candidate.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
     shapes = [(8192, 8192), (4096, 14336), (28672, 8192), (28672, 4096), (24576, 8192), (40960, 8192), (57344, 8192), (128256, 4096), (8192, 28672), (2048, 8192), (5120, 16384),
               (10240, 8192), (1024, 16384), (14336, 4096), (32000, 4096), (4096, 4096), (16384, 16384), (2048, 28672), (11008, 4096), (4096, 11008), (2048, 2048), (512, 8192), (8192, 1024),
               (1024, 32768), (2048, 16384), (4096, 8192), (4096, 24576), (8192, 4096), (8192, 14336), (16384, 4096), (16384, 8192), (65536, 2048), (3072, 3072), (6144, 4096), (1024, 4096),
@@ -526,31 +551,11 @@ def calibration_sweep(hk, torch):
               (6144, 6144), (12288, 6144), (3072, 12288), (20480, 5120), (18432, 9216), (7168, 20480), (49152, 4096), (2560, 10240), (13824, 5120), (5120, 13824), (100352, 2048), (1536, 32768)]
     rows_of_a = [1, 8, 12, 16, 24, 32, 40, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1536, 2048, 3072, 4096, 8192]
 
-    def time_us(ops, C, la, lb, kernel, k_split, reps=8):
-        prev_k, prev_s = tk.set_kernel(kernel), tk.set_k_split(k_split)
-        try:
-            for i in range(2):
-                hk.dispatch_micro(*ops[i % len(ops)], C, layout_a=la, layout_b=lb)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for i in range(reps):
-                hk.dispatch_micro(*ops[i % len(ops)], C, layout_a=la, layout_b=lb)
-            e1.record()
-            torch.cuda.synchronize()
-        except RuntimeError:
-            return None
-        finally:
-            tk.set_kernel(prev_k)
-            tk.set_k_split(prev_s)
-        return e0.elapsed_time(e1) / reps * 1e3
-
     points = []
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
     for N, K in shapes:
-        bs = [hk.quantize(torch.randn(N, K, device="cuda", generator=g) * 0.02, 2) for _ in range(2)]
-        bts = [(hk.tile_operand(b), hk.tile_scales(sc, K)) for b, sc in bs]
+        sets, row, tile = weight_sets(hk, torch, N, K, g)
         for M in rows_of_a:
             if M * N > 1 << 28:
                 continue
@@ -560,31 +565,31 @@ def calibration_sweep(hk, torch):
                 if la and (M % 32 or K % 128):
                     continue
                 at, ast = (hk.tile_operand(a), hk.tile_scales(asc, K)) if la else (a, asc)
-                ops = [(at, (bts if lb else bs)[i][0], ast, (bts if lb else bs)[i][1]) for i in range(2)]
                 layouts = la | lb << 1
-                measured, model = [], []
+
+                def t(kernel, k_split):
+                    return probe_time_us(P, torch, at, ast, tile if lb else row, sets, C, M, N, K, la, lb, kernel, k_split)
+                measured = []
                 for cand, (name, kernel, k_split) in enumerate(CANDIDATES):
                     m, c, sh = ctypes.c_double(), ctypes.c_double(), ctypes.c_int()
                     prev = P.mxfp6_set_k_split(k_split)
                     rc = P.mxfp6_probe_candidate(M, N, K, layouts, cand, 0, ctypes.byref(m), ctypes.byref(c), ctypes.byref(sh))
                     P.mxfp6_set_k_split(prev)
                     assert rc == 0, rc
-                    t = None
-                    if m.value >= 0:
-                        t = time_us(ops, C, la, lb, kernel, k_split)
-                        t2 = time_us(ops, C, la, lb, kernel, k_split) if t is not None else None
-                        t = min(t, t2) if t2 is not None else t
-                    measured.append(round(t, 2) if t is not None else None)
-                    model.append(round(m.value, 2) if m.value >= 0 else None)
-                auto = time_us(ops, C, la, lb, 0, 0)
-                point = {"M": M, "N": N, "K": K, "layouts": layouts, "measured_us": measured, "model_us": model, "auto_us": round(auto, 2), "choice": tk.kernel_choice(M, N, K, la, lb)}
+                    us = None
+                    if m.value >= 0:  # the candidate takes the shape (a split: the shape has one)
+                        us = t(kernel, k_split)
+                        us2 = t(kernel, k_split) if us is not None else None
+                        us = min(us, us2) if us2 is not None else us
+                    measured.append(round(us, 2) if us is not None else None)
+                point = {"M": M, "N": N, "K": K, "layouts": layouts, "measured_us": measured, "auto_us": round(t(0, 0), 2), "choice": tk.kernel_choice(M, N, K, la, lb)}
                 if measured[-1] is not None:  # the ring kernel as one share of K: not a candidate of its own, a point for the model's per-workgroup rate
-                    one = time_us(ops, C, la, lb, CANDIDATES[-1][1], 1)
+                    one = t(CANDIDATES[-1][1], 1)
                     point["ring_one_share_us"] = round(one, 2) if one is not None else None
                 points.append(point)
-        del bs, bts
+        del row, tile
         torch.cuda.empty_cache()
-    return {"what": "calibration sweep of the kernel choice: measured and modelled microseconds per candidate", "candidates": [c[0] for c in CANDIDATES],
+    return {"what": "calibration sweep of the kernel choice: measured microseconds per candidate (GPU-side timing, weights rotating through 400 MB)", "candidates": [c[0] for c in CANDIDATES],
             "device": torch.cuda.get_device_name(0), "cus": torch.cuda.get_device_properties(0).multi_processor_count, "points": points}
 
 
@@ -660,7 +665,7 @@ def main():
     p.add_argument("--sweep-settings", choices=["all", "default", "ksplit-order"], default="all",
                    help="with --raster-sweep: all raster settings, only the kernel's own (to compare schedules under a profiler), or the kernel's own and, as "
                         "xcd_remap=2, a K split's workgroups in tile-by-tile order instead of share by share (for shapes that take a K split)")
-    p.add_argument("--dispatch-sweep", choices=["small", "full", "offgrid", "calibrate"], default=None,
+    p.add_argument("--dispatch-sweep", choices=["small", "full", "offgrid", "offgrid2", "calibrate"], default=None,
                    help="only compare the automatic kernel choice with every forced kernel / tile shape / K split over a grid of shapes and print one JSON line")
     p.add_argument("--layouts", choices=["both", "row"], default="both", help="row: skip the decode run with tile-major weights (used for profiling one layout of the skinny kernel)")
     p.add_argument("--profile-kernels", action="store_true", help="only loops of the tiled kernel (8192^3, tile-major), the skinny kernel (configs[3], row-major) and the ring "

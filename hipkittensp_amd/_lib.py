@@ -115,6 +115,10 @@ def probes() -> ctypes.CDLL:
         L.mxfp6_probe_ksplit_plan.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci)]
         L.mxfp6_probe_block.restype = ci
         L.mxfp6_probe_block.argtypes = [ci]
+        L.mxfp6_probe_candidate.restype = ci
+        L.mxfp6_probe_candidate.argtypes = [ci] * 6 + [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ci)]
+        L.mxfp6_probe_time_gemm.restype = ci
+        L.mxfp6_probe_time_gemm.argtypes = [vp] * 5 + [ci] * 9 + [ctypes.c_size_t, ctypes.c_size_t, ci, ci, ctypes.POINTER(ctypes.c_double), vp]
         _probes = L
     return _probes
 

@@ -612,6 +612,32 @@ int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int* t
   return n;
 }
 
+int mxfp6_probe_time_gemm(const void* A, const void* B, const void* As, const void* Bs, void* C, int M, int N, int K, int fmt_a, int fmt_b,
+                          int layout_a, int layout_b, int out_f32, int b_sets, size_t b_stride, size_t bs_stride, int warmup, int reps, double* us,
+                          void* stream) {
+  if (!us || b_sets < 1 || warmup < 0 || reps < 1) return MXFP6_EINVAL_PTR;
+  hipStream_t s = (hipStream_t)stream;
+  auto launch = [&](int i) {
+    const size_t set = (size_t)(i % b_sets);
+    return gemm_common(A, (const uint8_t*)B + set * b_stride, As, (const uint8_t*)Bs + set * bs_stride, C, M, N, K, fmt_a, fmt_b, out_f32 != 0, layout_a, layout_b, stream);
+  };
+  for (int i = 0; i < warmup; i++) {
+    const int rc = launch(i);
+    if (rc) return rc;
+  }
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return (int)hipErrorOutOfMemory;
+  int rc = (int)hipEventRecord(e0, s);
+  for (int i = 0; i < reps && !rc; i++) rc = launch(warmup + i);
+  if (!rc) rc = (int)hipEventRecord(e1, s);
+  if (!rc) rc = (int)hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (!rc) rc = (int)hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0), (void)hipEventDestroy(e1);
+  *us = ms * 1e3 / reps;
+  return rc;
+}
+
 int mxfp6_probe_candidate(int M, int N, int K, int layouts, int candidate, int cus, double* model_us, double* calibrated_us, int* shares) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 32 || candidate < 0 || candidate >= mxfp6::kNumCandidates || cus < 0) return MXFP6_EINVAL_SHAPE;
   if (layouts < 0 || layouts > 3) return MXFP6_EINVAL_LAYOUT;

@@ -8,6 +8,8 @@
 #ifndef MXFP6_PROBES_H
 #define MXFP6_PROBES_H
 
+#include <stddef.h>
+
 #include "mxfp6_gemm.h"
 
 #ifdef __cplusplus
@@ -66,12 +68,22 @@ int mxfp6_probe_raster(int group_m, int xcd_remap);
  * on them). */
 int mxfp6_probe_ksplit_plan(int M, int N, int K, int layouts, int shares, int *tile_rows);
 
+/* Times a GEMM as the library would run it under this thread's mxfp6_set_kernel / mxfp6_set_k_split settings: `warmup`
+ * untimed and `reps` timed back-to-back launches between two events on `hip_stream`, mean microseconds per launch in *us.
+ * Launch i takes its B operand and B scales from B + (i % b_sets) * b_stride and Bs + (i % b_sets) * bs_stride (bytes), so that
+ * a caller can rotate through more weights than the last-level cache holds, as a model's layers do.  Synchronises the
+ * stream.  bf16 output unless out_f32.  The calibration sweep of the kernel choice and its checks time with this (no
+ * interpreter between the launches: shapes of a few microseconds are timed on the GPU's side, as a replayed graph runs them). */
+int mxfp6_probe_time_gemm(const void *A, const void *B, const void *A_scale, const void *B_scale, void *C, int M, int N, int K,
+                          int fmt_a, int fmt_b, int layout_a, int layout_b, int out_f32, int b_sets, size_t b_stride,
+                          size_t bs_stride, int warmup, int reps, double *us, void *hip_stream);
+
 /* The kernel choice's view of one candidate on a shape (e2m3 x e2m3, bf16 output, 16-byte aligned tensors): *model_us is the
  * structural time model's figure in microseconds (negative: the candidate does not take the shape), *calibrated_us that figure
  * times the calibration factor of the nearest calibrated shape (what the choice compares), *shares the K split the candidate
  * would run with under the thread's mxfp6_set_k_split setting.  candidate: 0 - 2 the tiled kernel with tiles of 256 x 256 /
- * 128 x 256 / 128 x 128, 3 block, 4 block with tiles of 128 x 256, 5 skinny, 6 / 7 the tiled / the block kernel with its K
- * split, 8 ring.  cus: compute units to plan for (0 = the current device's).  Pure host code: the calibration tool
+ * 128 x 256 / 128 x 128, 3 block, 4 block with tiles of 128 x 256, 5 skinny, 6 / 7 the tiled kernel's K split with tiles of
+ * 256 / 128 rows, 8 the block kernel's K split, 9 ring.  cus: compute units to plan for (0 = the current device's).  Pure host code: the calibration tool
  * (python -m hipkittensp_amd.calibrate) calls it to turn a sweep's measured times into the table's factors. */
 int mxfp6_probe_candidate(int M, int N, int K, int layouts, int candidate, int cus, double *model_us, double *calibrated_us,
                           int *shares);
