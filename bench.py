@@ -294,7 +294,7 @@ def stream_probe(torch, P):
 
 
 def cpu_legs(cfg, ops, rows, k_slice, gpu_f32):
-    """The CPU baseline on this run's own bytes, in the two forms the survey names: the OpenMP C port of
+    """The CPU baseline on this run's own bytes, in two forms: the OpenMP C port of
     dequantise-and-matmul (oracle/mxfp6_oracle.c) and dequantise (the C oracle's) + torch.matmul in fp32, each part timed.
     rows: the first `rows` rows of A; k_slice: the first K / k_slice columns of K (1 = all of K).  gpu_f32: the library's
     fp32 result for the same rows over the same K range, compared with the C port's with the parity metric."""
