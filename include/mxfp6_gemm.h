@@ -27,9 +27,10 @@
  *   - mxfp6_gemm_fused_fp6 on shapes the LDS-tiled kernel does not run: 4 M N bytes;
  *   - the gemm entry points on decode shapes whose K range is split between workgroups (M <= 32, N <= 2048,
  *     K >= 24576): 2 MB;
- *   - the gemm entry points on problems of few output tiles and long K (up to a few hundred rows of A, K >= 5120; see
- *     mxfp6_set_k_split), where the LDS-tiled kernel or the block kernel splits K between workgroups: shares * 4 M N
- *     bytes, at most 64 MB (one workspace for both kernels).
+ *   - the gemm entry points on problems of few output tiles and long K (up to a few hundred rows of A; see
+ *     mxfp6_set_k_split), where the LDS-tiled kernel, the block kernel or the ring kernel splits K between workgroups:
+ *     shares * 4 M N bytes of partial sums (tiles times shares never exceed the CUs: at most 64 MB, 256 tiles of
+ *     256 x 256 fp32), one workspace for the three kernels, and for the ring kernel one counter per output tile.
  * While `hip_stream` is being captured nothing is allocated: the pre-pass and the K splits are left out
  * (same results up to the order of fp32 sums, other kernels) unless their workspace exists already, and mxfp6_gemm_fused_fp6 returns
  * hipErrorStreamCaptureUnsupported where it would need a new one.  A workspace that a capture did use is recorded in the
@@ -132,11 +133,11 @@ int mxfp6_gemm_f32out(const void *A_packed, const void *B_packed, const void *A_
  *       private LDS slots, A comes through a ring that a loader wave fills and flags guard, no barrier per K-tile;
  *       splits K between workgroups by the thread's mxfp6_set_k_split setting
  *   22  block kernel: output tiles of 128 x 128, four waves in step with the operand fragments double-buffered in
- *       registers, one barrier per K-tile (needs N % 8 == 0, K % 128 == 0); chosen automatically where
- *       its tiles do not outnumber the CUs and K is of moderate length (a few hundred rows of A);
+ *       registers, one barrier per K-tile (needs N % 8 == 0, K % 128 == 0); typically chosen for a few hundred to a few
+ *       thousand rows of A;
  *       23 / 24: with an operand ring of three slots (two workgroups per CU) / six slots (one); 26: with tiles of
  *       128 x 256 and eight waves.  22 - 24 split K between workgroups by the thread's mxfp6_set_k_split setting
- *       (0: where the library's rule for this kernel says so; the same per-stream workspace as the tiled kernel's split)
+ *       (0: where the library's time model prefers the split; the same per-stream workspace as the tiled kernel's split)
  * No counterpart in the reference, whose shapes are compile-time constants per binary
  * (analysis/bf16_gemm/mi350x/mi355x_benchmark.sh).
  */
