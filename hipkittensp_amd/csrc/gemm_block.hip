@@ -441,7 +441,7 @@ bool gemm_block_supports(const GemmArgs& g) {
 
 // g.ksplit > 1 (with g.ks_part): the K range of every output tile split between that many workgroups, then
 // ksplit_reduce_kernel (gemm_tiled.hip), which also applies a fused epilogue.  The caller has checked that the last share
-// is not empty (block_ksplit_plan).
+// is not empty (block_split_shares, dispatch.hip).
 hipError_t launch_gemm_block(const GemmArgs& g, hipStream_t s) {
   const int bn = g.tile_cols == 256 ? 256 : 128, nsplit = g.ksplit > 1 ? g.ksplit : 1;
   BlockArgs a{g.A, g.B, g.As, g.Bs, nsplit > 1 ? (void*)g.ks_part : g.C, g.M, g.N, g.K, (g.M + kBM - 1) / kBM, (g.N + bn - 1) / bn, g.layout_a, g.layout_b,

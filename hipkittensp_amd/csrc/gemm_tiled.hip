@@ -49,7 +49,7 @@
 // row-major / tile-major operands).
 //
 // This file is compiled five times (build.py): once as it is, which gives the host-side part (shape checks, tile
-// shape and grid, time estimates, the K split's plan and reduction, the dispatcher), and once per pair of operand
+// shape and grid, the K split's reduction, the launcher that picks the format pair), and once per pair of operand
 // formats with -DMXFP6_TILED_FMT=22 / 23 / 32 / 33, which gives that pair's kernel instantiations and launcher: the
 // instantiations are what takes the time to compile, and four objects compile side by side.
 #include "common.hpp"
